@@ -1,0 +1,263 @@
+"""The cache of all live sequences: keys and values per layer call, in blocks, and
+per-sequence state of fixed size.
+
+A slot stands for one sequence and has its own length. Layer calls whose key/
+value rows have the same shape and window form a group; a group has storage of
+its own (one pool of blocks, one block table) and its own rule for which blocks
+a sequence of a given length holds: all of them, or those a window still sees.
+Storage of one call: keys [blocks, kv_heads, BLOCK_TOKENS, head_dim], values
+[blocks, kv_heads, head_dim, BLOCK_TOKENS] (values transposed inside a block, so
+that the keys of one block are contiguous along head_dim and the values along
+tokens, which is how the attention kernels read them).
+
+The reference keeps one paged cache per sequence with rows of all KV heads,
+float32 (crates/xrt-runtime/src/kv_cache.rs:4-45); `truncate` follows its
+rollback (kv_cache.rs:159-168).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+from ..parts.base import CacheNeeds, KVSpec
+from .allocator import BLOCK_TOKENS, CacheError, CacheFull, Pool, blocks_for
+
+
+@dataclass
+class KVView:
+    """What an attention kernel needs of one layer call's keys and values."""
+    spec: KVSpec
+    k: torch.Tensor             # [blocks, kv_heads, BLOCK_TOKENS, head_dim]
+    v: torch.Tensor             # [blocks, kv_heads, head_dim, BLOCK_TOKENS]
+    block_table: torch.Tensor   # int32 [slots, max_blocks]: logical block -> physical block, -1 = none
+
+
+@dataclass
+class LayerCache:
+    kv: Optional[KVView]
+    state: Optional[torch.Tensor]   # [slots, *shape]
+    writable: bool
+
+
+class KVGroup:
+    """Storage and block accounting of the layer calls that share one KVSpec."""
+
+    def __init__(self, spec: KVSpec, calls: List[int], n_blocks: int, max_slots: int,
+                 max_blocks_per_sequence: int, dtype: torch.dtype, device):
+        self.spec = spec
+        self.calls = calls
+        self.pool = Pool(n_blocks, "block")
+        self.max_blocks_per_sequence = max_blocks_per_sequence
+        # host table: the truth; device table: what kernels read, refreshed before a step
+        self.table = torch.full((max_slots, max_blocks_per_sequence), -1, dtype=torch.int32)
+        self.device_table = self.table.to(device)
+        self.dirty = False
+        self._floor: Dict[int, int] = {}   # slot -> lowest logical block it may still hold
+        shape_k = (len(calls), n_blocks, spec.n_kv_heads, BLOCK_TOKENS, spec.head_dim)
+        shape_v = (len(calls), n_blocks, spec.n_kv_heads, spec.head_dim, BLOCK_TOKENS)
+        self.k = torch.zeros(shape_k, dtype=dtype, device=device)
+        self.v = torch.zeros(shape_v, dtype=dtype, device=device)
+
+    def first_needed_block(self, length: int) -> int:
+        """Lowest logical block that a query at position >= length can still see."""
+        if self.spec.window is None:
+            return 0
+        return max(0, length + 1 - self.spec.window) // BLOCK_TOKENS
+
+    def held(self, slot: int) -> List[int]:
+        row = self.table[slot]
+        return [int(b) for b in row[row >= 0]]
+
+    def grow(self, slot: int, new_length: int) -> List[int]:
+        """Acquire the blocks that tokens up to new_length need; returns the logical indices added."""
+        need = blocks_for(new_length)
+        if need > self.max_blocks_per_sequence:
+            raise CacheError(f"sequence of {new_length} tokens exceeds the cache's limit per sequence")
+        added = []
+        try:
+            for logical in range(need):
+                if self.table[slot, logical] < 0 and logical >= self._floor.get(slot, 0):
+                    self.table[slot, logical] = self.pool.acquire()
+                    added.append(logical)
+        except CacheFull:
+            self.drop(slot, added)
+            raise
+        if added:
+            self.dirty = True
+        return added
+
+    def drop(self, slot: int, logicals: List[int]) -> None:
+        for logical in logicals:
+            self.pool.release(int(self.table[slot, logical]))
+            self.table[slot, logical] = -1
+        if logicals:
+            self.dirty = True
+
+    def shrink_to(self, slot: int, length: int) -> None:
+        """Release what a sequence of `length` tokens no longer needs: blocks past its end,
+        and blocks that have slid out of the window."""
+        past_end = [l for l in range(blocks_for(length), self.max_blocks_per_sequence)
+                    if self.table[slot, l] >= 0]
+        floor = self.first_needed_block(length)
+        below = [l for l in range(0, min(floor, self.max_blocks_per_sequence)) if self.table[slot, l] >= 0]
+        self._floor[slot] = floor
+        self.drop(slot, past_end + below)
+
+    def release_all(self, slot: int) -> None:
+        self.drop(slot, [l for l in range(self.max_blocks_per_sequence) if self.table[slot, l] >= 0])
+        self._floor.pop(slot, None)
+
+    def sync(self) -> None:
+        if self.dirty:
+            self.device_table.copy_(self.table, non_blocking=False)
+            self.dirty = False
+
+
+class SequenceCache:
+    """Slots, their lengths, and the storage of every layer call.
+
+    needs:       for each schedule entry its CacheNeeds, or None if it reads another entry's
+    reads_from:  for each schedule entry the entry whose cache it reads (itself if it owns one)
+    max_tokens:  tokens that live sequences may hold together, each rounded up to BLOCK_TOKENS
+    max_slots:   sequences that may be live together
+    max_context: longest sequence
+    """
+
+    def __init__(self, needs: List[Optional[CacheNeeds]], reads_from: List[int], max_tokens: int,
+                 max_slots: int, max_context: int, dtype: torch.dtype, device):
+        if max_tokens <= 0 or max_slots <= 0 or max_context <= 0:
+            raise ValueError("max_tokens, max_slots and max_context must be positive")
+        self.n_blocks = blocks_for(max_tokens)
+        self.max_slots = max_slots
+        self.max_context = min(max_context, self.n_blocks * BLOCK_TOKENS)
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.slots = Pool(max_slots, "slot")
+        self.lengths = [0] * max_slots
+        self.reads_from = list(reads_from)
+        self.needs = list(needs)
+
+        max_blocks = blocks_for(self.max_context)
+        self.groups: List[KVGroup] = []
+        self._group_of: Dict[int, KVGroup] = {}
+        by_spec: Dict[KVSpec, List[int]] = {}
+        for call, need in enumerate(needs):
+            if need is not None and need.kv is not None:
+                by_spec.setdefault(need.kv, []).append(call)
+        for spec, calls in by_spec.items():
+            group = KVGroup(spec, calls, self.n_blocks, max_slots, max_blocks, dtype, device)
+            self.groups.append(group)
+            for call in calls:
+                self._group_of[call] = group
+
+        self.states: Dict[int, torch.Tensor] = {}
+        for call, need in enumerate(needs):
+            if need is not None and need.state is not None:
+                self.states[call] = torch.zeros((max_slots, *need.state.shape),
+                                                dtype=need.state.dtype, device=device)
+
+    # -- slots ---------------------------------------------------------------
+    def alloc_slot(self) -> int:
+        slot = self.slots.acquire()
+        self.lengths[slot] = 0
+        for state in self.states.values():
+            state[slot].zero_()
+        return slot
+
+    def free_slot(self, slot: int) -> None:
+        if not self.slots.is_held(slot):
+            raise CacheError(f"slot {slot} is freed twice or was never allocated")
+        for group in self.groups:
+            group.release_all(slot)
+        self.lengths[slot] = 0
+        self.slots.release(slot)
+
+    def length(self, slot: int) -> int:
+        self._require(slot)
+        return self.lengths[slot]
+
+    def _require(self, slot: int) -> None:
+        if not self.slots.is_held(slot):
+            raise CacheError(f"slot {slot} is not allocated")
+
+    # -- growth by a step ----------------------------------------------------
+    def reserve(self, slot: int, new_length: int) -> None:
+        """Make room for the sequence to grow to new_length; its length is unchanged."""
+        self._require(slot)
+        if new_length > self.max_context:
+            raise CacheError(f"slot {slot}: {new_length} tokens exceed the context limit {self.max_context}")
+        grown = []
+        try:
+            for group in self.groups:
+                grown.append((group, group.grow(slot, new_length)))
+        except CacheFull:
+            for group, added in grown:
+                group.drop(slot, added)
+            raise
+
+    def commit(self, slot: int, new_length: int) -> None:
+        """The step has run: the sequence now has new_length tokens."""
+        self._require(slot)
+        self.lengths[slot] = new_length
+        for group in self.groups:
+            if group.spec.window is not None:
+                group.shrink_to(slot, new_length)
+
+    def cancel(self, slot: int) -> None:
+        """Give back what `reserve` took beyond the sequence's current length."""
+        self._require(slot)
+        for group in self.groups:
+            group.shrink_to(slot, self.lengths[slot])
+
+    def truncate(self, slot: int, length: int) -> None:
+        """Forget the tokens from position `length` on (reference: kv_cache.rs:159-168).
+
+        Only for layer calls that keep rows per token; state of fixed size cannot be rolled back."""
+        self._require(slot)
+        if length > self.lengths[slot]:
+            raise CacheError(f"slot {slot}: cannot truncate {self.lengths[slot]} tokens to {length}")
+        if self.states and length != self.lengths[slot]:
+            raise CacheError("a cache with per-sequence state cannot be truncated")
+        self.lengths[slot] = length
+        for group in self.groups:
+            group.shrink_to(slot, length)
+
+    def sync(self) -> None:
+        """Bring the device's block tables up to date; call before kernels read them."""
+        for group in self.groups:
+            group.sync()
+
+    # -- views ---------------------------------------------------------------
+    def layer_cache(self, call: int) -> LayerCache:
+        source = self.reads_from[call]
+        group = self._group_of.get(source)
+        kv = None
+        if group is not None:
+            index = group.calls.index(source)
+            kv = KVView(group.spec, group.k[index], group.v[index], group.device_table)
+        return LayerCache(kv=kv, state=self.states.get(source), writable=(source == call))
+
+    # -- accounting ----------------------------------------------------------
+    def held_blocks(self) -> int:
+        return max((group.pool.n_held for group in self.groups), default=0)
+
+    def check(self) -> None:
+        """Invariants: no slot or block lost or held twice; free slots hold nothing."""
+        self.slots.check()
+        for group in self.groups:
+            group.pool.check()
+            seen = set()
+            for slot in range(self.max_slots):
+                held = group.held(slot)
+                if not self.slots.is_held(slot) and held:
+                    raise CacheError(f"free slot {slot} still holds blocks {held}")
+                for block in held:
+                    if block in seen:
+                        raise CacheError(f"block {block} is held by two sequences")
+                    if not group.pool.is_held(block):
+                        raise CacheError(f"block {block} is in a table but free in the pool")
+                    seen.add(block)
+            if len(seen) != group.pool.n_held:
+                raise CacheError(f"{group.pool.n_held - len(seen)} blocks are held by no sequence")

@@ -1,0 +1,183 @@
+"""The engine: a model with its weights on the GPU, its cache, and one step function.
+
+`step` is the only way tokens reach the model. It takes a batch of sequences,
+each with the next tokens of that sequence (a whole prompt, or one token), runs
+exactly these tokens as one batch against what the cache holds, appends them to
+the cache and returns float32 logits at the wanted places. The reference has
+three entry points for one sequence each (crates/xrt-models/src/llama.rs:388-394
+forward_token, :617-622 forward_batch, :830-835 forward_batch_all_logits);
+positions are implied here by each sequence's length in the cache, where the
+reference checks the caller's position against it (llama.rs:434-439).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache import BLOCK_TOKENS, CacheError, CacheFull, SequenceCache
+from ..config import architecture, load_config
+from ..models import DecoderModel, ModelSpec
+from ..parts.base import Runtime
+from ..weights import check_names, load_tensors, random_tensors
+from .batch import StepBatch, build_batch
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+           "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32}
+
+
+def compute_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype must be bfloat16 or float32, found {name}")
+        return name
+    if name not in _DTYPES:
+        raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, found {name!r}")
+    return _DTYPES[name]
+
+
+class StepError(ValueError):
+    """A step that cannot run; nothing was computed and the cache is unchanged."""
+
+
+class Engine:
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype="bfloat16",
+                 max_tokens: int = 4096, max_slots: Optional[int] = None,
+                 max_context: Optional[int] = None, device="cuda:0", ops=None):
+        self.dtype = compute_dtype(dtype)
+        self.device = torch.device(device)
+        if ops is None:
+            from ..ops import load_ops
+            ops = load_ops()            # raises if the HIP library cannot be loaded: there is no other path
+        self.ops = ops
+        self.runtime = Runtime(ops, self.dtype, self.device)
+        self.config = spec.config
+        self.model = DecoderModel(spec, tensors, self.runtime)
+        model_context = getattr(spec.config, "max_position_embeddings", None)
+        limit = max_context if max_context is not None else model_context
+        if limit is None:
+            limit = max_tokens
+        if model_context is not None:
+            limit = min(limit, model_context)
+        if max_slots is None:
+            max_slots = max(1, min((max_tokens + BLOCK_TOKENS - 1) // BLOCK_TOKENS, 1024))
+        schedule = spec.schedule
+        reads_from = [i if call.reads_cache_of is None else call.reads_cache_of
+                      for i, call in enumerate(schedule)]
+        self.cache = SequenceCache(spec.cache_needs(), reads_from, max_tokens, max_slots, limit,
+                                   self.dtype, self.device)
+        self.vocab_size = spec.head.vocab
+
+    # -- construction ----------------------------------------------------------
+    @classmethod
+    def load(cls, folder: str, dtype="bfloat16", **options) -> "Engine":
+        """From a folder with config.json and model.safetensors (or shards with an index)."""
+        config = load_config(folder)
+        spec = architecture(config.architecture).build(config)
+        device = options.get("device", "cuda:0")
+        tensors = load_tensors(folder, spec.weight_specs(), spec.ignored_names(), device=device)
+        return cls(spec, tensors, dtype=dtype, **options)
+
+    @classmethod
+    def random(cls, config, seed: int = 0, dtype="bfloat16", std: float = 0.02, **options) -> "Engine":
+        """With random weights made on the device; no file is written."""
+        spec = architecture(config.architecture).build(config)
+        device = options.get("device", "cuda:0")
+        stored = torch.bfloat16 if compute_dtype(dtype) == torch.bfloat16 else torch.float32
+        engine = cls.__new__(cls)
+        tensors = LazyRandom(spec.weight_specs(), seed, std, stored, device)
+        cls.__init__(engine, spec, tensors, dtype=dtype, **options)
+        return engine
+
+    # -- slots -------------------------------------------------------------------
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    @property
+    def max_context(self) -> int:
+        return self.cache.max_context
+
+    # -- the step ----------------------------------------------------------------
+    def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> torch.Tensor:
+        """Run the next tokens of some sequences; return logits [wanted, vocab] (float32, on the device).
+
+        entries: (slot, tokens, want) per sequence; `want` are indices into `tokens`, in the order
+        in which their logits are returned (entries first, then want). The sequences of a step either
+        all start (length 0) or all continue; their token counts may differ.
+        """
+        batch = self.prepare(entries)
+        try:
+            logits = self.model.forward(batch, self.cache)
+        except Exception:
+            for slot in batch.host_slots:
+                self.cache.cancel(slot)
+            raise
+        for slot, start, count in zip(batch.host_slots, batch.host_starts, batch.host_counts):
+            self.cache.commit(slot, start + count)
+        return logits
+
+    def prepare(self, entries) -> StepBatch:
+        """Check a step, reserve its cache blocks, and pack it. Raises StepError before anything changes."""
+        if len(entries) == 0:
+            raise StepError("a step needs at least one sequence")
+        slots, tokens, wants, starts = [], [], [], []
+        seen = set()
+        for slot, ids, want in entries:
+            ids = list(ids)
+            want = list(want)
+            if slot in seen:
+                raise StepError(f"slot {slot} appears twice in one step")
+            seen.add(slot)
+            if not self.cache.slots.is_held(slot):
+                raise StepError(f"slot {slot} is not allocated")
+            if len(ids) == 0:                                   # llama.rs:624-626
+                raise StepError(f"slot {slot}: a step needs at least one token per sequence")
+            for token in ids:                                   # llama.rs:1044-1049
+                if not 0 <= int(token) < self.vocab_size:
+                    raise StepError(f"slot {slot}: token id {token} exceeds embedding rows {self.vocab_size}")
+            for index in want:
+                if not 0 <= int(index) < len(ids):
+                    raise StepError(f"slot {slot}: wanted index {index} is outside the {len(ids)} tokens given")
+            start = self.cache.length(slot)
+            if start + len(ids) > self.cache.max_context:
+                raise StepError(f"slot {slot}: {start} + {len(ids)} tokens exceed the context limit "
+                                f"{self.cache.max_context}")
+            slots.append(slot)
+            tokens.append(ids)
+            wants.append(want)
+            starts.append(start)
+        reserved = []
+        try:
+            for slot, ids, start in zip(slots, tokens, starts):
+                self.cache.reserve(slot, start + len(ids))
+                reserved.append(slot)
+        except (CacheFull, CacheError) as error:
+            for slot in reserved:
+                self.cache.cancel(slot)
+            raise StepError(f"the cache cannot hold this step: {error}") from None
+        self.cache.sync()
+        return build_batch(slots, tokens, starts, wants, self.device)
+
+
+class LazyRandom(dict):
+    """Random tensors by name, each made on the device when a part asks for it."""
+
+    def __init__(self, specs, seed, std, dtype, device):
+        super().__init__()
+        self._specs = specs
+        self._index = {name: i for i, name in enumerate(specs)}
+        self._args = (seed, std, dtype, device)
+
+    def __missing__(self, name):
+        from ..weights.random_init import _make
+        seed, std, dtype, device = self._args
+        return _make(self._specs[name], seed, self._index[name], std, dtype, device)
+
+    def __contains__(self, name):
+        return name in self._specs

@@ -1,0 +1,114 @@
+"""Causal attention with grouped key/value heads over the cache.
+
+The reference's attention (crates/xrt-models/src/llama.rs:447-577 decode,
+:695-784 prefill): q, k, v projections without bias; optional RMSNorm of every
+head of q and k with one weight [head_dim] each (:1025-1040), after the
+projection and before the position encoding; keys (encoded) and values (raw)
+appended to the cache; query head h reads key/value head h // group; a token at
+position P sees keys 0..P; softmax of q.k * scale in float32; output projection
+added to the residual stream.
+
+Q, K and V are bound as one matrix [(n_heads + 2 n_kv_heads) head_dim][hidden], so
+one product reads the normed activations once (the reference fuses the three
+dispatches, llama.rs:447-464).
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from .base import CacheNeeds, KVSpec, Mixer, PositionEncoding, Runtime, WeightSpec, register_part
+from .position import Rotary
+
+
+class Attention(Mixer):
+    def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                 position: Optional[PositionEncoding] = None, qk_norm: bool = False,
+                 qk_norm_eps: float = 0.0, scale: Optional[float] = None,
+                 window: Optional[int] = None):
+        if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
+            raise ValueError(f"head counts {n_heads}/{n_kv_heads}: the first must be a multiple of the second")
+        if head_dim <= 0 or head_dim % 16 != 0:
+            raise ValueError(f"head_dim {head_dim} must be a positive multiple of 16")
+        self.prefix = prefix
+        self.hidden = hidden
+        self.n_heads = n_heads
+        self.n_kv_heads = n_kv_heads
+        self.head_dim = head_dim
+        self.position = position
+        self.qk_norm = qk_norm
+        self.qk_norm_eps = float(qk_norm_eps)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)  # llama.rs:506
+        self.window = window
+        self.q_width = n_heads * head_dim
+        self.kv_width = n_kv_heads * head_dim
+        self.w_qkv = None
+        self.w_o = None
+        self.q_norm = None
+        self.k_norm = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        p = self.prefix
+        specs = {
+            p + "q_proj.weight": WeightSpec((self.q_width, self.hidden)),
+            p + "k_proj.weight": WeightSpec((self.kv_width, self.hidden)),
+            p + "v_proj.weight": WeightSpec((self.kv_width, self.hidden)),
+            p + "o_proj.weight": WeightSpec((self.hidden, self.q_width)),
+        }
+        if self.qk_norm:
+            specs[p + "q_norm.weight"] = WeightSpec((self.head_dim,), init="ones", kind="vector")
+            specs[p + "k_norm.weight"] = WeightSpec((self.head_dim,), init="ones", kind="vector")
+        return specs
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds(kv=KVSpec(self.n_kv_heads, self.head_dim, self.window))
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        p = self.prefix
+        self.w_qkv = torch.cat([runtime.matrix(tensors[p + name])
+                                for name in ("q_proj.weight", "k_proj.weight", "v_proj.weight")],
+                               dim=0).contiguous()
+        self.w_o = runtime.matrix(tensors[p + "o_proj.weight"])
+        if self.qk_norm:
+            self.q_norm = runtime.vector(tensors[p + "q_norm.weight"])
+            self.k_norm = runtime.vector(tensors[p + "k_norm.weight"])
+        if self.position is not None:
+            self.position.bind(tensors, runtime)
+
+    def forward(self, h: torch.Tensor, batch, cache, residual: torch.Tensor) -> None:
+        rt = self.runtime
+        ops = rt.ops
+        tokens = h.shape[0]
+        kv = cache.kv
+        qkv = rt.empty((tokens, self.q_width + 2 * self.kv_width))
+        ops.linear(h, self.w_qkv, qkv)
+
+        dims = (self.n_heads, self.n_kv_heads, self.head_dim)
+        write_to = kv if cache.writable else None
+        rotary = self.position if isinstance(self.position, Rotary) else None
+        if rotary is not None or self.position is None:
+            # one pass: head norms, rotation, cache write
+            ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots,
+                            q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.qk_norm_eps,
+                            rope_theta=None if rotary is None else rotary.theta,
+                            rope_dim=0 if rotary is None else rotary.rope_dim,
+                            rope_scale=1.0 if rotary is None else rotary.scale,
+                            kv=write_to)
+        else:
+            # any other position encoding: norms, then the encoding, then the cache write
+            if self.qk_norm:
+                ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots,
+                                q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.qk_norm_eps)
+            self.position.apply(qkv, *dims, batch)
+            if write_to is not None:
+                ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots, kv=write_to)
+
+        out = rt.empty((tokens, self.q_width))
+        ops.attention(qkv, *dims, kv, batch, out, scale=self.scale, window=self.window)
+        ops.linear(out, self.w_o, residual, accumulate=True)
+
+
+register_part("mixer", "attention", Attention)

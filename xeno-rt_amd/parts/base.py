@@ -1,0 +1,174 @@
+"""What every part of a model is: the interfaces, and the registry of part kinds.
+
+A model is put together from parts: a mixer (attention here), a feed-forward,
+norms, a position encoding, and a block that arranges them. A part is built with
+its sizes and constants as arguments and with the prefix of its tensors in the
+checkpoint; it does not know which model it is in. It says which tensors it
+binds (`weight_specs`), what it needs from the cache (`cache_needs`, mixers
+only), takes its tensors at load (`bind`) and runs on the tokens of one step
+(`forward`).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, Optional, Tuple
+
+import torch
+
+
+# ----------------------------------------------------------------------------
+# declarations a part makes
+# ----------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class WeightSpec:
+    """One tensor of the checkpoint that a part binds.
+
+    init: how the random-weights mode fills it ("normal": N(0, std), "ones", "zeros").
+    kind: "matrix" is converted to the engine's compute dtype when bound;
+          "vector" keeps 32-bit storage if the file stores it so;
+          "table" is an integer table, kept as int32.
+    """
+    shape: Tuple[int, ...]
+    init: str = "normal"
+    kind: str = "matrix"
+
+
+@dataclass(frozen=True)
+class KVSpec:
+    """Keys and values for every token: rows of n_kv_heads x head_dim.
+
+    window = None keeps all tokens; window = W keeps what a query can still see
+    when it looks at the W most recent tokens (itself included).
+    """
+    n_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """State of fixed size for each sequence, zero when the sequence starts."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class CacheNeeds:
+    kv: Optional[KVSpec] = None
+    state: Optional[StateSpec] = None
+
+
+class Runtime:
+    """What a part needs to run: the kernels, the compute dtype and the device."""
+
+    def __init__(self, ops, dtype: torch.dtype, device):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"compute dtype must be bfloat16 or float32, found {dtype}")
+        self.ops = ops
+        self.dtype = dtype
+        self.device = torch.device(device)
+
+    def matrix(self, tensor: torch.Tensor) -> torch.Tensor:
+        """A weight matrix in the compute dtype, contiguous, on the device."""
+        return tensor.to(device=self.device, dtype=self.dtype).contiguous()
+
+    def vector(self, tensor: torch.Tensor) -> torch.Tensor:
+        """A small float vector: float32 on the 32-bit path, else as the file stores it."""
+        if self.dtype == torch.float32 or tensor.dtype == torch.float32:
+            return tensor.to(device=self.device, dtype=torch.float32).contiguous()
+        return tensor.to(device=self.device, dtype=torch.bfloat16).contiguous()
+
+    def empty(self, shape, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)
+
+
+# ----------------------------------------------------------------------------
+# interfaces
+# ----------------------------------------------------------------------------
+
+class Part:
+    """Base of all parts."""
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        """Full checkpoint name -> WeightSpec of every tensor this part binds."""
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], runtime: Runtime) -> None:
+        """Take the tensors named in `weight_specs` (stored dtype, any device)."""
+        self.runtime = runtime
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Normalise the float32 rows of x (only `rows`, if given); result in the compute dtype."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def apply(self, qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, batch) -> None:
+        """Encode the positions of the step's tokens into q and k, in place.
+
+        qkv is [tokens, (n_heads + 2*n_kv_heads) * head_dim]: queries, then keys, then values.
+        """
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information along the sequence; owns what it keeps in the cache."""
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds()
+
+    def forward(self, h: torch.Tensor, batch, cache, residual: torch.Tensor) -> None:
+        """Add the mixer's output for h [tokens, hidden] to the float32 `residual`, in place.
+
+        `batch` is the step's StepBatch; `cache` the LayerCache of this call
+        (`.kv` a KVView or None, `.state` a tensor [slots, *shape] or None,
+        `.writable` False when the call reads another call's cache).
+        """
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, batch, residual: torch.Tensor) -> None:
+        """Add the feed-forward's output for h [tokens, hidden] to `residual`, in place."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    """The arrangement of a mixer, a feed-forward and their norms around the residual stream."""
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds()
+
+    def forward(self, x: torch.Tensor, batch, cache) -> None:
+        """Update the float32 residual stream x [tokens, hidden] in place."""
+        raise NotImplementedError
+
+
+# ----------------------------------------------------------------------------
+# registry of part kinds, by name
+# ----------------------------------------------------------------------------
+
+_KINDS = ("mixer", "feed_forward", "norm", "position", "block")
+_PARTS: Dict[str, Dict[str, Callable]] = {kind: {} for kind in _KINDS}
+
+
+def register_part(kind: str, name: str, factory: Callable) -> None:
+    """Make `factory(**arguments)` available to model builders as (kind, name)."""
+    if kind not in _PARTS:
+        raise KeyError(f"unknown part kind '{kind}'; kinds: {_KINDS}")
+    _PARTS[kind][name] = factory
+
+
+def create_part(kind: str, name: str, **arguments):
+    if kind not in _PARTS:
+        raise KeyError(f"unknown part kind '{kind}'; kinds: {_KINDS}")
+    if name not in _PARTS[kind]:
+        raise KeyError(f"no {kind} named '{name}'; registered: {sorted(_PARTS[kind])}")
+    return _PARTS[kind][name](**arguments)
+
+
+def registered_parts(kind: str):
+    return sorted(_PARTS[kind])

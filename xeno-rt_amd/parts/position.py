@@ -1,0 +1,45 @@
+"""Position encodings applied to queries and keys before the keys are cached.
+
+Rotary: pairs (i, i + rope_dim/2) of every head are rotated by the angle
+pos * scale / theta_i with theta_i = base^(2i/rope_dim); formulas of the
+reference's crates/xrt-kernels/src/cpu/rope.rs:10-16 (table), :59-68 (angle),
+:71-89 (rotation). Table, angle, sine and cosine are float32.
+"""
+from __future__ import annotations
+
+import torch
+
+from .base import PositionEncoding, Runtime, register_part
+
+
+class Rotary(PositionEncoding):
+    def __init__(self, rope_dim: int, base: float, scale: float = 1.0):
+        if rope_dim <= 0 or rope_dim % 2 != 0:
+            raise ValueError(f"rotary width must be positive and even, found {rope_dim}")
+        self.rope_dim = rope_dim
+        self.base = float(base)
+        self.scale = float(scale)
+        self.theta = None
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        pair = torch.arange(self.rope_dim // 2, dtype=torch.float32)
+        # float32 power, like the reference's powf (rope.rs:13)
+        theta = torch.tensor(self.base, dtype=torch.float32) ** ((2.0 * pair) / float(self.rope_dim))
+        self.theta = theta.to(runtime.device)
+
+    def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch) -> None:
+        self.runtime.ops.qkv_prepare(
+            qkv, n_heads, n_kv_heads, head_dim, batch.positions, batch.slots,
+            rope_theta=self.theta, rope_dim=self.rope_dim, rope_scale=self.scale)
+
+
+class NoPosition(PositionEncoding):
+    """Leaves queries and keys as they are."""
+
+    def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch) -> None:
+        return None
+
+
+register_part("position", "rotary", Rotary)
+register_part("position", "none", NoPosition)

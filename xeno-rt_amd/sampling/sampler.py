@@ -1,0 +1,87 @@
+"""Choosing the next token from logits.
+
+Options and their meaning are the reference's (crates/xrt-runtime/src/sampler.rs):
+temperature <= 1e-5 is greedy: the first index of the maximum (:62-65, :83-98);
+otherwise the k largest logits are kept (top_k 0 keeps all, :107, :116-145), their
+probabilities are softmax((logit - max)/temperature) (:147-164), the shortest
+descending prefix whose probability reaches top_p is kept (:166-183), and one
+uniform number picks a token by inverse CDF (:185-195). A repetition penalty > 1
+divides positive and multiplies negative logits of tokens already in the
+sequence, for greedy too (:77-91, :110-125).
+
+The work is done by one kernel on the device for all rows of a batch. Two things
+differ from the reference by design: tokens whose logit equals the k-th largest
+(or the last of the top_p prefix) are all kept, and the uniform numbers come from
+a counter-based generator keyed by (seed, request, step), so that a request draws
+the same numbers alone and in any batch.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import torch
+
+GREEDY_BELOW = 1e-5      # sampler.rs:63
+
+
+@dataclass(frozen=True)
+class SamplerConfig:
+    """Defaults are the reference's (sampler.rs:15-25)."""
+    temperature: float = 0.8
+    top_k: int = 40
+    top_p: float = 0.95
+    repetition_penalty: float = 1.1
+    seed: Optional[int] = None
+
+    def is_greedy(self) -> bool:
+        return self.temperature <= GREEDY_BELOW
+
+
+_MASK = (1 << 64) - 1
+
+
+def _mix(value: int) -> int:
+    """splitmix64 finaliser."""
+    value = (value + 0x9E3779B97F4A7C15) & _MASK
+    value = ((value ^ (value >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    value = ((value ^ (value >> 27)) * 0x94D049BB133111EB) & _MASK
+    return value ^ (value >> 31)
+
+
+def uniform(seed: int, request: int, step: int) -> float:
+    """A number in [0, 1) that depends only on (seed, request, step)."""
+    word = _mix(_mix(_mix(seed & _MASK) ^ (request & _MASK)) ^ (step & _MASK))
+    return (word >> 40) / float(1 << 24)
+
+
+class Sampler:
+    """Samples one token for each row of a batch of logits, on the device."""
+
+    def __init__(self, ops, device):
+        self.ops = ops
+        self.device = torch.device(device)
+
+    def sample(self, logits: torch.Tensor, configs: Sequence[SamplerConfig],
+               histories: Sequence[Sequence[int]], draws: Sequence[float]) -> List[int]:
+        """logits [rows, vocab] float32; for each row its options, the tokens of its sequence so
+        far (read only if its penalty is > 1) and its uniform number. Returns the token ids."""
+        rows = logits.shape[0]
+        if logits.dim() != 2 or logits.shape[1] == 0:
+            raise ValueError("cannot sample from an empty logits vector")     # sampler.rs:56-60
+        if not (rows == len(configs) == len(histories) == len(draws)):
+            raise ValueError("one config, history and draw per row of logits")
+        history: List[int] = []
+        offsets = [0]
+        for config, tokens in zip(configs, histories):
+            if config.repetition_penalty > 1.0:
+                history.extend(int(t) for t in tokens)
+            offsets.append(len(history))
+        floats = torch.tensor(
+            [[c.temperature for c in configs], [c.top_p for c in configs],
+             [c.repetition_penalty for c in configs], list(draws)], dtype=torch.float32).to(self.device)
+        ints = torch.tensor([c.top_k for c in configs] + offsets + history, dtype=torch.int32).to(self.device)
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2],
+                        ints[2 * rows + 1:], ints[rows:2 * rows + 1], floats[3])
+        return out.tolist()
