@@ -1,0 +1,79 @@
+// Shared device and host helpers of the kernel library (gfx950, 64-wide wavefronts).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+typedef __bf16 bf16;
+
+// element type codes of the C interface
+enum { XRT_F32 = 0, XRT_BF16 = 1 };
+
+// tokens per cache block; keys are [kv_head][token][dim], values [kv_head][dim][token] inside a block
+#define XRT_BLOCK_TOKENS 64
+#define XRT_WAVE 64
+
+// ---- error reporting -------------------------------------------------------
+void xrt_set_error(const char* format, ...);
+
+#define XRT_REQUIRE(condition, ...)            \
+    do {                                       \
+        if (!(condition)) {                    \
+            xrt_set_error(__VA_ARGS__);        \
+            return 1;                          \
+        }                                      \
+    } while (0)
+
+#define XRT_LAUNCH_CHECK(name)                                                      \
+    do {                                                                            \
+        hipError_t launch_error_ = hipGetLastError();                               \
+        if (launch_error_ != hipSuccess) {                                          \
+            xrt_set_error("%s: launch failed: %s", name, hipGetErrorString(launch_error_)); \
+            return 1;                                                               \
+        }                                                                           \
+    } while (0)
+
+// ---- conversions -----------------------------------------------------------
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16 v) { return (float)v; }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16 from_float<bf16>(float v) { return (bf16)v; }   // round to nearest even
+
+// ---- wave reductions (fixed butterfly order: results do not depend on the launch) ----
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int offset = XRT_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, XRT_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int offset = XRT_WAVE / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, XRT_WAVE));
+    return v;
+}
+
+// Orders the LDS accesses of the lanes of one wavefront: what any lane wrote before is
+// seen by every lane after. (A wavefront's LDS operations execute in order; the fences keep
+// the compiler from moving accesses across.)
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// sum over a block of up to 1024 threads; every thread gets the result. `scratch` holds 32 floats.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
+    const int waves = (blockDim.x + XRT_WAVE - 1) / XRT_WAVE;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < waves; ++w) total += scratch[w];
+    return total;
+}

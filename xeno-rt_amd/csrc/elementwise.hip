@@ -1,0 +1,84 @@
+// Embedding gather, residual add and RMSNorm.
+//
+// RMSNorm: y = (x * r) * w, r = 1/sqrt(mean(x^2) + eps), all in float32
+// (reference: crates/xrt-kernels/src/cpu/rmsnorm.rs:26-43). One workgroup per row;
+// the order of the sum depends only on the row length, so a row's result is the
+// same in any batch.
+#include "common.h"
+#include "xrt_hip.h"
+
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int hidden) {
+    const long token = blockIdx.x;
+    const T* row = table + (long)ids[token] * hidden;
+    float* dst = out + token * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]);
+}
+
+template <typename T>
+__global__ void add_kernel(float* __restrict__ residual, const T* __restrict__ delta, long count) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) residual[i] += to_float(delta[i]);
+}
+
+template <typename TW, typename TO>
+__global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ weight,
+                                                      float eps, TO* __restrict__ out,
+                                                      const int* __restrict__ rows, int hidden) {
+    __shared__ float scratch[32];
+    const long src = rows ? rows[blockIdx.x] : blockIdx.x;
+    const float* row = x + src * hidden;
+    TO* dst = out + (long)blockIdx.x * hidden;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) sum = fmaf(row[i], row[i], sum);
+    sum = block_sum(sum, scratch);
+    const float inv_rms = 1.0f / sqrtf(sum / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+        dst[i] = from_float<TO>((row[i] * inv_rms) * to_float(weight[i]));
+}
+
+extern "C" int xrt_embed(const void* table, int table_dtype, const int* ids, float* out, int tokens,
+                         int hidden, int vocab, void* stream) {
+    XRT_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes tokens=%d hidden=%d vocab=%d", tokens, hidden, vocab);
+    XRT_REQUIRE(table_dtype == XRT_F32 || table_dtype == XRT_BF16, "embed: unknown dtype %d", table_dtype);
+    if (tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (table_dtype == XRT_F32)
+        embed_kernel<float><<<tokens, 256, 0, s>>>((const float*)table, ids, out, hidden);
+    else
+        embed_kernel<bf16><<<tokens, 256, 0, s>>>((const bf16*)table, ids, out, hidden);
+    XRT_LAUNCH_CHECK("embed");
+    return 0;
+}
+
+extern "C" int xrt_add(float* residual, const void* delta, int delta_dtype, long count, void* stream) {
+    XRT_REQUIRE(count >= 0, "add: negative count");
+    XRT_REQUIRE(delta_dtype == XRT_F32 || delta_dtype == XRT_BF16, "add: unknown dtype %d", delta_dtype);
+    if (count == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned blocks = (unsigned)((count + 255) / 256);
+    if (delta_dtype == XRT_F32)
+        add_kernel<float><<<blocks, 256, 0, s>>>(residual, (const float*)delta, count);
+    else
+        add_kernel<bf16><<<blocks, 256, 0, s>>>(residual, (const bf16*)delta, count);
+    XRT_LAUNCH_CHECK("add");
+    return 0;
+}
+
+extern "C" int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype, float eps, void* out,
+                           int out_dtype, const int* rows, int n_rows, int hidden, void* stream) {
+    XRT_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d hidden=%d", n_rows, hidden);
+    XRT_REQUIRE((weight_dtype == XRT_F32 || weight_dtype == XRT_BF16) && (out_dtype == XRT_F32 || out_dtype == XRT_BF16),
+                "rmsnorm: unknown dtype weight=%d out=%d", weight_dtype, out_dtype);
+    if (n_rows == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+#define XRT_RMS(TW, TO) rmsnorm_kernel<TW, TO><<<n_rows, 256, 0, s>>>(x, (const TW*)weight, eps, (TO*)out, rows, hidden)
+    if (weight_dtype == XRT_F32 && out_dtype == XRT_F32) XRT_RMS(float, float);
+    else if (weight_dtype == XRT_F32) XRT_RMS(float, bf16);
+    else if (out_dtype == XRT_F32) XRT_RMS(bf16, float);
+    else XRT_RMS(bf16, bf16);
+#undef XRT_RMS
+    XRT_LAUNCH_CHECK("rmsnorm");
+    return 0;
+}

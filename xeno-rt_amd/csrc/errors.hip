@@ -1,0 +1,14 @@
+// Last-error text of the calling thread.
+#include "common.h"
+#include "xrt_hip.h"
+
+static thread_local char last_error_text[1024] = "";
+
+void xrt_set_error(const char* format, ...) {
+    va_list arguments;
+    va_start(arguments, format);
+    vsnprintf(last_error_text, sizeof(last_error_text), format, arguments);
+    va_end(arguments);
+}
+
+extern "C" const char* xrt_last_error(void) { return last_error_text; }

@@ -1,0 +1,133 @@
+// Plain tiled matrix product out[m, n] = sum_k a[m, k] * w[n, k] with float32 accumulation
+// on the vector ALUs (no matrix cores, no reduced precision): the product of the 32-bit
+// path, and the fallback of the bfloat16 path for shapes its fast kernels refuse.
+//
+// Every output element is the sum over k = 0, 1, 2, ... in that order, whatever the
+// number of rows, the tile it falls in or the batch around it; so a token's result does
+// not depend on how a request was cut into steps. Semantics of the reference's
+// row-major matvec (crates/xrt-kernels/src/cpu/matmul.rs:153-167, 269-288): w is
+// [out][in], no bias.
+#include "common.h"
+#include "xrt_hip.h"
+
+namespace {
+
+constexpr int BM = 64, BN = 64, BK = 16, PAD = 4;
+enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
+
+template <typename T>
+__device__ __forceinline__ void load4(const T* __restrict__ base, long row, int n_rows, int k, int K,
+                                      bool vector_ok, float (&v)[4]) {
+    if (row < n_rows && vector_ok && k + 3 < K) {
+        const T* p = base + row * (long)K + k;
+        if constexpr (sizeof(T) == 4) {
+            const float4 q = *reinterpret_cast<const float4*>(p);
+            v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        } else {
+            struct alignas(8) Four { T e[4]; };
+            const Four q = *reinterpret_cast<const Four*>(p);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = to_float(q.e[i]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            v[i] = (row < n_rows && k + i < K) ? to_float(base[row * (long)K + k + i]) : 0.f;
+    }
+}
+
+__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }   // silu.rs:1-3
+
+template <typename TI, typename TO, int MODE>
+__global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__ a, const TI* __restrict__ w,
+                                                          TO* __restrict__ out, int M, int N, int K,
+                                                          int vector_ok) {
+    __shared__ __attribute__((aligned(16))) float As[BK][BM + PAD];
+    __shared__ __attribute__((aligned(16))) float Ws[BK][BN + PAD];
+    __shared__ __attribute__((aligned(16))) float Us[MODE == MODE_GATED ? BK : 1][BN + PAD];
+
+    const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+    const long m0 = (long)blockIdx.y * BM, n0 = (long)blockIdx.x * BN;
+    const int load_row = tid / 4, load_k = (tid % 4) * 4;
+
+    float acc[4][4] = {}, acc_up[MODE == MODE_GATED ? 4 : 1][4] = {};
+
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        float va[4], vw[4];
+        load4(a, m0 + load_row, M, k0 + load_k, K, vector_ok, va);
+        load4(w, n0 + load_row, N, k0 + load_k, K, vector_ok, vw);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            As[load_k + i][load_row] = va[i];
+            Ws[load_k + i][load_row] = vw[i];
+        }
+        if constexpr (MODE == MODE_GATED) {
+            float vu[4];
+            // rows of the "up" half follow the N rows of the "gate" half
+            load4(w + (long)N * K, n0 + load_row, N, k0 + load_k, K, vector_ok, vu);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) Us[load_k + i][load_row] = vu[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK; ++kk) {
+            const float4 av = *reinterpret_cast<const float4*>(&As[kk][ty * 4]);
+            const float4 wv = *reinterpret_cast<const float4*>(&Ws[kk][tx * 4]);
+            const float ar[4] = {av.x, av.y, av.z, av.w};
+            const float wr[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
+            if constexpr (MODE == MODE_GATED) {
+                const float4 uv = *reinterpret_cast<const float4*>(&Us[kk][tx * 4]);
+                const float ur[4] = {uv.x, uv.y, uv.z, uv.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc_up[i][j] = fmaf(ar[i], ur[j], acc_up[i][j]);
+            }
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const long m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const long n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            TO* dst = out + m * (long)N + n;
+            if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(acc[i][j]);
+            if constexpr (MODE == MODE_ACCUMULATE) *dst = from_float<TO>(to_float(*dst) + acc[i][j]);
+            if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(silu(acc[i][j]) * acc_up[i][j]);
+        }
+    }
+}
+
+template <typename TI, typename TO>
+int launch(const void* a, const void* w, void* out, int M, int N, int K, int mode, hipStream_t s) {
+    const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+    const int vector_ok = (K % 4 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
+    if (mode == MODE_STORE)
+        gemm_simple_kernel<TI, TO, MODE_STORE><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+    else if (mode == MODE_ACCUMULATE)
+        gemm_simple_kernel<TI, TO, MODE_ACCUMULATE><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+    else
+        gemm_simple_kernel<TI, TO, MODE_GATED><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+    XRT_LAUNCH_CHECK("linear (plain)");
+    return 0;
+}
+
+}  // namespace
+
+int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
+                     int mode, hipStream_t s) {
+    if (dtype == XRT_F32 && out_dtype == XRT_F32) return launch<float, float>(a, w, out, M, N, K, mode, s);
+    if (dtype == XRT_BF16 && out_dtype == XRT_F32) return launch<bf16, float>(a, w, out, M, N, K, mode, s);
+    if (dtype == XRT_BF16 && out_dtype == XRT_BF16) return launch<bf16, bf16>(a, w, out, M, N, K, mode, s);
+    xrt_set_error("linear: unsupported dtypes in=%d out=%d", dtype, out_dtype);
+    return 1;
+}

@@ -1,0 +1,19 @@
+// Entry point of all matrix products: checks the operands and picks the kernel.
+#include "common.h"
+#include "xrt_hip.h"
+
+int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
+                     int mode, hipStream_t s);
+
+extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N,
+                          int K, int mode, void* stream) {
+    XRT_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
+    XRT_REQUIRE(mode >= 0 && mode <= 2, "linear: unknown mode %d", mode);
+    XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "linear: unknown dtype %d", dtype);
+    XRT_REQUIRE(out_dtype == XRT_F32 || out_dtype == XRT_BF16, "linear: unknown output dtype %d", out_dtype);
+    XRT_REQUIRE(!(dtype == XRT_F32 && out_dtype == XRT_BF16), "linear: float32 operands need a float32 output");
+    XRT_REQUIRE(mode != 1 || out_dtype == XRT_F32, "linear: accumulation needs a float32 output");
+    XRT_REQUIRE(a && w && out, "linear: null operand");
+    if (M == 0) return 0;
+    return xrt_linear_plain(a, w, dtype, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
+}

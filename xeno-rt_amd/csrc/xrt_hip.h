@@ -1,0 +1,50 @@
+// C interface of the kernel library. Every function returns 0 on success; otherwise
+// xrt_last_error() describes what was refused. Pointers are device pointers unless
+// said otherwise; `stream` is a hipStream_t. Element type codes: 0 = float32, 1 = bfloat16.
+#pragma once
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* xrt_last_error(void);
+
+// out[t, :] = table[ids[t], :] as float32
+int xrt_embed(const void* table, int table_dtype, const int* ids, float* out, int tokens, int hidden,
+              int vocab, void* stream);
+
+// residual[i] += delta[i]
+int xrt_add(float* residual, const void* delta, int delta_dtype, long count, void* stream);
+
+// out[r, :] = rmsnorm(x[rows ? rows[r] : r, :]) * weight ; x float32, out of out_dtype
+int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype, float eps, void* out, int out_dtype,
+                const int* rows, int n_rows, int hidden, void* stream);
+
+// out[m, n] (+)= sum_k a[m, k] * w[n, k]   (mode 0 store, 1 accumulate into float32 out,
+// 2 gated: out[m, n] = silu(a.w[n]) * (a.w[n + N]) with w of 2N rows)
+int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
+               int mode, void* stream);
+
+// per-head RMSNorm of q and k (optional), rotation of q and k (optional), write of k and v
+// into the cache (optional); qkv rows are [q heads | k heads | v heads]
+int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
+                    const int* positions, const int* slots,
+                    const void* q_norm, const void* k_norm, int norm_dtype, float norm_eps,
+                    const float* rope_theta, int rope_dim, float rope_scale,
+                    void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                    void* stream);
+
+// causal attention of every token over its sequence's cache
+int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
+                  const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
+                  int n_blocks, const int* positions, const int* slots, void* out, float scale, int window,
+                  void* stream);
+
+// one token per row of float32 logits
+int xrt_sample(const float* logits, int rows, int vocab, int* out, const float* temperature,
+               const int* top_k, const float* top_p, const float* penalty, const int* history,
+               const int* history_offsets, const float* uniforms, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,197 @@
+"""Python face of the HIP kernel library: checks tensors, passes raw pointers.
+
+Every operation works on the current torch stream of the tensors' device. A
+tensor of the wrong dtype, shape, layout or device is refused here, before a
+kernel could read outside of it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+_CODES = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    """The kernel library refused an operation, or could not be loaded."""
+
+
+def _code(tensor: torch.Tensor) -> int:
+    if tensor.dtype not in _CODES:
+        raise KernelError(f"unsupported element type {tensor.dtype}")
+    return _CODES[tensor.dtype]
+
+
+def _ptr(tensor: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
+
+
+class HipOps:
+    name = "hip"
+    _instance = None
+
+    @classmethod
+    def instance(cls) -> "HipOps":
+        if cls._instance is None:
+            cls._instance = cls()
+        return cls._instance
+
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: the kernels of this library run on an MI355X only")
+        path = _build.find_library()
+        if path is None:
+            try:
+                path = _build.build()
+            except _build.BuildError as error:
+                raise KernelError(f"the HIP kernel library is missing and cannot be built: {error}") from None
+        try:
+            self.lib = ctypes.CDLL(path)
+        except OSError as error:
+            raise KernelError(f"cannot load {path}: {error}") from None
+        self.path = path
+        self.lib.xrt_last_error.restype = ctypes.c_char_p
+        for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
+                     "xrt_attention", "xrt_sample"):
+            getattr(self.lib, name).restype = ctypes.c_int
+
+    # -- helpers -------------------------------------------------------------
+    def _check(self, status: int) -> None:
+        if status != 0:
+            raise KernelError(self.lib.xrt_last_error().decode())
+
+    @staticmethod
+    def _stream(tensor: torch.Tensor):
+        return ctypes.c_void_p(torch.cuda.current_stream(tensor.device).cuda_stream)
+
+    @staticmethod
+    def _require(tensor: torch.Tensor, what: str, dtype=None, shape=None, like=None) -> None:
+        if not isinstance(tensor, torch.Tensor) or not tensor.is_cuda:
+            raise KernelError(f"{what}: expected a tensor on the GPU")
+        if like is not None and tensor.device != like.device:
+            raise KernelError(f"{what}: on {tensor.device}, expected {like.device}")
+        if not tensor.is_contiguous():
+            raise KernelError(f"{what}: must be contiguous")
+        if dtype is not None and tensor.dtype != dtype:
+            raise KernelError(f"{what}: dtype {tensor.dtype}, expected {dtype}")
+        if shape is not None and tuple(tensor.shape) != tuple(shape):
+            raise KernelError(f"{what}: shape {tuple(tensor.shape)}, expected {tuple(shape)}")
+
+    # -- operations ----------------------------------------------------------
+    def embed(self, table, ids, out):
+        vocab, hidden = table.shape
+        tokens = ids.shape[0]
+        self._require(table, "embed table")
+        self._require(ids, "embed ids", torch.int32, (tokens,), table)
+        self._require(out, "embed out", torch.float32, (tokens, hidden), table)
+        self._check(self.lib.xrt_embed(_ptr(table), _code(table), _ptr(ids), _ptr(out), tokens, hidden, vocab,
+                                       self._stream(out)))
+
+    def add(self, residual, delta):
+        self._require(residual, "add residual", torch.float32)
+        self._require(delta, "add delta", None, residual.shape, residual)
+        self._check(self.lib.xrt_add(_ptr(residual), _ptr(delta), _code(delta),
+                                     ctypes.c_long(residual.numel()), self._stream(residual)))
+
+    def rmsnorm(self, x, weight, eps, out, rows=None):
+        hidden = x.shape[-1]
+        self._require(x, "rmsnorm x", torch.float32)
+        if x.dim() != 2:
+            raise KernelError("rmsnorm x: expected [rows, hidden]")
+        n_rows = x.shape[0] if rows is None else rows.shape[0]
+        self._require(weight, "rmsnorm weight", None, (hidden,), x)
+        self._require(out, "rmsnorm out", None, (n_rows, hidden), x)
+        if rows is not None:
+            self._require(rows, "rmsnorm rows", torch.int32, (n_rows,), x)
+        self._check(self.lib.xrt_rmsnorm(_ptr(x), _ptr(weight), _code(weight), ctypes.c_float(eps), _ptr(out),
+                                         _code(out), _ptr(rows), n_rows, hidden, self._stream(x)))
+
+    def _linear(self, a, w, out, mode, n):
+        if a.dim() != 2 or w.dim() != 2:
+            raise KernelError("linear: operands must be [rows, k]")
+        m, k = a.shape
+        self._require(a, "linear a")
+        self._require(w, "linear w", a.dtype, None, a)
+        if w.shape[1] != k:
+            raise KernelError(f"linear: a has {k} columns, w has {w.shape[1]}")
+        self._require(out, "linear out", None, (m, n), a)
+        self._check(self.lib.xrt_linear(_ptr(a), _ptr(w), _code(a), _ptr(out), _code(out), m, n, k, mode,
+                                        self._stream(a)))
+
+    def linear(self, a, w, out, accumulate=False):
+        self._linear(a, w, out, 1 if accumulate else 0, w.shape[0])
+
+    def linear_glu(self, a, w_gate_up, out):
+        if w_gate_up.shape[0] % 2 != 0:
+            raise KernelError("linear_glu: the weight needs gate rows followed by as many up rows")
+        self._linear(a, w_gate_up, out, 2, w_gate_up.shape[0] // 2)
+
+    def qkv_prepare(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm=None, k_norm=None,
+                    norm_eps=0.0, rope_theta=None, rope_dim=0, rope_scale=1.0, kv=None):
+        tokens = qkv.shape[0]
+        width = (n_heads + 2 * n_kv_heads) * head_dim
+        self._require(qkv, "qkv", None, (tokens, width))
+        self._require(positions, "positions", torch.int32, (tokens,), qkv)
+        self._require(slots, "slots", torch.int32, (tokens,), qkv)
+        if (q_norm is None) != (k_norm is None):
+            raise KernelError("qkv_prepare: q_norm and k_norm come together")
+        norm_code = 0
+        if q_norm is not None:
+            self._require(q_norm, "q_norm", None, (head_dim,), qkv)
+            self._require(k_norm, "k_norm", q_norm.dtype, (head_dim,), qkv)
+            norm_code = _code(q_norm)
+        if rope_theta is not None:
+            self._require(rope_theta, "rope_theta", torch.float32, (rope_dim // 2,), qkv)
+        k_cache = v_cache = table = None
+        stride = n_blocks = 0
+        if kv is not None:
+            k_cache, v_cache, table, stride, n_blocks = self._kv(kv, qkv, n_kv_heads, head_dim)
+        self._check(self.lib.xrt_qkv_prepare(
+            _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(positions), _ptr(slots),
+            _ptr(q_norm), _ptr(k_norm), norm_code, ctypes.c_float(norm_eps), _ptr(rope_theta), int(rope_dim),
+            ctypes.c_float(rope_scale), _ptr(k_cache), _ptr(v_cache), _ptr(table), stride, n_blocks,
+            self._stream(qkv)))
+
+    def _kv(self, kv, like, n_kv_heads, head_dim):
+        from ..cache import BLOCK_TOKENS
+        n_blocks = kv.k.shape[0]
+        self._require(kv.k, "key cache", like.dtype, (n_blocks, n_kv_heads, BLOCK_TOKENS, head_dim), like)
+        self._require(kv.v, "value cache", like.dtype, (n_blocks, n_kv_heads, head_dim, BLOCK_TOKENS), like)
+        self._require(kv.block_table, "block table", torch.int32, None, like)
+        if kv.block_table.dim() != 2:
+            raise KernelError("block table: expected [slots, blocks]")
+        return kv.k, kv.v, kv.block_table, kv.block_table.shape[1], n_blocks
+
+    def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None):
+        tokens = qkv.shape[0]
+        width = (n_heads + 2 * n_kv_heads) * head_dim
+        self._require(qkv, "qkv", None, (tokens, width))
+        self._require(out, "attention out", qkv.dtype, (tokens, n_heads * head_dim), qkv)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), qkv)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), qkv)
+        k_cache, v_cache, table, stride, n_blocks = self._kv(kv, qkv, n_kv_heads, head_dim)
+        self._check(self.lib.xrt_attention(
+            _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(k_cache), _ptr(v_cache),
+            _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out),
+            ctypes.c_float(scale), int(window or 0), self._stream(qkv)))
+
+    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms):
+        if logits.dim() != 2:
+            raise KernelError("sample: logits must be [rows, vocab]")
+        rows, vocab = logits.shape
+        self._require(logits, "logits", torch.float32)
+        self._require(out, "sample out", torch.int32, (rows,), logits)
+        for what, tensor, dtype, shape in (
+                ("temperature", temperature, torch.float32, (rows,)), ("top_k", top_k, torch.int32, (rows,)),
+                ("top_p", top_p, torch.float32, (rows,)), ("penalty", penalty, torch.float32, (rows,)),
+                ("history_offsets", history_offsets, torch.int32, (rows + 1,)),
+                ("uniforms", uniforms, torch.float32, (rows,)), ("history", history, torch.int32, None)):
+            self._require(tensor, f"sample {what}", dtype, shape, logits)
+        self._check(self.lib.xrt_sample(_ptr(logits), rows, vocab, _ptr(out), _ptr(temperature), _ptr(top_k),
+                                        _ptr(top_p), _ptr(penalty), _ptr(history), _ptr(history_offsets),
+                                        _ptr(uniforms), self._stream(logits)))
