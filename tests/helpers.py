@@ -1,0 +1,95 @@
+"""Helpers of the GPU tests: tolerances, schedules, comparison with the plain model."""
+import torch
+
+# Largest difference allowed between the engine's logits and the plain implementation's,
+# relative to the largest logit of the compared block.
+#   float32: both sides round each operation to 2^-24; sums of a few hundred terms in
+#            different orders differ by about 1e-6 of the largest term.
+#   bfloat16: activations are rounded to 8 bits (2^-9 relative) about six times per layer;
+#            with the tests' weights (std 0.2: sharp attention, gains above one) that comes
+#            to one or two percent of the largest logit. The root-mean-square bound is
+#            tighter because it does not ride on the single worst element.
+TOLERANCE = {"float32": dict(max=2e-5, rms=5e-6), "bfloat16": dict(max=5e-2, rms=1.5e-2)}
+
+
+def errors(got: torch.Tensor, want: torch.Tensor):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    assert got.shape == want.shape, (got.shape, want.shape)
+    scale = float(want.abs().max())
+    diff = got - want
+    return float(diff.abs().max()) / scale, float(diff.pow(2).mean().sqrt()) / scale
+
+
+def assert_logits(got, want, dtype, what=""):
+    assert torch.isfinite(got).all(), f"{what}: logits are not finite"
+    worst, rms = errors(got, want)
+    limit = TOLERANCE[dtype]
+    assert worst <= limit["max"] and rms <= limit["rms"], \
+        f"{what} [{dtype}]: max error {worst:.3e} (limit {limit['max']:.1e}), rms {rms:.3e} (limit {limit['rms']:.1e})"
+    return worst, rms
+
+
+def first_bad_position(got, want, dtype):
+    """Index of the first row whose error exceeds the limit, or None: where to look first."""
+    limit = TOLERANCE[dtype]["max"]
+    scale = float(want.abs().max())
+    for t in range(want.shape[0]):
+        if float((got[t].double().cpu() - want[t].double()).abs().max()) / scale > limit:
+            return t
+    return None
+
+
+def token_ids(vocab, length, seed):
+    return torch.randint(0, vocab, (length,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def run_whole(engine, ids):
+    """One request alone, whole, logits at every position."""
+    slot = engine.alloc_slot()
+    try:
+        return engine.step([(slot, ids, list(range(len(ids))))])
+    finally:
+        engine.free_slot(slot)
+
+
+def run_tail_decoded(engine, ids, tail=32):
+    """The first len - tail tokens in one step (at least one), the rest one by one."""
+    head = max(1, len(ids) - tail)
+    slot = engine.alloc_slot()
+    try:
+        rows = [engine.step([(slot, ids[:head], list(range(head)))])]
+        for t in range(head, len(ids)):
+            rows.append(engine.step([(slot, [ids[t]], [0])]))
+        return torch.cat(rows)
+    finally:
+        engine.free_slot(slot)
+
+
+def run_batched(engine, requests, prompts):
+    """All requests start together: request i brings its first prompts[i] tokens in one step, then
+    one token per step; a request whose tokens are used up ends (its slot is freed) while the
+    others go on. Returns the logits [len, vocab] of every request."""
+    slots = [engine.alloc_slot() for _ in requests]
+    rows = [[] for _ in requests]
+    done = [False] * len(requests)
+    try:
+        logits = engine.step([(slot, ids[:p], list(range(p))) for slot, ids, p in zip(slots, requests, prompts)])
+        at = 0
+        for i, p in enumerate(prompts):
+            rows[i].append(logits[at:at + p]); at += p
+        position = list(prompts)
+        while True:
+            for i, ids in enumerate(requests):
+                if not done[i] and position[i] >= len(ids):
+                    engine.free_slot(slots[i]); done[i] = True
+            live = [i for i in range(len(requests)) if not done[i]]
+            if not live:
+                break
+            logits = engine.step([(slots[i], [requests[i][position[i]]], [0]) for i in live])
+            for row, i in enumerate(live):
+                rows[i].append(logits[row:row + 1]); position[i] += 1
+        return [torch.cat(r) for r in rows]
+    finally:
+        for i, slot in enumerate(slots):
+            if not done[i]:
+                engine.free_slot(slot)

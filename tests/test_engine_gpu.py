@@ -1,0 +1,153 @@
+"""The engine on the GPU against the plain implementation: whole requests, decoded tails,
+unequal batches with slot reuse, long decoding, first tokens, greedy generation; in 32-bit
+and in bfloat16, for two tiny configurations that differ in every size and option."""
+import pytest
+import torch
+
+from conftest import TINY, make_folder
+from helpers import (TOLERANCE, assert_logits, first_bad_position, run_batched, run_tail_decoded, run_whole,
+                     token_ids)
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+LENGTHS = {"llama": [5, 11, 17, 64, 65, 128], "qwen3": [1, 7, 23, 30, 129, 200]}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """name -> (folder, plain model, {length: (ids, plain logits)})"""
+    out = {}
+    for name in ("llama", "qwen3"):
+        folder = make_folder(TINY[name], tmp_path_factory.mktemp(name), seed=31 if name == "llama" else 47, std=0.2)
+        plain = P.PlainModel(folder)
+        cases = {}
+        for index, length in enumerate(LENGTHS[name]):
+            ids = token_ids(plain.config.vocab_size, length, seed=100 + index)
+            cases[length] = (ids, plain.logits(ids))
+        out[name] = (folder, plain, cases)
+    return out
+
+
+@pytest.fixture(scope="module")
+def engines(models):
+    from xeno_rt_amd.engine import Engine
+    cache = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in cache:
+            # eight blocks and three slots: batches must reuse both
+            cache[(name, dtype)] = Engine.load(models[name][0], dtype=dtype, max_tokens=64 * 8, max_slots=3)
+        return cache[(name, dtype)]
+    return get
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["llama", "qwen3"])
+def test_each_request_alone_and_whole(name, dtype, models, engines):
+    engine = engines(name, dtype)
+    for length, (ids, want) in models[name][2].items():
+        got = run_whole(engine, ids)
+        assert_logits(got, want, dtype, f"{name} whole length {length}, first bad row {first_bad_position(got, want, dtype)}")
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["llama", "qwen3"])
+def test_last_32_tokens_one_by_one(name, dtype, models, engines):
+    engine = engines(name, dtype)
+    for length, (ids, want) in models[name][2].items():
+        got = run_tail_decoded(engine, ids)
+        assert_logits(got, want, dtype, f"{name} decoded tail length {length}, first bad row {first_bad_position(got, want, dtype)}")
+        if dtype == "float32":
+            # the 32-bit kernels sum in an order that does not depend on the step's shape
+            assert torch.equal(got, run_whole(engine, ids)), f"{name} length {length}: cutting changed float32 bits"
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["llama", "qwen3"])
+def test_unequal_batches_one_after_another(name, dtype, models, engines):
+    engine = engines(name, dtype)
+    cases = models[name][2]
+    lengths = LENGTHS[name]
+    # three batches through three slots; prompts are shorter than the requests, so the tail of
+    # every request is decoded, and shorter requests end while longer ones go on
+    batches = [lengths[0:3], lengths[3:5] + [lengths[1]], [lengths[5], lengths[0], lengths[2]]]
+    for batch in batches:
+        requests = [cases[n][0] for n in batch]
+        prompts = [max(1, n - 1 - 3 * i) for i, n in enumerate(batch)]
+        got = run_batched(engine, requests, prompts)
+        for n, logits in zip(batch, got):
+            assert_logits(logits, cases[n][1], dtype,
+                          f"{name} batch {batch} request of {n}, first bad row {first_bad_position(logits, cases[n][1], dtype)}")
+            if dtype == "float32":
+                assert torch.equal(logits, run_whole(engine, cases[n][0])), f"{name} {n}: batching changed float32 bits"
+        engine.cache.check()
+        assert engine.cache.slots.n_held == 0 and engine.cache.held_blocks() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["llama", "qwen3"])
+def test_long_decoding_from_the_first_token(name, dtype, models, engines):
+    engine = engines(name, dtype)
+    folder, plain, _ = models[name]
+    length = plain.config.max_position            # up to the last position of the context
+    ids = token_ids(plain.config.vocab_size, length, seed=9)
+    want = plain.logits(ids)
+    got = run_tail_decoded(engine, ids, tail=length - 1)      # one token, then all others one by one
+    assert_logits(got[:4], want[:4], dtype, f"{name} first tokens")
+    assert_logits(got, want, dtype, f"{name} long decoding, first bad row {first_bad_position(got, want, dtype)}")
+    assert engine.cache.held_blocks() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["llama", "qwen3"])
+def test_greedy_generation_through_the_entry_point(name, dtype, models, engines):
+    from xeno_rt_amd.engine import GenerateRequest, generate
+    engine = engines(name, dtype)
+    folder, plain, cases = models[name]
+    prompts = [cases[n][0] for n in LENGTHS[name][:4]] + [[]]
+    limits = [9, 14, 5, 12, 4]
+    requests = [GenerateRequest(p, max_tokens=n, temperature=0.0, repetition_penalty=1.0, stop_ids=[])
+                for p, n in zip(prompts, limits)]
+    results = generate(engine, requests, batch_size=3)
+    bos = [plain.config.bos_id]
+    for prompt, limit, result in zip(prompts, limits, results):
+        assert len(result.tokens) == limit and result.finish_reason == "length"
+        if dtype == "float32":
+            assert result.tokens == P.generate_greedy(plain, prompt, limit, stop_ids=[])
+        else:
+            # bfloat16 may pick another of two near-equal logits: every chosen token must be
+            # the plain model's best within the tolerance, given the tokens chosen before it
+            history = list(prompt or bos)
+            for token in result.tokens:
+                row = plain.logits(history)[-1]
+                assert float(row.max() - row[token]) <= 2 * TOLERANCE[dtype]["max"] * float(row.abs().max())
+                history.append(token)
+    # stop tokens: the request ends before the token, the others go on
+    free = results[1].tokens
+    again = generate(engine, [GenerateRequest(prompts[1], max_tokens=14, temperature=0.0, repetition_penalty=1.0,
+                                              stop_ids=[free[5]]),
+                              GenerateRequest(prompts[0], max_tokens=9, temperature=0.0, repetition_penalty=1.0,
+                                              stop_ids=[])])
+    assert again[0].tokens == free[:free.index(free[5])] and again[0].finish_reason == "stop"
+    assert again[1].tokens == results[0].tokens
+    engine.cache.check()
+    assert engine.cache.slots.n_held == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_far_keys_among_hundreds(dtype, tmp_path):
+    """Several hundred tokens of context with weights that make attention sharp: the keys that
+    matter lie far back, in other cache blocks than the query."""
+    from xeno_rt_amd.engine import Engine
+    raw = dict(TINY["llama"], max_position_embeddings=1024, num_hidden_layers=1, rope_theta=50000.0)
+    folder = make_folder(raw, tmp_path / "far", seed=5, std=0.3)
+    plain = P.PlainModel(folder)
+    ids = token_ids(plain.config.vocab_size, 700, seed=3)
+    want = plain.logits(ids)
+    engine = Engine.load(folder, dtype=dtype, max_tokens=1024)
+    assert_logits(run_whole(engine, ids), want, dtype, "700 tokens whole")
+    got = run_tail_decoded(engine, ids)
+    assert_logits(got, want, dtype, f"700 tokens, tail decoded, first bad row {first_bad_position(got, want, dtype)}")

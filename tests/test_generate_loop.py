@@ -1,0 +1,175 @@
+"""The generation loop's decisions and the step function's checks, on the CPU: the
+engine's own step function, cache and loop run with the test stand-in for the kernels."""
+import pytest
+import torch
+
+from conftest import TINY, make_folder
+from ops_emulation import EmulatedOps
+import plain_llama as P
+from xeno_rt_amd.engine import (Engine, GenerateRequest, StepError, decide, generate, plan_batches,
+                                resolve_prompt)
+from xeno_rt_amd.sampling import SamplerConfig, uniform
+
+GREEDY = dict(temperature=0.0, repetition_penalty=1.0)
+
+
+@pytest.fixture(scope="module")
+def pair(tmp_path_factory):
+    folder = make_folder(TINY["llama"], tmp_path_factory.mktemp("loop"), seed=4, std=0.2)
+    engine = Engine.load(folder, dtype="float32", device="cpu", ops=EmulatedOps(), max_tokens=64 * 6, max_slots=3)
+    return engine, P.PlainModel(folder)
+
+
+def test_decide_follows_the_references_order():
+    stops = {1}
+    assert decide(1, stops, 5, 10, 0, 4) == (False, "stop")          # session.rs:117-119, checked first
+    assert decide(7, stops, 10, 10, 0, 4) == (False, "context")      # session.rs:120-122
+    assert decide(1, stops, 10, 10, 0, 4) == (False, "stop")
+    assert decide(7, stops, 5, 10, 0, 4) == (True, None)
+    assert decide(7, stops, 5, 10, 3, 4) == (True, "length")         # the last allowed token is kept
+    assert decide(7, set(), 5, 10, 0, 1) == (True, "length")
+
+
+def test_resolve_prompt():
+    assert resolve_prompt([], 3, 10) == [3]                          # session.rs:78-86
+    with pytest.raises(ValueError, match="no BOS"):
+        resolve_prompt([], None, 10)
+    with pytest.raises(ValueError, match="exceeds model context length"):
+        resolve_prompt(list(range(11)), 0, 10)                       # session.rs:87-93
+    assert resolve_prompt(list(range(10)), 0, 10) == list(range(10))
+
+
+def test_plan_batches_respects_slots_and_cache():
+    assert plan_batches([5, 5, 5, 5, 5], [10] * 5, 2, 64, 64 * 100, 128) == [[0, 1], [2, 3], [4]]
+    # 60 + 10 tokens round up to 128 each: two fit into 256, not three
+    assert plan_batches([60, 60, 60], [10, 10, 10], 8, 64, 256, 128) == [[0, 1], [2]]
+    # the context bounds what a request can come to hold
+    assert plan_batches([60, 60], [1000, 1000], 8, 64, 256, 128) == [[0, 1]]
+    with pytest.raises(ValueError, match="may hold"):
+        plan_batches([300], [10], 8, 64, 256, 512)
+
+
+def test_uniform_depends_on_seed_and_step_only():
+    draws = [uniform(5, 0, step) for step in range(200)]
+    assert all(0.0 <= d < 1.0 for d in draws) and len(set(draws)) > 190
+    assert draws[:3] == [uniform(5, 0, 0), uniform(5, 0, 1), uniform(5, 0, 2)]
+    assert uniform(6, 0, 0) != draws[0]
+    assert 0.4 < sum(draws) / len(draws) < 0.6
+
+
+def test_batches_of_unequal_prompts_match_the_plain_loop(pair):
+    engine, plain = pair
+    prompts = [[4, 8, 15, 16, 23], [42], list(range(30, 47)), [9, 9, 9], [7] * 11, [200, 100]]
+    limits = [6, 9, 3, 1, 5, 7]
+    requests = [GenerateRequest(p, max_tokens=n, stop_ids=[], **GREEDY) for p, n in zip(prompts, limits)]
+    seen = []
+    results = generate(engine, requests, batch_size=3, on_token=lambda i, t: seen.append((i, t)))
+    for prompt, limit, result in zip(prompts, limits, results):
+        assert result.tokens == P.generate_greedy(plain, prompt, limit, stop_ids=[])
+        assert result.finish_reason == "length" and result.prompt_length == len(prompt)
+    for index, result in enumerate(results):
+        assert [t for i, t in seen if i == index] == result.tokens
+    engine.cache.check()
+    assert engine.cache.slots.n_held == 0 and engine.cache.held_blocks() == 0   # two batches, slots used again
+
+
+def test_stop_tokens_end_a_request_early_and_are_not_returned(pair):
+    engine, plain = pair
+    prompt = [4, 8, 15]
+    free = P.generate_greedy(plain, prompt, 8, stop_ids=[])
+    stop = free[3]
+    other = [50, 60]
+    results = generate(engine, [GenerateRequest(prompt, max_tokens=8, stop_ids=[stop], **GREEDY),
+                                GenerateRequest(other, max_tokens=8, stop_ids=[], **GREEDY)])
+    assert results[0].tokens == free[:free.index(stop)] and results[0].finish_reason == "stop"
+    assert results[1].tokens == P.generate_greedy(plain, other, 8, stop_ids=[])   # the longer one went on alone
+    # the configuration's eos ids are the default stop set
+    default = generate(engine, [GenerateRequest(prompt, max_tokens=8, **GREEDY)])[0]
+    assert default.tokens == P.generate_greedy(plain, prompt, 8)
+
+
+def test_context_and_zero_length_limits(pair):
+    engine, plain = pair
+    context = engine.max_context
+    assert context == 128
+    prompt = list(range(1, context - 1))                             # two tokens fit
+    result = generate(engine, [GenerateRequest(prompt, max_tokens=10, stop_ids=[], **GREEDY)])[0]
+    assert result.finish_reason == "context" and len(result.tokens) == 2
+    assert result.tokens == P.generate_greedy(plain, prompt, 10, stop_ids=[])
+    full = generate(engine, [GenerateRequest(list(range(context)), max_tokens=3, stop_ids=[], **GREEDY)])[0]
+    assert full.tokens == [] and full.finish_reason == "context"
+    none = generate(engine, [GenerateRequest([1, 2], max_tokens=0, **GREEDY)])[0]
+    assert none.tokens == [] and none.finish_reason == "length"
+    empty = generate(engine, [GenerateRequest([], max_tokens=2, stop_ids=[], **GREEDY)])[0]
+    assert empty.prompt_length == 1 and empty.tokens == P.generate_greedy(plain, [], 2, stop_ids=[])
+    with pytest.raises(ValueError, match="exceeds model context length"):
+        generate(engine, [GenerateRequest(list(range(context + 1)), max_tokens=1)])
+    engine.cache.check()
+    assert engine.cache.slots.n_held == 0
+
+
+def test_sampling_is_the_same_alone_and_in_a_batch(pair):
+    engine, _ = pair
+    make = lambda seed, prompt: GenerateRequest(prompt, max_tokens=8, temperature=0.9, top_k=20, top_p=0.9,
+                                                repetition_penalty=1.3, seed=seed, stop_ids=[])
+    together = generate(engine, [make(1, [3, 4, 5]), make(2, [6]), make(1, [3, 4, 5])])
+    alone = generate(engine, [make(1, [3, 4, 5])])[0]
+    assert together[0].tokens == alone.tokens == together[2].tokens
+    assert together[1].tokens != alone.tokens
+    assert generate(engine, [make(9, [3, 4, 5])])[0].tokens != alone.tokens
+
+
+def test_steps_that_cannot_run_are_refused_and_change_nothing(pair):
+    engine, plain = pair
+    slot = engine.alloc_slot()
+    engine.step([(slot, [1, 2, 3], [])])
+    held = engine.cache.held_blocks()
+    for entries, text in [
+        ([], "at least one sequence"),
+        ([(slot, [], [])], "at least one token"),                         # llama.rs:624-626
+        ([(slot, [256], [0])], "exceeds embedding rows"),                 # llama.rs:1044-1049
+        ([(slot, [-1], [0])], "exceeds embedding rows"),
+        ([(slot, [1], [1])], "wanted index"),
+        ([(2, [1], [0])], "not allocated"),
+        ([(slot, [1], [0]), (slot, [2], [0])], "appears twice"),
+        ([(slot, [1] * 126, [0])], "context limit"),
+    ]:
+        with pytest.raises(StepError, match=text):
+            engine.step(entries)
+        assert engine.length(slot) == 3 and engine.cache.held_blocks() == held
+    engine.cache.check()
+    # the refused steps left the sequence intact: its next logits are those of the plain model
+    fresh = engine.alloc_slot()
+    got = engine.step([(fresh, [1, 2, 3, 9], [3])])
+    assert float((got[0] - plain.logits([1, 2, 3, 9])[3]).abs().max()) < 1e-4
+    engine.free_slot(fresh); engine.free_slot(slot)
+    assert engine.cache.held_blocks() == 0
+
+
+def test_a_step_that_the_cache_cannot_hold_takes_nothing(tmp_path):
+    folder = make_folder(TINY["qwen3"], tmp_path / "m", seed=4, std=0.2)
+    engine = Engine.load(folder, dtype="float32", device="cpu", ops=EmulatedOps(), max_tokens=128, max_slots=2)
+    a, b = engine.alloc_slot(), engine.alloc_slot()
+    engine.step([(a, [1, 2, 3], [])])
+    with pytest.raises(StepError, match="cannot hold"):
+        engine.step([(a, [1] * 70, []), (b, [1] * 10, [])])          # 2 + 1 blocks of 2
+    assert engine.cache.held_blocks() == 1 and engine.length(a) == 3 and engine.length(b) == 0
+    engine.cache.check()
+    engine.step([(b, [1] * 10, [])])                                  # what fits still runs
+    assert engine.cache.held_blocks() == 2
+
+
+def test_padding_changes_no_result(pair):
+    from xeno_rt_amd.engine.batch import build_batch
+    engine, plain = pair
+    slot = engine.alloc_slot()
+    ids = [5, 6, 7, 8, 9]
+    engine.cache.reserve(slot, 5); engine.cache.sync()
+    batch = build_batch([slot], [ids], [0], [[4]], "cpu", pad_tokens_to=16)
+    assert batch.n_tokens == 16 and int(batch.slots[5]) == -1
+    logits = engine.model.forward(batch, engine.cache)
+    engine.cache.commit(slot, 5)
+    assert float((logits[0] - plain.logits(ids)[4]).abs().max()) < 1e-4
+    nxt = engine.step([(slot, [11], [0])])
+    assert float((nxt[0] - plain.logits(ids + [11])[5]).abs().max()) < 1e-4
+    engine.free_slot(slot)

@@ -1,0 +1,353 @@
+"""Each HIP kernel alone against its plain reference (the test stand-in, written with
+elementary tensor operations), at sizes other than the engine's: head sizes 16 to 256,
+one to eight query heads per key/value head, widths and vocabularies that are no power
+of two. Inputs are built so that a fault shows: a far key that must win, the edge of a
+window, a block boundary of the cache."""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from ops_emulation import EmulatedOps
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+# elementwise kernels round once: half a unit in the last place of the output type
+ULP = {"float32": 2e-6, "bfloat16": 4e-3}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from xeno_rt_amd.ops import load_ops
+    return load_ops()
+
+
+REF = EmulatedOps()
+
+
+def rand(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def rel(got, want):
+    return float((got.double() - want.double()).abs().max()) / max(1e-30, float(want.double().abs().max()))
+
+
+# ---- embedding, add, rmsnorm -----------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed_and_add(ops, dtype):
+    table = rand(777, 200, dtype=DT[dtype])
+    ids = torch.tensor([0, 776, 5, 5, 123], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 200, device=DEV)
+    ops.embed(table, ids, out)
+    assert torch.equal(out, table[ids.long()].float())
+    delta = rand(5, 200, dtype=DT[dtype], seed=2)
+    want = out + delta.float()
+    ops.add(out, delta)
+    assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [1, 96, 1000, 5120])
+def test_rmsnorm(ops, dtype, hidden):
+    x = rand(7, hidden, seed=hidden, scale=3.0)
+    for weight in (rand(hidden, seed=1) + 1.0, (rand(hidden, seed=1) + 1.0).to(torch.bfloat16)):
+        out = torch.empty(7, hidden, dtype=DT[dtype], device=DEV)
+        ops.rmsnorm(x, weight, 1e-3, out)
+        want = P.rmsnorm(x.double().cpu(), weight.double().cpu(), 1e-3)
+        assert rel(out.cpu(), want) < ULP[dtype]
+        rows = torch.tensor([6, 0, 6], dtype=torch.int32, device=DEV)
+        picked = torch.empty(3, hidden, dtype=DT[dtype], device=DEV)
+        ops.rmsnorm(x, weight, 1e-3, picked, rows=rows)
+        assert torch.equal(picked, out[rows.long()])          # a row's result does not depend on the batch
+
+
+def test_rmsnorm_reference_vector(ops):
+    # tests/kernels_test.rs:75-91 of the reference
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0]], device=DEV)
+    w = torch.tensor([1.0, 1.5, 2.0, 2.5], device=DEV)
+    out = torch.empty(1, 4, device=DEV)
+    ops.rmsnorm(x, w, 1e-5, out)
+    inv = 1.0 / math.sqrt(7.5 + 1e-5)
+    assert rel(out.cpu(), torch.tensor([[inv, 3 * inv, 6 * inv, 10 * inv]])) < 1e-6
+
+
+# ---- matrix products -----------------------------------------------------------------------
+
+SHAPES = [(1, 64, 64), (3, 200, 96), (8, 1000, 176), (17, 96, 192), (64, 333, 520), (130, 257, 72),
+          (300, 520, 1032), (1, 3, 5), (5, 7, 13)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_linear(ops, dtype, m, n, k):
+    a = rand(m, k, dtype=DT[dtype], seed=m)
+    w = rand(n, k, dtype=DT[dtype], seed=n, scale=0.1)
+    want = a.double().cpu() @ w.double().cpu().t()
+    out32 = torch.empty(m, n, device=DEV)
+    ops.linear(a, w, out32)
+    assert rel(out32.cpu(), want) < 1e-5                        # float32 accumulation in both paths
+    out = torch.empty(m, n, dtype=DT[dtype], device=DEV)
+    ops.linear(a, w, out)
+    assert rel(out.cpu(), want) < ULP[dtype] * 2
+    base = rand(m, n, seed=5)
+    acc = base.clone()
+    ops.linear(a, w, acc, accumulate=True)
+    assert rel(acc.cpu(), base.double().cpu() + want) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("m,n,k", [(1, 176, 64), (9, 100, 96), (64, 520, 200), (200, 1000, 72)])
+def test_linear_glu(ops, dtype, m, n, k):
+    a = rand(m, k, dtype=DT[dtype], seed=1)
+    w = rand(2 * n, k, dtype=DT[dtype], seed=2, scale=0.3)
+    both = a.double().cpu() @ w.double().cpu().t()
+    want = P.swiglu(both[:, :n], both[:, n:])
+    out = torch.empty(m, n, dtype=DT[dtype], device=DEV)
+    ops.linear_glu(a, w, out)
+    assert rel(out.cpu(), want) < ULP[dtype] * 2
+
+
+def test_linear_rows_do_not_depend_on_the_batch(ops):
+    a = rand(70, 200, seed=3)
+    w = rand(130, 200, seed=4)
+    whole = torch.empty(70, 130, device=DEV)
+    ops.linear(a, w, whole)
+    for row in (0, 63, 64, 69):
+        one = torch.empty(1, 130, device=DEV)
+        ops.linear(a[row:row + 1].contiguous(), w, one)
+        assert torch.equal(one[0], whole[row])                  # same bits: same order of the sum
+
+
+def test_linear_refuses_what_it_cannot_do(ops):
+    from xeno_rt_amd.ops.hip import KernelError
+    a, w = rand(2, 8), rand(4, 8)
+    with pytest.raises(KernelError, match="columns"):
+        ops.linear(a, rand(4, 16), torch.empty(2, 4, device=DEV))
+    with pytest.raises(KernelError, match="shape"):
+        ops.linear(a, w, torch.empty(2, 5, device=DEV))
+    with pytest.raises(KernelError, match="float32 output"):
+        ops.linear(a, w, torch.empty(2, 4, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(KernelError, match="contiguous"):
+        ops.linear(rand(8, 2).t(), w, torch.empty(2, 4, device=DEV))
+    with pytest.raises(KernelError, match="GPU"):
+        ops.linear(a.cpu(), w, torch.empty(2, 4, device=DEV))
+
+
+# ---- q/k/v preparation and attention ------------------------------------------------------
+
+def make_cache(n_blocks, nkv, hd, dtype, slots, max_blocks):
+    k = torch.zeros(n_blocks, nkv, 64, hd, dtype=dtype, device=DEV)
+    v = torch.zeros(n_blocks, nkv, hd, 64, dtype=dtype, device=DEV)
+    table = torch.full((slots, max_blocks), -1, dtype=torch.int32, device=DEV)
+    return SimpleNamespace(k=k, v=v, block_table=table)
+
+
+def clone_cache(kv):
+    return SimpleNamespace(k=kv.k.clone(), v=kv.v.clone(), block_table=kv.block_table.clone())
+
+
+def i32(values):
+    return torch.tensor(values, dtype=torch.int32, device=DEV)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,rope_dim", [(4, 2, 16, 16), (6, 3, 32, 32), (8, 1, 128, 128),
+                                                (5, 5, 48, 48), (2, 1, 256, 256), (4, 4, 64, 32)])
+def test_qkv_prepare(ops, dtype, nh, nkv, hd, rope_dim):
+    tokens = 9
+    qkv = rand(tokens, (nh + 2 * nkv) * hd, dtype=DT[dtype], seed=hd)
+    positions = i32([0, 1, 63, 64, 65, 127, 128, 500, 1000])
+    slots = i32([0, 0, 0, 0, 1, 1, -1, 1, 0])                  # one token is padding
+    kv = make_cache(40, nkv, hd, DT[dtype], 2, 16)
+    kv.block_table[0, :16] = torch.arange(3, 19, dtype=torch.int32)
+    kv.block_table[1, :16] = torch.arange(39, 23, -1, dtype=torch.int32)
+    theta = (torch.tensor(10000.0) ** (torch.arange(rope_dim // 2) * 2.0 / rope_dim)).to(DEV)
+    qn, kn = rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0
+    for norms in (False, True):
+        got, want = qkv.clone(), qkv.clone()
+        kv_got, kv_want = clone_cache(kv), clone_cache(kv)
+        args = dict(q_norm=qn if norms else None, k_norm=kn if norms else None, norm_eps=1e-4,
+                    rope_theta=theta, rope_dim=rope_dim, rope_scale=1.0)
+        ops.qkv_prepare(got, nh, nkv, hd, positions, slots, kv=kv_got, **args)
+        REF.qkv_prepare(want, nh, nkv, hd, positions, slots, kv=kv_want, **args)
+        # sine and cosine of angles up to 1000 rad differ by float32 rounding of the angle
+        tol = 3e-5 if dtype == "float32" else ULP[dtype]
+        assert rel(got.float(), want.float()) < tol
+        assert rel(kv_got.k.float(), kv_want.k.float()) < tol
+        assert torch.equal(kv_got.v, kv_want.v)
+        assert int((kv_got.k != 0).any(-1).sum()) == 8 * nkv      # eight tokens cached, padding not
+
+
+def test_rope_reference_vector_and_pairing(ops):
+    # tests/kernels_test.rs:94-108: one head of 4, position 2, base 1e4 -> pairs (0,2), (1,3)
+    qkv = torch.zeros(1, 3 * 16, device=DEV)
+    qkv[0, :4] = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    theta = torch.tensor([1.0, 100.0], device=DEV)
+    ops.qkv_prepare(qkv, 1, 1, 16, i32([2]), i32([-1]), rope_theta=theta, rope_dim=4)
+    a0, a1 = 2.0, 0.02
+    want = torch.tensor([1 * math.cos(a0) - 3 * math.sin(a0), 2 * math.cos(a1) - 4 * math.sin(a1),
+                         1 * math.sin(a0) + 3 * math.cos(a0), 2 * math.sin(a1) + 4 * math.cos(a1)])
+    assert rel(qkv[0, :4].cpu(), want) < 1e-6
+    assert float(qkv[0, 4:].abs().max()) == 0.0                   # beyond rope_dim nothing moves
+
+
+def filled_cache(nkv, hd, dtype, lengths, seed=0):
+    """A cache holding `lengths[s]` random tokens for slot s, blocks deliberately out of order."""
+    max_blocks = max((n + 63) // 64 for n in lengths) + 1
+    n_blocks = len(lengths) * max_blocks + 3
+    kv = make_cache(n_blocks, nkv, hd, dtype, len(lengths), max_blocks)
+    order = torch.randperm(n_blocks, generator=torch.Generator().manual_seed(seed)).tolist()
+    keys, values = [], []
+    for s, n in enumerate(lengths):
+        k = rand(n, nkv, hd, dtype=dtype, seed=seed + 10 * s + 1)
+        v = rand(n, nkv, hd, dtype=dtype, seed=seed + 10 * s + 2)
+        keys.append(k); values.append(v)
+        for b in range((n + 63) // 64):
+            block = order.pop()
+            kv.block_table[s, b] = block
+            part = slice(b * 64, min(n, b * 64 + 64))
+            kv.k[block, :, :part.stop - part.start, :] = k[part].transpose(0, 1)
+            kv.v[block, :, :, :part.stop - part.start] = v[part].permute(1, 2, 0)
+    # what lies beyond a sequence's end must never be read: poison it
+    for s, n in enumerate(lengths):
+        if n % 64:
+            block = int(kv.block_table[s, n // 64])
+            kv.k[block, :, n % 64:, :] = float("nan")
+            kv.v[block, :, :, n % 64:] = float("nan")
+    return kv, keys, values
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 16), (6, 3, 32), (8, 1, 128), (5, 5, 48), (2, 2, 256), (32, 8, 128)])
+def test_attention(ops, dtype, nh, nkv, hd):
+    lengths = [200, 65, 1]
+    kv, keys, values = filled_cache(nkv, hd, DT[dtype], lengths, seed=hd)
+    # queries: the last tokens of every sequence (a prompt's end), some in the middle, one padding
+    slots = [0, 0, 0, 0, 1, 1, 2, -1, 0]
+    positions = [199, 198, 64, 0, 64, 63, 0, 0, 127]
+    qkv = rand(len(slots), (nh + 2 * nkv) * hd, dtype=DT[dtype], seed=7)
+    batch = SimpleNamespace(slots=i32(slots), positions=i32(positions))
+    out = torch.full((len(slots), nh * hd), 7.0, dtype=DT[dtype], device=DEV)
+    scale = 1.0 / math.sqrt(hd)
+    ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=scale)
+    for t, (slot, pos) in enumerate(zip(slots, positions)):
+        if slot < 0:
+            assert float(out[t].abs().max()) == 0.0
+            continue
+        q = qkv[t:t + 1, :nh * hd].double().cpu()
+        k = keys[slot][:pos + 1].reshape(pos + 1, nkv * hd).double().cpu()
+        v = values[slot][:pos + 1].reshape(pos + 1, nkv * hd).double().cpu()
+        want = P.causal_attention(q, k, v, nh, nkv, hd, start_position=pos)
+        assert rel(out[t:t + 1].cpu(), want) < (2e-5 if dtype == "float32" else 1e-2), (t, slot, pos)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_finds_a_far_key(ops, dtype):
+    """One key among 900 matches the query: the output must be that key's value, wherever it lies."""
+    nh, nkv, hd = 4, 2, 64
+    kv, keys, values = filled_cache(nkv, hd, DT[dtype], [900], seed=1)
+    for far in (0, 5, 63, 64, 500, 899):
+        qkv = torch.zeros(1, (nh + 2 * nkv) * hd, dtype=DT[dtype], device=DEV)
+        for head in range(nh):
+            qkv[0, head * hd:(head + 1) * hd] = keys[0][far, head // 2] * 40.0
+        batch = SimpleNamespace(slots=i32([0]), positions=i32([899]))
+        out = torch.empty(1, nh * hd, dtype=DT[dtype], device=DEV)
+        ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=1.0 / math.sqrt(hd))
+        for head in range(nh):
+            got = out[0, head * hd:(head + 1) * hd].float()
+            assert rel(got, values[0][far, head // 2].float()) < 2e-2, (far, head)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_window_edge(ops, dtype):
+    """With a window of W a query at P sees keys P-W+1..P: a loud key just outside must be
+    ignored, the same key just inside must win."""
+    nh, nkv, hd, window = 2, 1, 32, 100
+    kv, keys, values = filled_cache(nkv, hd, DT[dtype], [400], seed=2)
+    pos = 399
+    for key_at, inside in ((300, True), (299, False)):
+        qkv = torch.zeros(1, (nh + 2 * nkv) * hd, dtype=DT[dtype], device=DEV)
+        for head in range(nh):
+            qkv[0, head * hd:(head + 1) * hd] = keys[0][key_at, 0] * 40.0
+        batch = SimpleNamespace(slots=i32([0]), positions=i32([pos]))
+        out = torch.empty(1, nh * hd, dtype=DT[dtype], device=DEV)
+        ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=1.0 / math.sqrt(hd), window=window)
+        ref = torch.empty(1, nh * hd, dtype=DT[dtype], device=DEV)
+        REF.attention(qkv, nh, nkv, hd, kv, batch, ref, 1.0 / math.sqrt(hd), window=window)
+        assert rel(out.float(), ref.float()) < (2e-5 if dtype == "float32" else 1e-2)
+        hit = rel(out[0, :hd].float(), values[0][key_at, 0].float()) < 2e-2
+        assert hit == inside
+
+
+# ---- sampling ------------------------------------------------------------------------------
+
+def sample(ops, logits, temperature=0.0, top_k=0, top_p=1.0, penalty=1.0, history=(), draws=None):
+    rows = logits.shape[0]
+    f = lambda v: torch.full((rows,), float(v), device=DEV)
+    offsets = i32([len(history) * r for r in range(rows + 1)])
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    uniforms = torch.tensor(draws if draws is not None else [0.5] * rows, dtype=torch.float32, device=DEV)
+    ops.sample(logits, out, f(temperature), torch.full((rows,), top_k, dtype=torch.int32, device=DEV), f(top_p),
+               f(penalty), i32(list(history) * rows), offsets, uniforms)
+    return out.tolist()
+
+
+def test_sample_reference_cases(ops):
+    # tests/sampler_test.rs:101-127 of the reference
+    assert sample(ops, torch.tensor([[-1.0, 0.5, 3.25, 2.0]], device=DEV), top_k=1, top_p=0.1) == [2]
+    assert sample(ops, torch.tensor([[1.2, 1.5]], device=DEV), penalty=2.0, history=[1]) == [0]
+    assert sample(ops, torch.tensor([[1.2, 1.5]], device=DEV), penalty=1.0, history=[1]) == [1]
+    assert sample(ops, torch.tensor([[1.0, 3.0, 3.0, float("nan")]], device=DEV)) == [1]   # ties: lowest id; NaN never wins
+    # tests/sampler_test.rs:24-98: a draw between p0 and p0+p1 picks token 1 when hot, token 0 when cold
+    e = math.exp
+    logits = torch.tensor([[2.0, 1.0, 0.0]], device=DEV)
+    hot0, hot1 = e(1) / (e(1) + e(0.5) + 1), e(0.5) / (e(1) + e(0.5) + 1)
+    draw = hot0 + hot1 / 2
+    assert sample(ops, logits, temperature=2.0, draws=[draw]) == [1]
+    assert sample(ops, logits, temperature=0.5, draws=[draw]) == [0]
+    logits = torch.tensor([[4.0, 3.0, 2.0, 1.0]], device=DEV)
+    total = e(4) + e(3) + e(2) + e(1)
+    draw = (e(4) + e(3) + e(2) / 2) / total                         # falls on token 2 of the full distribution
+    assert sample(ops, logits, temperature=1.0, draws=[draw]) == [2]
+    assert sample(ops, logits, temperature=1.0, top_k=2, draws=[draw]) == [1]
+    assert sample(ops, logits, temperature=1.0, top_p=0.85, draws=[draw]) == [1]
+
+
+@pytest.mark.parametrize("vocab", [384, 1000, 128256])
+def test_sample_matches_the_plain_distribution(ops, vocab):
+    g = torch.Generator().manual_seed(vocab)
+    row = torch.randn(vocab, generator=g) * 2.0
+    history = [3, 7, 7, vocab - 1]
+    for temperature, top_k, top_p, penalty in [(1.0, 0, 1.0, 1.0), (0.7, 40, 0.95, 1.1), (1.5, 5, 1.0, 2.0),
+                                               (1.0, 0, 0.5, 1.0)]:
+        adjusted = P.apply_repetition_penalty(row, history, penalty)
+        dist = P.sampling_distribution(adjusted, temperature, top_k, top_p) if vocab <= 1000 else None
+        draws = 512
+        logits = row.to(DEV)[None, :].expand(draws, vocab).contiguous()
+        u = ((torch.arange(draws) + 0.5) / draws).tolist()          # an even sweep of the unit interval
+        picks = sample(ops, logits, temperature, top_k, top_p, penalty, history, draws=u)
+        counts = torch.bincount(torch.tensor(picks), minlength=vocab).double() / draws
+        if dist is not None:
+            # an even sweep reproduces every probability to within 1/draws per token
+            assert float((counts - dist).abs().max()) <= 1.5 / draws + 1e-6
+            assert set(torch.nonzero(counts).flatten().tolist()) <= set(torch.nonzero(dist).flatten().tolist())
+        if top_k:
+            kept = set(torch.topk(adjusted, top_k).indices.tolist())
+            assert set(picks) <= kept
+        greedy = sample(ops, logits[:2].contiguous(), 0.0, top_k, top_p, penalty, history)
+        assert greedy == [P.greedy(adjusted)] * 2
+
+
+def test_sample_rows_are_independent(ops):
+    g = torch.Generator().manual_seed(1)
+    logits = (torch.randn(5, 777, generator=g) * 3).to(DEV)
+    u = [0.1, 0.5, 0.9, 0.3, 0.7]
+    together = sample(ops, logits, 0.9, 50, 0.9, 1.0, draws=u)
+    alone = [sample(ops, logits[r:r + 1].contiguous(), 0.9, 50, 0.9, 1.0, draws=[u[r]])[0] for r in range(5)]
+    assert together == alone

@@ -1,0 +1,122 @@
+"""bin/trace_run as a user runs it: the same requests replayed whole, with the last 32
+tokens decoded one by one, and in batches of unequal lengths through reused slots, in
+32-bit and in bfloat16; every logits file is compared with the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, TINY, make_folder
+from helpers import assert_logits, token_ids
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+
+
+def replay(folder, dtype, out, steps, max_tokens):
+    """Run bin/trace_run over `steps`; returns {step: array [wanted, vocab]}."""
+    text = "".join(json.dumps(step) + "\n" for step in steps)
+    done = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", str(max_tokens)],
+                          input=text, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    lines = [line for line in done.stdout.splitlines() if line.startswith("done ")]
+    assert lines == [f"done {step['step']}" for step in steps]
+    vocab = json.load(open(os.path.join(folder, "config.json")))["vocab_size"]
+    result = {}
+    for step in steps:
+        path = os.path.join(str(out), f"{step['step']}.f32")
+        wanted = sum(len(e.get("want", [])) for e in step["entries"])
+        assert os.path.exists(path) == (wanted > 0)
+        if wanted:
+            result[step["step"]] = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(wanted, vocab))
+    return result
+
+
+def trace_whole(requests):
+    return [{"step": i, "entries": [{"id": name, "tokens": ids, "want": list(range(len(ids)))}], "end": [name]}
+            for i, (name, ids) in enumerate(requests.items())]
+
+
+def trace_tail(requests, tail=32):
+    steps = []
+    for name, ids in requests.items():
+        head = max(1, len(ids) - tail)
+        steps.append({"step": len(steps), "entries": [{"id": name, "tokens": ids[:head], "want": list(range(head))}], "end": []})
+        for t in range(head, len(ids)):
+            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": [ids[t]], "want": [0]}],
+                          "end": [name] if t == len(ids) - 1 else []})
+        if head == len(ids):
+            steps[-1]["end"] = [name]
+    return steps
+
+
+def trace_batches(batches, prompt_of):
+    """Each batch starts together with unequal prompts, then one token per live request; a
+    request ends after its last token; the next batch starts when the batch is over."""
+    steps = []
+    for batch in batches:
+        at = {name: prompt_of(name, ids) for name, ids in batch.items()}
+        entries = [{"id": n, "tokens": ids[:at[n]], "want": list(range(at[n]))} for n, ids in batch.items()]
+        steps.append({"step": len(steps), "entries": entries, "end": [n for n, ids in batch.items() if at[n] == len(ids)]})
+        while any(at[n] < len(ids) for n, ids in batch.items()):
+            live = [n for n, ids in batch.items() if at[n] < len(ids)]
+            entries = [{"id": n, "tokens": [batch[n][at[n]]], "want": [0]} for n in live]
+            for n in live:
+                at[n] += 1
+            steps.append({"step": len(steps), "entries": entries, "end": [n for n in live if at[n] == len(batch[n])]})
+    return steps
+
+
+def collect(steps, outputs):
+    """{request: logits [len, vocab]} from the files of a replay."""
+    rows = {}
+    for step in steps:
+        if step["step"] not in outputs:
+            continue
+        at = 0
+        for entry in step["entries"]:
+            n = len(entry["want"])
+            rows.setdefault(entry["id"], []).append(outputs[step["step"]][at:at + n])
+            at += n
+    return {name: torch.cat(parts) for name, parts in rows.items()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["llama", "qwen3"])
+def test_replay_schedules(name, dtype, tmp_path):
+    folder = make_folder(TINY[name], tmp_path / "model", seed=13, std=0.2)
+    plain = P.PlainModel(folder)
+    vocab = plain.config.vocab_size
+    lengths = {"a": 40, "b": 7, "c": 100, "d": 65, "e": 1, "f": 90}
+    requests = {n: token_ids(vocab, length, seed=length) for n, length in lengths.items()}
+    want = {n: plain.logits(ids) for n, ids in requests.items()}
+
+    whole = trace_whole(requests)
+    got_whole = collect(whole, replay(folder, dtype, tmp_path / "whole", whole, 128))
+    tail = trace_tail(requests)
+    got_tail = collect(tail, replay(folder, dtype, tmp_path / "tail", tail, 128))
+    names = list(requests)
+    batches = [{n: requests[n] for n in names[:3]}, {n: requests[n] for n in names[3:]}]
+    batched = trace_batches(batches, lambda n, ids: max(1, len(ids) - 5 - ord(n) % 3))
+    # 64 + 64 + 128 tokens are held by the first batch at its fullest
+    got_batched = collect(batched, replay(folder, dtype, tmp_path / "batched", batched, 256))
+    for n in names:
+        assert_logits(got_whole[n], want[n], dtype, f"{name} whole {n}")
+        assert_logits(got_tail[n], want[n], dtype, f"{name} tail {n}")
+        assert_logits(got_batched[n], want[n], dtype, f"{name} batched {n}")
+        if dtype == "float32":
+            assert torch.equal(got_whole[n], got_tail[n]) and torch.equal(got_whole[n], got_batched[n])
+
+
+def test_replay_without_wanted_logits_writes_no_file(tmp_path):
+    folder = make_folder(TINY["llama"], tmp_path / "model", seed=1)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": [1, 2, 3], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": [4], "want": [0]}], "end": ["x"]}]
+    out = replay(folder, "float32", tmp_path / "out", steps, 64)
+    assert list(out) == [1]
+    assert_logits(out[1], P.PlainModel(folder).logits([1, 2, 3, 4])[3:], "float32")

@@ -7,6 +7,7 @@ giving something back twice, is an error and never silent.
 """
 from __future__ import annotations
 
+import heapq
 from typing import List
 
 BLOCK_TOKENS = 64   # tokens per block: the unit in which live requests hold cache
@@ -21,14 +22,14 @@ class CacheError(RuntimeError):
 
 
 class Pool:
-    """`size` numbered items, handed out lowest-first and reused after release."""
+    """`size` numbered items; the lowest free one is handed out, released ones are used again."""
 
     def __init__(self, size: int, what: str):
         if size < 0:
             raise ValueError(f"pool of {what}s needs a non-negative size")
         self.size = size
         self.what = what
-        self._free: List[int] = list(range(size - 1, -1, -1))   # a stack; pop() gives the lowest
+        self._free: List[int] = list(range(size))               # a heap: the lowest number on top
         self._held = [False] * size
 
     @property
@@ -45,7 +46,7 @@ class Pool:
     def acquire(self) -> int:
         if not self._free:
             raise CacheFull(f"no free {self.what} (all {self.size} are in use)")
-        item = self._free.pop()
+        item = heapq.heappop(self._free)
         if self._held[item]:
             raise CacheError(f"{self.what} {item} was on the free list while held")
         self._held[item] = True
@@ -57,7 +58,7 @@ class Pool:
         if not self._held[item]:
             raise CacheError(f"{self.what} {item} is released twice or was never acquired")
         self._held[item] = False
-        self._free.append(item)
+        heapq.heappush(self._free, item)
 
     def check(self) -> None:
         """Every item is either free once or held; raises CacheError otherwise."""
