@@ -80,7 +80,8 @@ def test_rmsnorm_reference_vector(ops):
 # ---- matrix products -----------------------------------------------------------------------
 
 SHAPES = [(1, 64, 64), (3, 200, 96), (8, 1000, 176), (17, 96, 192), (64, 333, 520), (130, 257, 72),
-          (300, 520, 1032), (1, 3, 5), (5, 7, 13)]
+          (300, 520, 1032), (1, 3, 5), (5, 7, 13), (33, 4100, 264), (64, 40, 4096), (65, 40, 4096),
+          (2048, 6144, 128), (2000, 6200, 136)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -102,7 +103,8 @@ def test_linear(ops, dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("m,n,k", [(1, 176, 64), (9, 100, 96), (64, 520, 200), (200, 1000, 72)])
+@pytest.mark.parametrize("m,n,k", [(1, 176, 64), (9, 100, 96), (64, 520, 200), (200, 1000, 72), (48, 2000, 520),
+                                   (2048, 3100, 64), (300, 130, 1032)])
 def test_linear_glu(ops, dtype, m, n, k):
     a = rand(m, k, dtype=DT[dtype], seed=1)
     w = rand(2 * n, k, dtype=DT[dtype], seed=2, scale=0.3)
@@ -283,6 +285,84 @@ def test_attention_window_edge(ops, dtype):
         assert rel(out.float(), ref.float()) < (2e-5 if dtype == "float32" else 1e-2)
         hit = rel(out[0, :hd].float(), values[0][key_at, 0].float()) < 2e-2
         assert hit == inside
+
+
+def described(slots, counts, starts):
+    """A batch namespace with the per-sequence arrays, as the engine builds it."""
+    token_slots, positions, offsets = [], [], [0]
+    for slot, count, start in zip(slots, counts, starts):
+        token_slots += [slot] * count
+        positions += list(range(start, start + count))
+        offsets.append(offsets[-1] + count)
+    return SimpleNamespace(slots=i32(token_slots), positions=i32(positions), sequence_offsets=i32(offsets),
+                           sequence_slots=i32(slots), sequence_starts=i32(starts), n_sequences=len(slots),
+                           max_count=max(counts), max_context=max(s + c for s, c in zip(starts, counts)))
+
+
+def expected_attention(qkv, batch_slots, batch_positions, keys, values, nh, nkv, hd):
+    rows = []
+    for t, (slot, pos) in enumerate(zip(batch_slots, batch_positions)):
+        q = qkv[t:t + 1, :nh * hd].double().cpu()
+        k = keys[slot][:pos + 1].reshape(pos + 1, nkv * hd).double().cpu()
+        v = values[slot][:pos + 1].reshape(pos + 1, nkv * hd).double().cpu()
+        rows.append(P.causal_attention(q, k, v, nh, nkv, hd, start_position=pos))
+    return torch.cat(rows)
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 4, 64), (8, 2, 128), (32, 8, 128), (16, 1, 64), (40, 2, 128)])
+def test_attention_decode_on_matrix_cores(ops, nh, nkv, hd):
+    """One token per sequence (the decode kernels): lengths at block edges, one sequence far longer
+    than the others, groups of 1 to 20 query heads per key/value head."""
+    lengths = [1, 64, 65, 700, 128, 2]
+    kv, keys, values = filled_cache(nkv, hd, torch.bfloat16, lengths, seed=hd + nh)
+    slots = list(range(len(lengths)))
+    batch = described(slots, [1] * len(lengths), [n - 1 for n in lengths])
+    qkv = rand(len(lengths), (nh + 2 * nkv) * hd, dtype=torch.bfloat16, seed=3)
+    out = torch.full((len(lengths), nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=1.0 / math.sqrt(hd))
+    want = expected_attention(qkv, slots, [n - 1 for n in lengths], keys, values, nh, nkv, hd)
+    assert torch.isfinite(out).all()
+    assert rel(out.cpu(), want) < 1e-2
+    # a padded batch: the extra token has no slot and gets zeros, the others do not change
+    padded = SimpleNamespace(**vars(batch))
+    padded.slots, padded.positions = i32(slots + [-1]), i32([n - 1 for n in lengths] + [0])
+    out2 = torch.full((len(lengths) + 1, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention(torch.cat([qkv, qkv[:1]]), nh, nkv, hd, kv, padded, out2, scale=1.0 / math.sqrt(hd))
+    assert torch.equal(out2[:-1], out) and float(out2[-1].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 4, 64), (8, 2, 128), (32, 8, 128), (6, 3, 64)])
+def test_attention_prefill_on_matrix_cores(ops, nh, nkv, hd):
+    """Whole prompts of unequal lengths in one step, and a prompt that continues a cache."""
+    lengths = [200, 65, 1, 33, 500]
+    starts = [0, 0, 0, 20, 436]                               # the last two continue what the cache holds
+    kv, keys, values = filled_cache(nkv, hd, torch.bfloat16, lengths, seed=hd + nh)
+    slots = list(range(len(lengths)))
+    counts = [n - s for n, s in zip(lengths, starts)]
+    batch = described(slots, counts, starts)
+    tokens = sum(counts)
+    qkv = rand(tokens, (nh + 2 * nkv) * hd, dtype=torch.bfloat16, seed=5)
+    out = torch.full((tokens, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=1.0 / math.sqrt(hd))
+    want = expected_attention(qkv, batch.slots.tolist(), batch.positions.tolist(), keys, values, nh, nkv, hd)
+    assert torch.isfinite(out).all()
+    assert rel(out.cpu(), want) < 1e-2
+
+
+def test_matrix_core_attention_finds_a_far_key(ops):
+    nh, nkv, hd = 8, 2, 128
+    kv, keys, values = filled_cache(nkv, hd, torch.bfloat16, [900], seed=1)
+    for far in (0, 5, 63, 64, 500, 899):
+        q_row = torch.zeros((nh + 2 * nkv) * hd, dtype=torch.bfloat16, device=DEV)
+        for head in range(nh):
+            q_row[head * hd:(head + 1) * hd] = keys[0][far, head // 4] * 40.0
+        for batch, rows in ((described([0], [1], [899]), 1), (described([0], [40], [860]), 40)):
+            qkv = q_row[None, :].repeat(rows, 1).contiguous()
+            out = torch.empty(rows, nh * hd, dtype=torch.bfloat16, device=DEV)
+            ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=1.0 / math.sqrt(hd))
+            for head in range(nh):
+                got = out[-1, head * hd:(head + 1) * hd].float()
+                assert rel(got, values[0][far, head // 4].float()) < 2e-2, (far, head, rows)
 
 
 # ---- sampling ------------------------------------------------------------------------------

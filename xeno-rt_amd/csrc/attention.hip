@@ -1,4 +1,7 @@
 // Entry point of attention: checks the operands and picks the kernel.
+//   bfloat16, head size 64 or 128, no window: the matrix-core kernels: decode (every sequence
+//   brings one token) or prefill (any token counts);
+//   everything else (float32, other head sizes, windows): the general kernel.
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -6,11 +9,23 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
                           int window, hipStream_t s);
+bool xrt_attention_decode_accepts(int head_dim);
+int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
+                         const void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                         const int* positions, const int* slots, void* out, float scale, int max_context,
+                         float* workspace, long workspace_floats, hipStream_t s);
+bool xrt_attention_prefill_accepts(int head_dim);
+int xrt_attention_prefill(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
+                          const void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                          const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
+                          float scale, hipStream_t s);
 
 extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                              const void* k_cache, const void* v_cache, const int* block_table,
                              int table_stride, int n_blocks, const int* positions, const int* slots, void* out,
-                             float scale, int window, void* stream) {
+                             float scale, int window, const int* seq_offsets, const int* seq_slots,
+                             const int* seq_starts, int n_seqs, int max_count, int max_context,
+                             float* workspace, long workspace_floats, void* stream) {
     XRT_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention: head counts %d/%d: the first must be a multiple of the second", n_heads, n_kv_heads);
     XRT_REQUIRE(head_dim > 0 && head_dim % 16 == 0, "attention: head_dim %d must be a multiple of 16", head_dim);
@@ -19,6 +34,22 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
     XRT_REQUIRE(table_stride > 0 && n_blocks > 0, "attention: empty cache");
     XRT_REQUIRE(window >= 0, "attention: negative window");
     if (tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const bool described = seq_offsets && seq_slots && seq_starts && n_seqs > 0 && max_count > 0 && max_context > 0;
+    if (dtype == XRT_BF16 && window == 0 && described) {
+        if (max_count == 1 && workspace != nullptr && xrt_attention_decode_accepts(head_dim))
+            return xrt_attention_decode(qkv, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
+                                        table_stride, n_blocks, positions, slots, out, scale, max_context, workspace,
+                                        workspace_floats, s);
+        if (max_count > 1 && xrt_attention_prefill_accepts(head_dim)) {
+            // tokens beyond the sequences (padding) get zeros
+            // (their rows are read by nothing, but must not hold what a later product could choke on)
+            XRT_REQUIRE(n_seqs <= tokens, "attention: more sequences than tokens");
+            return xrt_attention_prefill(qkv, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
+                                         table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, out,
+                                         scale, s);
+        }
+    }
     return xrt_attention_generic(qkv, dtype, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
-                                 table_stride, n_blocks, positions, slots, out, scale, window, (hipStream_t)stream);
+                                 table_stride, n_blocks, positions, slots, out, scale, window, s);
 }

@@ -1,0 +1,227 @@
+// Decode attention on the matrix cores: every sequence brings one query token; its keys and
+// values are read once from the cache, in chunks spread over many wavefronts, and applied to
+// all query heads of a key/value head together.
+//
+// Formulas: crates/xrt-models/src/llama.rs:504-574 of the reference (score = q.k * scale over
+// keys 0..pos, online softmax with running maximum and sum, weighted sum of values, division
+// by the sum); query head h uses key/value head h / group.
+//
+// One wavefront takes one chunk of keys of one (token, key/value head, tile of 16 query
+// heads). Scores: S[key][head] = K Q^T with v_mfma_f32_16x16x32_bf16, keys as rows (A operand,
+// read straight from the cache block, 16 bytes per lane), the query heads as columns. Values:
+// O[dim][head] += V^T P, with the transposed value block as A operand (again 16 contiguous
+// bytes per lane) and the probabilities, still in the registers the scores came in, as B
+// operand: key rows are assigned to accumulator rows such that every lane ends up holding
+// eight consecutive keys, exactly the K slots of the next product. Each wavefront leaves an
+// unnormalised partial result (maximum, sum, O); a second kernel merges the chunks of a token
+// in chunk order.
+#include "common.h"
+#include "xrt_hip.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVES = 4;
+constexpr float LOG2E = 1.4426950408889634f;
+
+// key (0..31 within a group of 32) that row r of score tile `tile` (0 or 1) stands for:
+// accumulator register i of lane group c is row c*4 + i, and must be key c*8 + tile*4 + i
+__device__ __forceinline__ int key_of_row(int tile, int r) { return (r / 4) * 8 + tile * 4 + (r % 4); }
+
+template <int HD>
+__global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
+    const bf16* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads,
+    const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
+    int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
+    float scale, int chunk_blocks, int n_chunks, int q_tiles,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    constexpr int KS = HD / 32;                    // K steps of the score product
+    constexpr int DT = HD / 16;                    // 16-row tiles of the value product
+    const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
+    const int r = lane % 16, c = lane / 16;
+    const int chunk = blockIdx.x * WAVES + wave;
+    const int kv_head = blockIdx.y / q_tiles, q_tile = blockIdx.y % q_tiles;
+    const int token = blockIdx.z;
+    const int slot = slots[token];
+    if (slot < 0 || chunk >= n_chunks) return;
+    const int n_keys = positions[token] + 1;
+    const int first_block = chunk * chunk_blocks;
+    if (first_block * XRT_BLOCK_TOKENS >= n_keys) return;
+    const int last_block = min((n_keys - 1) / XRT_BLOCK_TOKENS, first_block + chunk_blocks - 1);
+    const int group = n_heads / n_kv_heads;
+    const int head_in_group = q_tile * 16 + r;             // this lane's query head (column of the products)
+    const bool head_valid = head_in_group < group;
+    const int head = kv_head * group + head_in_group;
+
+    bf16x8 q[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+        q[ks] = head_valid ? *reinterpret_cast<const bf16x8*>(qkv + (long)token * row_width + (long)head * HD + ks * 32 + c * 8)
+                           : bf16x8{};
+
+    const float scale2 = scale * LOG2E;                    // scores are kept in units of log2
+    float m = -INFINITY, l = 0.f;
+    floatx4 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    for (int b = first_block; b <= last_block; ++b) {
+        const int block = block_table[(long)slot * table_stride + b];
+        if (block < 0 || block >= n_blocks) continue;      // the host never lets this happen
+        const bf16* kb = k_cache + ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * HD;
+        const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * XRT_BLOCK_TOKENS;
+        const int valid = min(XRT_BLOCK_TOKENS, n_keys - b * XRT_BLOCK_TOKENS);   // keys of this block that exist
+
+        // ---- scores of 64 keys: two groups of 32, two tiles of 16 rows each
+        floatx4 s[2][2];
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                s[g][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+                const bf16* key = kb + (long)(g * 32 + key_of_row(t, r)) * HD + c * 8;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    s[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(key + ks * 32), q[ks], s[g][t], 0, 0, 0);
+            }
+        // register i of s[g][t] is key g*32 + c*8 + t*4 + i, for query head r
+        float block_max = -INFINITY;
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = g * 32 + c * 8 + t * 4 + i;
+                    const float v = key < valid ? s[g][t][i] * scale2 : -INFINITY;   // also drops whatever lies past the end
+                    s[g][t][i] = v;
+                    block_max = fmaxf(block_max, v);
+                }
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 16, XRT_WAVE));
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 32, XRT_WAVE));
+        const float m_new = fmaxf(m, block_max);           // finite: key 0 of the block exists
+        const float correction = __builtin_amdgcn_exp2f(m - m_new);
+        m = m_new;
+        l *= correction;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[dt] *= correction;
+
+        // ---- probabilities, and the value product
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            bf16x8 p;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float e = __builtin_amdgcn_exp2f(s[g][t][i] - m_new);
+                    l += e;
+                    p[t * 4 + i] = (bf16)e;
+                }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                bf16x8 v = *reinterpret_cast<const bf16x8*>(vb + (long)(dt * 16 + r) * XRT_BLOCK_TOKENS + g * 32 + c * 8);
+                if (valid < XRT_BLOCK_TOKENS) {
+                    // the block's tail belongs to nobody: whatever it holds must not meet the zeros of p
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (g * 32 + c * 8 + e >= valid) v[e] = (bf16)0.f;
+                }
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p, o[dt], 0, 0, 0);
+            }
+        }
+    }
+    l += __shfl_xor(l, 16, XRT_WAVE);
+    l += __shfl_xor(l, 32, XRT_WAVE);
+
+    if (head_valid) {
+        const long slot_index = ((long)token * n_heads + head) * n_chunks + chunk;
+        float* dst = part_o + slot_index * HD;
+        // accumulator register i of tile dt is dimension dt*16 + c*4 + i, for query head r
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<floatx4*>(dst + dt * 16 + c * 4) = o[dt];
+        if (c == 0) {
+            part_ml[slot_index * 2] = m;
+            part_ml[slot_index * 2 + 1] = l;
+        }
+    }
+}
+
+template <int HD>
+__global__ void __launch_bounds__(HD) attention_decode_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
+    const int* __restrict__ slots, int n_heads, int chunk_blocks, int n_chunks, bf16* __restrict__ out) {
+    const int token = blockIdx.y, head = blockIdx.x, d = threadIdx.x;
+    bf16* dst = out + ((long)token * n_heads + head) * HD;
+    if (slots[token] < 0) {
+        dst[d] = (bf16)0.f;
+        return;
+    }
+    const int n_keys = positions[token] + 1;
+    const int chunk_keys = chunk_blocks * XRT_BLOCK_TOKENS;
+    const int chunks = min(n_chunks, (n_keys + chunk_keys - 1) / chunk_keys);
+    const long base = ((long)token * n_heads + head) * n_chunks;
+    float m = -INFINITY;
+    for (int k = 0; k < chunks; ++k) m = fmaxf(m, part_ml[(base + k) * 2]);
+    float l = 0.f, acc = 0.f;
+    for (int k = 0; k < chunks; ++k) {
+        const float w = __builtin_amdgcn_exp2f(part_ml[(base + k) * 2] - m);
+        l += w * part_ml[(base + k) * 2 + 1];
+        acc += w * part_o[(base + k) * HD + d];
+    }
+    dst[d] = (bf16)(l > 0.f ? acc / l : 0.f);
+}
+
+template <int HD>
+int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
+           const int* block_table, int table_stride, int n_blocks, const int* positions, const int* slots, bf16* out,
+           float scale, int max_context, float* workspace, long workspace_floats, hipStream_t s) {
+    const int group = n_heads / n_kv_heads;
+    const int q_tiles = (group + 15) / 16;
+    const int max_blocks = (max_context + XRT_BLOCK_TOKENS - 1) / XRT_BLOCK_TOKENS;
+    // enough wavefronts to fill the chip, but chunks as long as that allows
+    long chunk_blocks = ((long)tokens * n_kv_heads * q_tiles * max_blocks) / 4096;
+    chunk_blocks = chunk_blocks < 1 ? 1 : (chunk_blocks > 16 ? 16 : chunk_blocks);
+    const int n_chunks = (int)((max_blocks + chunk_blocks - 1) / chunk_blocks);
+    const long need = (long)tokens * n_heads * n_chunks * (HD + 2);
+    XRT_REQUIRE(workspace != nullptr && workspace_floats >= need,
+                "attention (decode): workspace of %ld floats given, %ld needed", workspace_floats, need);
+    float* part_o = workspace;
+    float* part_ml = workspace + (long)tokens * n_heads * n_chunks * HD;
+    const int row_width = (n_heads + 2 * n_kv_heads) * HD;
+    XRT_REQUIRE(tokens <= 65535 && n_kv_heads * q_tiles <= 65535, "attention (decode): grid too large");
+    const dim3 grid((n_chunks + WAVES - 1) / WAVES, n_kv_heads * q_tiles, tokens);
+    attention_decode_kernel<HD><<<grid, WAVES * XRT_WAVE, 0, s>>>(
+        qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, positions, slots,
+        scale, (int)chunk_blocks, n_chunks, q_tiles, part_o, part_ml);
+    XRT_LAUNCH_CHECK("attention (decode)");
+    attention_decode_merge_kernel<HD><<<dim3(n_heads, tokens), HD, 0, s>>>(
+        part_o, part_ml, positions, slots, n_heads, (int)chunk_blocks, n_chunks, out);
+    XRT_LAUNCH_CHECK("attention (decode merge)");
+    return 0;
+}
+
+}  // namespace
+
+bool xrt_attention_decode_accepts(int head_dim) { return head_dim == 64 || head_dim == 128; }
+
+// floats of workspace that a decode step of `tokens` sequences may need
+long xrt_attention_decode_workspace(int tokens, int n_heads, int n_kv_heads, int head_dim, int max_context) {
+    const int max_blocks = (max_context + XRT_BLOCK_TOKENS - 1) / XRT_BLOCK_TOKENS;
+    return (long)tokens * n_heads * max_blocks * (head_dim + 2);     // chunks of one block: the most there can be
+}
+
+int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
+                         const void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                         const int* positions, const int* slots, void* out, float scale, int max_context,
+                         float* workspace, long workspace_floats, hipStream_t s) {
+    if (head_dim == 64)
+        return launch<64>((const bf16*)qkv, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache,
+                          block_table, table_stride, n_blocks, positions, slots, (bf16*)out, scale, max_context,
+                          workspace, workspace_floats, s);
+    return launch<128>((const bf16*)qkv, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache,
+                       block_table, table_stride, n_blocks, positions, slots, (bf16*)out, scale, max_context,
+                       workspace, workspace_floats, s);
+}

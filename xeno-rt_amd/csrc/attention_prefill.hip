@@ -1,0 +1,187 @@
+// Prefill attention on the matrix cores: causal attention of the new tokens of every sequence
+// of a step over that sequence's cache (which already holds the new keys and values), without
+// ever forming the score matrix in memory.
+//
+// Formulas: crates/xrt-models/src/llama.rs:727-770 of the reference (the token at position P
+// sees keys 0..P; score = q.k * scale; softmax; weighted sum of values; query head h uses
+// key/value head h / group), computed with the running maximum and sum of its decode loop
+// (:514-574) instead of a stored row of scores.
+//
+// A wavefront owns 32 consecutive query tokens of one sequence and one head; the four
+// wavefronts of a workgroup take four neighbouring heads, which mostly share a key/value head
+// and so hit the same cache lines. Everything is kept transposed so that one lane owns one
+// query: S^T[key][query] = K Q^T and O^T[dim][query] += V^T P^T with
+// v_mfma_f32_32x32x16_bf16. Maximum, sum and rescaling of a query are then private to a lane
+// (plus its partner 32 lanes away), and the probabilities are already in the registers, and
+// the order, that the second product wants as its B operand: key rows are assigned to
+// accumulator rows such that a lane holds eight consecutive keys per K step, which are also
+// 16 contiguous bytes of the transposed value block.
+#include "common.h"
+#include "xrt_hip.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int WAVES = 4;
+constexpr int QT = 32;                 // query tokens per wavefront
+constexpr float LOG2E = 1.4426950408889634f;
+
+// Key (0..31 within a tile of 32 keys) that row r of the score tile stands for. Accumulator
+// register i of lane half h is row (i/4)*8 + h*4 + i%4 and must be key (i/8)*16 + h*8 + i%8.
+__device__ __forceinline__ int key_of_row(int r) { return (r / 16) * 16 + ((r % 8) / 4) * 8 + ((r / 8) % 2) * 4 + r % 4; }
+
+template <int HD>
+__global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
+    const bf16* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads,
+    const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
+    int table_stride, int n_blocks, const int* __restrict__ seq_offsets, const int* __restrict__ seq_slots,
+    const int* __restrict__ seq_starts, int n_seqs, bf16* __restrict__ out, float scale) {
+    constexpr int KS = HD / 16;            // K steps of the score product
+    constexpr int DT = HD / 32;            // 32-row tiles of the value product
+    const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
+    const int col = lane % 32, half = lane / 32;
+    const int head = blockIdx.y * WAVES + wave;
+    if (head >= n_heads) return;
+
+    // which sequence and which of its query tiles this workgroup has
+    int tile = blockIdx.x, seq = 0, count = 0;
+    for (; seq < n_seqs; ++seq) {
+        count = seq_offsets[seq + 1] - seq_offsets[seq];
+        const int tiles = (count + QT - 1) / QT;
+        if (tile < tiles) break;
+        tile -= tiles;
+    }
+    if (seq >= n_seqs) return;
+    const int slot = seq_slots[seq];
+    const int start = seq_starts[seq];                       // tokens in the cache before this step
+    const int q_first = tile * QT;                           // index among the sequence's new tokens
+    const int q_count = min(QT, count - q_first);
+    const bool q_valid = col < q_count;
+    const long token = (long)seq_offsets[seq] + q_first + col;   // row of qkv and out (if valid)
+    const int q_pos = start + q_first + col;                 // absolute position of this lane's query
+    const int last_key = start + q_first + q_count - 1;      // the furthest key any query of the tile sees
+    const int kv_head = head / (n_heads / n_kv_heads);
+
+    bf16x8 q[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+        q[ks] = q_valid ? *reinterpret_cast<const bf16x8*>(qkv + token * row_width + (long)head * HD + ks * 16 + half * 8)
+                        : bf16x8{};
+
+    const float scale2 = scale * LOG2E;
+    float m = -INFINITY, l = 0.f;
+    floatx16 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
+
+    const int row_key = key_of_row(col);                     // the key this lane's A-operand row stands for
+    const int first_masked = start + q_first;                // tiles whose keys all lie at or before this need no mask
+
+    for (int k0 = 0; k0 <= last_key; k0 += 32) {
+        const int block = block_table[(long)slot * table_stride + k0 / XRT_BLOCK_TOKENS];
+        if (block < 0 || block >= n_blocks) continue;        // the host never lets this happen
+        const int in_block = k0 % XRT_BLOCK_TOKENS;
+        const bf16* kb = k_cache + (((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS + in_block + row_key) * HD + half * 8;
+        const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * XRT_BLOCK_TOKENS + in_block + half * 8;
+
+        floatx16 s;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kb + ks * 16), q[ks], s, 0, 0, 0);
+
+        // register i is key k0 + (i/8)*16 + half*8 + i%8, for this lane's query
+        const bool edge = k0 + 31 > first_masked;            // some key of the tile may lie beyond some query
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int key = k0 + (i / 8) * 16 + half * 8 + i % 8;
+            float v = s[i] * scale2;
+            if (edge && key > q_pos) v = -INFINITY;           // causal: keys after the query do not exist for it
+            s[i] = v;
+            tile_max = fmaxf(tile_max, v);
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, XRT_WAVE));
+        const float m_new = fmaxf(m, tile_max);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // a query that sees none of these keys yet
+        const float correction = __builtin_amdgcn_exp2f(m - m_safe);
+        m = m_new;
+        l *= correction;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[dt][e] *= correction;
+
+        bf16x8 p[2];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float e = __builtin_amdgcn_exp2f(s[i] - m_safe);
+            l += e;
+            p[i / 8][i % 8] = (bf16)e;
+        }
+#pragma unroll
+        for (int step = 0; step < 2; ++step)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                bf16x8 v = *reinterpret_cast<const bf16x8*>(vb + (long)(dt * 32 + col) * XRT_BLOCK_TOKENS + step * 16);
+                if (edge) {
+                    // beyond the sequence's last key the block holds nothing of ours: keep it away from the zeros of p
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (k0 + step * 16 + half * 8 + e > last_key) v[e] = (bf16)0.f;
+                }
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v, p[step], o[dt], 0, 0, 0);
+            }
+    }
+    l += __shfl_xor(l, 32, XRT_WAVE);
+
+    if (q_valid) {
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        bf16* dst = out + (token * n_heads + head) * HD;
+        // accumulator register i of tile dt is dimension dt*32 + (i/4)*8 + half*4 + i%4, for this lane's query
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                struct alignas(8) Four { bf16 e[4]; } four;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) four.e[i] = (bf16)(o[dt][g * 4 + i] * inv);
+                *reinterpret_cast<Four*>(dst + dt * 32 + g * 8 + half * 4) = four;
+            }
+    }
+}
+
+template <int HD>
+int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
+           const int* block_table, int table_stride, int n_blocks, const int* seq_offsets, const int* seq_slots,
+           const int* seq_starts, int n_seqs, bf16* out, float scale, hipStream_t s) {
+    const int row_width = (n_heads + 2 * n_kv_heads) * HD;
+    // every sequence has at most ceil(count/32) tiles; their sum is at most tokens/32 + n_seqs
+    const long tiles = (tokens + QT - 1) / QT + n_seqs;
+    const dim3 grid((unsigned)tiles, (n_heads + WAVES - 1) / WAVES);
+    attention_prefill_kernel<HD><<<grid, WAVES * XRT_WAVE, 0, s>>>(
+        qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, seq_offsets,
+        seq_slots, seq_starts, n_seqs, out, scale);
+    XRT_LAUNCH_CHECK("attention (prefill)");
+    return 0;
+}
+
+}  // namespace
+
+bool xrt_attention_prefill_accepts(int head_dim) { return head_dim == 64 || head_dim == 128; }
+
+int xrt_attention_prefill(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
+                          const void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                          const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
+                          float scale, hipStream_t s) {
+    if (head_dim == 64)
+        return launch<64>((const bf16*)qkv, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache,
+                          block_table, table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, (bf16*)out, scale, s);
+    return launch<128>((const bf16*)qkv, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache,
+                       block_table, table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, (bf16*)out, scale, s);
+}

@@ -1,0 +1,239 @@
+// Matrix product for many rows (prefill), bfloat16 operands, float32 accumulation on the
+// matrix cores: out[m, n] = sum_k a[m, k] * w[n, k]; both operands are contiguous along k.
+//
+// A workgroup computes a BM x BN tile of the output with v_mfma_f32_32x32x16_bf16. Tiles of
+// a and w, 64 wide in k, are staged through LDS: while the matrix cores work on one buffer,
+// the next tile travels global -> registers -> the other buffer (one barrier per step). LDS
+// rows are padded by 16 bytes so that the 16-byte operand reads of 16 consecutive rows fall
+// into different banks. Each wavefront owns a (BM/WM) x (BN/WN) part of the tile and keeps
+// its accumulators in registers for the whole K loop.
+//
+// Workgroup ids are remapped so that the workgroups that run on one XCD (ids are dealt
+// round-robin to the 8 XCDs) work on neighbouring tiles and share their operands in that
+// XCD's L2.
+//
+// Epilogues: store (bfloat16 or float32), accumulate into float32, or the gated pair
+// silu(gate) * up: then the w tile holds BN/2 gate rows and the BN/2 up rows that belong to
+// them (rows n and n + N of w), and the two halves meet through LDS after the K loop.
+#include "common.h"
+#include "xrt_hip.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 64;
+constexpr int PITCH = BK + 8;          // bf16 elements per LDS row
+enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
+
+__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
+
+template <int BM, int BN, int WM, int WN, int MODE, typename TO>
+__global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
+    const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
+    int tiles_m, int tiles_n) {
+    constexpr int THREADS = WM * WN * XRT_WAVE;
+    constexpr int WAVE_M = BM / WM, WAVE_N = BN / WN;        // part of the tile owned by one wavefront
+    constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;        // 32x32 accumulator tiles of a wavefront
+    constexpr int CHUNKS_A = BM * BK / 8 / THREADS;          // 16-byte chunks each thread moves per step
+    constexpr int CHUNKS_B = BN * BK / 8 / THREADS;
+    static_assert(BM * BK / 8 % THREADS == 0 && BN * BK / 8 % THREADS == 0, "tile does not divide among the threads");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    bf16* lds_a = reinterpret_cast<bf16*>(lds_raw);                    // [2][BM][PITCH]
+    bf16* lds_b = lds_a + 2 * BM * PITCH;                              // [2][BN][PITCH]
+
+    // ---- which tile: ids are dealt to XCDs round-robin; give each XCD a contiguous run of tiles,
+    // and walk a run m-fastest inside panels of 8 n-tiles so that concurrent tiles share w
+    const int total = tiles_m * tiles_n;
+    int id = blockIdx.x;
+    {
+        const int xcds = 8;
+        const int per = (total + xcds - 1) / xcds;
+        const int mapped = (id % xcds) * per + id / xcds;
+        id = mapped;
+    }
+    if (id >= total) return;
+    constexpr int PANEL = 8;
+    const int panel = id / (PANEL * tiles_m);
+    const int in_panel = id % (PANEL * tiles_m);
+    const int panel_width = min(PANEL, tiles_n - panel * PANEL);
+    const int tile_n = panel * PANEL + in_panel % panel_width;
+    const int tile_m = in_panel / panel_width;
+    const long m0 = (long)tile_m * BM;
+    constexpr int BN_OUT = MODE == MODE_GATED ? BN / 2 : BN;          // output columns of a tile
+    const long n0 = (long)tile_n * BN_OUT;
+
+    const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
+    const int wave_m = wave / WN, wave_n = wave % WN;
+
+    // row of w behind row r of the tile
+    auto w_row = [&](int r) -> long {
+        if constexpr (MODE == MODE_GATED) {
+            const long n = n0 + (r % BN_OUT);
+            return n < N ? n + (long)(r / BN_OUT) * N : -1;
+        } else {
+            const long n = n0 + r;
+            return n < N ? n : -1;
+        }
+    };
+
+    bf16x8 stage_a[CHUNKS_A], stage_b[CHUNKS_B];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < CHUNKS_A; ++i) {
+            const int chunk = tid + i * THREADS, r = chunk / 8, k = k0 + (chunk % 8) * 8;
+            const long m = m0 + r;
+            stage_a[i] = (m < M && k + 8 <= K) ? *reinterpret_cast<const bf16x8*>(a + m * (long)K + k) : bf16x8{};
+        }
+#pragma unroll
+        for (int i = 0; i < CHUNKS_B; ++i) {
+            const int chunk = tid + i * THREADS, r = chunk / 8, k = k0 + (chunk % 8) * 8;
+            const long n = w_row(r);
+            stage_b[i] = (n >= 0 && k + 8 <= K) ? *reinterpret_cast<const bf16x8*>(w + n * (long)K + k) : bf16x8{};
+        }
+    };
+    auto stash = [&](int buffer) {
+#pragma unroll
+        for (int i = 0; i < CHUNKS_A; ++i) {
+            const int chunk = tid + i * THREADS, r = chunk / 8, kc = chunk % 8;
+            *reinterpret_cast<bf16x8*>(lds_a + ((long)buffer * BM + r) * PITCH + kc * 8) = stage_a[i];
+        }
+#pragma unroll
+        for (int i = 0; i < CHUNKS_B; ++i) {
+            const int chunk = tid + i * THREADS, r = chunk / 8, kc = chunk % 8;
+            *reinterpret_cast<bf16x8*>(lds_b + ((long)buffer * BN + r) * PITCH + kc * 8) = stage_b[i];
+        }
+    };
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    int buffer = 0;
+    for (int k0 = 0; k0 < K; k0 += BK, buffer ^= 1) {
+        const bool more = k0 + BK < K;
+        if (more) fetch(k0 + BK);
+        const bf16* tile_a = lds_a + ((long)buffer * BM + wave_m * WAVE_M + lane % 32) * PITCH + (lane / 32) * 8;
+        const bf16* tile_b = lds_b + ((long)buffer * BN + wave_n * WAVE_N + lane % 32) * PITCH + (lane / 32) * 8;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8 ra[TM], rb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) ra[i] = *reinterpret_cast<const bf16x8*>(tile_a + i * 32 * PITCH + ks * 16);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) rb[j] = *reinterpret_cast<const bf16x8*>(tile_b + j * 32 * PITCH + ks * 16);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ra[i], rb[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) stash(buffer ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulator element e of tile (i, j) is row (e/4)*8 + (lane/32)*4 + e%4, column lane%32
+    if constexpr (MODE == MODE_GATED) {
+        // wavefronts of the right half (up) hand their accumulators to the wavefront that holds
+        // the gate values of the same rows and columns: wave_n and wave_n + WN/2
+        static_assert(WN % 2 == 0, "a gated tile needs an even number of wavefront columns");
+        float* exchange = reinterpret_cast<float*>(lds_raw);           // [pairs][TM*TN*16][64]
+        const int pair = wave_m * (WN / 2) + wave_n % (WN / 2);
+        float* mine = exchange + (long)pair * (TM * TN * 16) * XRT_WAVE;
+        if (wave_n >= WN / 2) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) mine[((i * TN + j) * 16 + e) * XRT_WAVE + lane] = acc[i][j][e];
+        }
+        __syncthreads();
+        if (wave_n < WN / 2) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
+                        const long n = n0 + wave_n * WAVE_N + j * 32 + lane % 32;
+                        const float up = mine[((i * TN + j) * 16 + e) * XRT_WAVE + lane];
+                        if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(silu(acc[i][j][e]) * up);
+                    }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
+                    const long n = n0 + wave_n * WAVE_N + j * 32 + lane % 32;
+                    if (m < M && n < N) {
+                        TO* dst = out + m * (long)N + n;
+                        if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(acc[i][j][e]);
+                        else *dst = from_float<TO>(to_float(*dst) + acc[i][j][e]);
+                    }
+                }
+    }
+}
+
+template <int BM, int BN, int WM, int WN, int MODE, typename TO>
+int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+    constexpr int BN_OUT = MODE == MODE_GATED ? BN / 2 : BN;
+    constexpr int THREADS = WM * WN * XRT_WAVE;
+    constexpr size_t staging = (size_t)2 * (BM + BN) * PITCH * sizeof(bf16);
+    constexpr size_t exchange = MODE == MODE_GATED ? (size_t)(WM * WN / 2) * (BM / WM / 32) * (BN / WN / 32) * 16 * XRT_WAVE * sizeof(float) : 0;
+    constexpr size_t lds = staging > exchange ? staging : exchange;
+    static_assert(lds <= 160 * 1024, "tile does not fit the LDS of a compute unit");
+    auto kernel = gemm_mfma_kernel<BM, BN, WM, WN, MODE, TO>;
+    static bool configured = false;          // per instantiation
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        XRT_REQUIRE(e == hipSuccess, "linear (mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        configured = true;
+    }
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN_OUT - 1) / BN_OUT;
+    const int total = tiles_m * tiles_n;
+    const unsigned grid = (unsigned)(((total + 7) / 8) * 8);           // a whole number of rounds over the XCDs
+    kernel<<<grid, THREADS, lds, s>>>(a, w, out, M, N, K, tiles_m, tiles_n);
+    XRT_LAUNCH_CHECK("linear (mfma)");
+    return 0;
+}
+
+template <typename TO>
+int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, hipStream_t s) {
+    // large tiles when they still fill the chip's 256 compute units, else smaller ones
+    const long big_tiles = (long)((M + 255) / 256) * ((N + 255) / 256);
+    const bool big = big_tiles >= 192;
+    if (mode == MODE_STORE) return big ? launch<256, 256, 2, 4, MODE_STORE, TO>(a, w, out, M, N, K, s)
+                                       : launch<128, 128, 2, 2, MODE_STORE, TO>(a, w, out, M, N, K, s);
+    if (mode == MODE_ACCUMULATE) return big ? launch<256, 256, 2, 4, MODE_ACCUMULATE, TO>(a, w, out, M, N, K, s)
+                                            : launch<128, 128, 2, 2, MODE_ACCUMULATE, TO>(a, w, out, M, N, K, s);
+    const long big_gated = (long)((M + 255) / 256) * ((N + 127) / 128);
+    return big_gated >= 192 ? launch<256, 256, 2, 4, MODE_GATED, TO>(a, w, out, M, N, K, s)
+                            : launch<128, 128, 2, 2, MODE_GATED, TO>(a, w, out, M, N, K, s);
+}
+
+}  // namespace
+
+bool xrt_linear_mfma_accepts(const void* a, const void* w, int K) {
+    return K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
+}
+
+int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+                    hipStream_t s) {
+    if (out_dtype == XRT_F32) return launch_shape<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, s);
+    return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, s);
+}

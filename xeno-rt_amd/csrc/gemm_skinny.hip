@@ -1,0 +1,177 @@
+// Matrix product for few rows (M <= 64: decode steps and short prompts), bfloat16 operands,
+// float32 accumulation on the matrix cores: out[m, n] = sum_k x[m, k] * w[n, k].
+//
+// Such a product is bound by reading w once from HBM, so the kernel is built around that
+// stream. A workgroup of 8 wavefronts owns 16 (or 32) rows of w. Each wavefront takes one
+// eighth of K and streams its part of those rows straight from global memory into the A
+// operand of v_mfma_f32_16x16x32_bf16: lane (r, c) reads 64 contiguous bytes of row r per
+// 128-wide K step (four 16-byte loads in flight), so a row is read in 256-byte runs. The B
+// operand holds the activations x (16 rows of m per tile), read with the same K permutation.
+// The eight partial sums are added in wavefront order through LDS, so the result does not
+// depend on timing. Epilogues: store (bfloat16 or float32), accumulate into float32, or the
+// gated pair silu(gate) * up with the two halves of w (rows n and n + N).
+#include "common.h"
+#include "xrt_hip.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVES = 8;
+constexpr int KSTEP = 128;       // K covered by one step of a wavefront: 4 lane groups x 32
+enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
+
+__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
+
+__device__ __forceinline__ bf16x8 load8(const bf16* __restrict__ base, long row, int n_rows, int k, int K) {
+    if (row < n_rows && k + 8 <= K) return *reinterpret_cast<const bf16x8*>(base + row * (long)K + k);
+    return bf16x8{};
+}
+
+// MT: tiles of 16 rows of x; RT: tiles of 16 rows of w per wavefront; GATED doubles the w tiles.
+template <int MT, int RT, int MODE, typename TO>
+__global__ void __launch_bounds__(WAVES * XRT_WAVE) gemm_skinny_kernel(
+    const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K) {
+    constexpr int WT = RT * (MODE == MODE_GATED ? 2 : 1);       // w tiles per wavefront
+    __shared__ floatx4 partial[2][WAVES][XRT_WAVE];
+
+    const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
+    const int r = lane % 16, c = lane / 16;
+    const long n0 = (long)blockIdx.x * (16 * RT);
+
+    const int steps = (K + KSTEP - 1) / KSTEP;
+    const int steps_per_wave = (steps + WAVES - 1) / WAVES;
+    const int k_begin = wave * steps_per_wave * KSTEP;
+    const int k_end = min(K, k_begin + steps_per_wave * KSTEP);
+
+    floatx4 acc[WT][MT];
+#pragma unroll
+    for (int t = 0; t < WT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[t][m] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // row of w that tile t of this lane reads
+    long w_row[WT];
+    int w_rows[WT];
+#pragma unroll
+    for (int t = 0; t < WT; ++t) {
+        const int rt = t % RT, half = t / RT;                   // half 1: the "up" rows of a gated product
+        w_row[t] = n0 + rt * 16 + r + (long)half * N;
+        w_rows[t] = (n0 + rt * 16 + r < N) ? (half + 1) * N : 0; // 0 rows: the load returns zeros
+    }
+
+    // two register sets for w, used in turn (indexed at compile time so that they stay in registers):
+    // while the matrix cores consume one, the loads of the next step are in flight
+    bf16x8 w_even[WT][4], w_odd[WT][4];
+    auto load_w = [&](bf16x8 (&regs)[WT][4], int kb) {
+#pragma unroll
+        for (int t = 0; t < WT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) regs[t][j] = load8(w, w_row[t], w_rows[t], kb + c * 32 + j * 8, K);
+    };
+    auto multiply = [&](const bf16x8 (&regs)[WT][4], int kb) {
+        bf16x8 xreg[MT][4];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xreg[m][j] = load8(x, m * 16 + r, M, kb + c * 32 + j * 8, K);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < WT; ++t)
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(regs[t][j], xreg[m][j], acc[t][m], 0, 0, 0);
+    };
+
+    if (k_begin < k_end) load_w(w_even, k_begin);
+    for (int kb = k_begin; kb < k_end; kb += 2 * KSTEP) {
+        const bool second = kb + KSTEP < k_end;
+        if (second) load_w(w_odd, kb + KSTEP);
+        multiply(w_even, kb);
+        if (second) {
+            if (kb + 2 * KSTEP < k_end) load_w(w_even, kb + 2 * KSTEP);
+            multiply(w_odd, kb + KSTEP);
+        }
+    }
+
+    // add the wavefronts' partial sums tile by tile, in wavefront order; the wavefront that
+    // sums a tile also writes it
+    constexpr int TILES = RT * MT;
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile) {
+        const int rt = tile / MT, m = tile % MT;
+        const int slot = tile & 1;
+        float4 gate_sum = {0.f, 0.f, 0.f, 0.f}, up_sum = {0.f, 0.f, 0.f, 0.f};
+        constexpr int PASSES = MODE == MODE_GATED ? 2 : 1;
+#pragma unroll
+        for (int pass = 0; pass < PASSES; ++pass) {
+            partial[slot][wave][lane] = acc[rt + pass * RT][m];
+            __syncthreads();
+            if (wave == tile % WAVES) {
+                floatx4 total = partial[slot][0][lane];
+#pragma unroll
+                for (int other = 1; other < WAVES; ++other) total += partial[slot][other][lane];
+                if (pass == 0) gate_sum = {total[0], total[1], total[2], total[3]};
+                else up_sum = {total[0], total[1], total[2], total[3]};
+            }
+            if (PASSES == 2) __syncthreads();
+        }
+        if (wave == tile % WAVES) {
+            const int mm = m * 16 + r;                          // lane holds column m = lane % 16 ...
+            const long nn = n0 + rt * 16 + c * 4;               // ... and rows n = (lane / 16) * 4 + i
+            if (mm < M) {
+                const float g[4] = {gate_sum.x, gate_sum.y, gate_sum.z, gate_sum.w};
+                const float u[4] = {up_sum.x, up_sum.y, up_sum.z, up_sum.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (nn + i >= N) continue;
+                    TO* dst = out + (long)mm * N + nn + i;
+                    if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(g[i]);
+                    if constexpr (MODE == MODE_ACCUMULATE) *dst = from_float<TO>(to_float(*dst) + g[i]);
+                    if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(silu(g[i]) * u[i]);
+                }
+            }
+        }
+        // slots alternate, and a slot is rewritten only two tiles later, after this tile's barrier
+    }
+}
+
+template <int MT, int RT, typename TO>
+int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, hipStream_t s) {
+    const unsigned grid = (unsigned)((N + 16 * RT - 1) / (16 * RT));
+    const dim3 block(WAVES * XRT_WAVE);
+    if (mode == MODE_STORE) gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K);
+    else if (mode == MODE_ACCUMULATE) gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K);
+    else if constexpr (RT == 1) gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K);
+    else { xrt_set_error("linear (skinny): a gated product takes one row tile per wavefront"); return 1; }
+    XRT_LAUNCH_CHECK("linear (skinny)");
+    return 0;
+}
+
+template <typename TO>
+int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, hipStream_t s) {
+    const int mt = (M + 15) / 16;
+    // two row tiles per wavefront halve the reads of x, if enough workgroups remain to fill the chip
+    const bool wide = (N / 32) >= 1024 && mode != MODE_GATED;
+    switch (mt) {
+        case 1: return wide ? launch_mode<1, 2, TO>(x, w, out, M, N, K, mode, s) : launch_mode<1, 1, TO>(x, w, out, M, N, K, mode, s);
+        case 2: return wide ? launch_mode<2, 2, TO>(x, w, out, M, N, K, mode, s) : launch_mode<2, 1, TO>(x, w, out, M, N, K, mode, s);
+        case 3: return wide ? launch_mode<3, 2, TO>(x, w, out, M, N, K, mode, s) : launch_mode<3, 1, TO>(x, w, out, M, N, K, mode, s);
+        default: return wide ? launch_mode<4, 2, TO>(x, w, out, M, N, K, mode, s) : launch_mode<4, 1, TO>(x, w, out, M, N, K, mode, s);
+    }
+}
+
+}  // namespace
+
+// Whether the skinny kernel takes this product (bfloat16 operands assumed by the caller).
+bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K) {
+    return M >= 1 && M <= 64 && K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
+}
+
+int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+                      hipStream_t s) {
+    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, s);
+    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, s);
+}

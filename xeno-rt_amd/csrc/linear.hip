@@ -4,6 +4,12 @@
 
 int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
                      int mode, hipStream_t s);
+bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K);
+int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+                      hipStream_t s);
+bool xrt_linear_mfma_accepts(const void* a, const void* w, int K);
+int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+                    hipStream_t s);
 
 extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N,
                           int K, int mode, void* stream) {
@@ -15,5 +21,10 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
     XRT_REQUIRE(mode != 1 || out_dtype == XRT_F32, "linear: accumulation needs a float32 output");
     XRT_REQUIRE(a && w && out, "linear: null operand");
     if (M == 0) return 0;
+    // bfloat16: the matrix-core kernels; float32, and shapes they refuse: the plain kernel
+    if (dtype == XRT_BF16 && xrt_linear_skinny_accepts(a, w, M, K))
+        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
+    if (dtype == XRT_BF16 && xrt_linear_mfma_accepts(a, w, K))
+        return xrt_linear_mfma(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
     return xrt_linear_plain(a, w, dtype, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
 }

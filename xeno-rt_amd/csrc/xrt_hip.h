@@ -34,11 +34,15 @@ int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, int n_kv_head
                     void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks,
                     void* stream);
 
-// causal attention of every token over its sequence's cache
+// causal attention of every token of a step over its sequence's cache. The sequences of the
+// step may be described (seq_* arrays, n_seqs, the largest token count of a sequence and the
+// longest sequence after the step): then the matrix-core kernels can be used; decode needs a
+// workspace of tokens * n_heads * ceil(max_context / 64) * (head_dim + 2) floats.
 int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                   const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                   int n_blocks, const int* positions, const int* slots, void* out, float scale, int window,
-                  void* stream);
+                  const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs,
+                  int max_count, int max_context, float* workspace, long workspace_floats, void* stream);
 
 // one token per row of float32 logits
 int xrt_sample(const float* logits, int rows, int vocab, int* out, const float* temperature,

@@ -168,6 +168,7 @@ class HipOps:
         return kv.k, kv.v, kv.block_table, kv.block_table.shape[1], n_blocks
 
     def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None):
+        from ..cache import BLOCK_TOKENS
         tokens = qkv.shape[0]
         width = (n_heads + 2 * n_kv_heads) * head_dim
         self._require(qkv, "qkv", None, (tokens, width))
@@ -175,10 +176,29 @@ class HipOps:
         self._require(batch.positions, "positions", torch.int32, (tokens,), qkv)
         self._require(batch.slots, "slots", torch.int32, (tokens,), qkv)
         k_cache, v_cache, table, stride, n_blocks = self._kv(kv, qkv, n_kv_heads, head_dim)
+        # the step's sequences, if the batch describes them: lets the matrix-core kernels run
+        offsets = getattr(batch, "sequence_offsets", None)
+        seq_slots = getattr(batch, "sequence_slots", None)
+        starts = getattr(batch, "sequence_starts", None)
+        n_seqs = max_count = max_context = 0
+        workspace, workspace_floats = None, 0
+        if offsets is not None and seq_slots is not None and starts is not None:
+            n_seqs = int(batch.n_sequences)
+            max_count, max_context = int(batch.max_count), int(batch.max_context)
+            self._require(offsets, "sequence offsets", torch.int32, (n_seqs + 1,), qkv)
+            self._require(seq_slots, "sequence slots", torch.int32, (n_seqs,), qkv)
+            self._require(starts, "sequence starts", torch.int32, (n_seqs,), qkv)
+            if max_context > stride * BLOCK_TOKENS:
+                raise KernelError(f"attention: a sequence of {max_context} tokens exceeds the block table")
+            if max_count == 1 and qkv.dtype == torch.bfloat16 and not window:
+                blocks = (max_context + BLOCK_TOKENS - 1) // BLOCK_TOKENS
+                workspace_floats = tokens * n_heads * blocks * (head_dim + 2)
+                workspace = torch.empty(workspace_floats, dtype=torch.float32, device=qkv.device)
         self._check(self.lib.xrt_attention(
             _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(k_cache), _ptr(v_cache),
             _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out),
-            ctypes.c_float(scale), int(window or 0), self._stream(qkv)))
+            ctypes.c_float(scale), int(window or 0), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
+            max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
 
     def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms):
         if logits.dim() != 2:
