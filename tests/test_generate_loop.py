@@ -173,3 +173,40 @@ def test_padding_changes_no_result(pair):
     nxt = engine.step([(slot, [11], [0])])
     assert float((nxt[0] - plain.logits(ids + [11])[5]).abs().max()) < 1e-4
     engine.free_slot(slot)
+
+
+def test_command_line_options_are_the_references():
+    # crates/xrt-cli/src/main.rs:28-49: names and defaults
+    from xeno_rt_amd.cli import build_parser, parse_prompts
+    args = build_parser().parse_args(["generate", "--model", "m", "--prompt-ids", "1,2,3"])
+    assert (args.max_tokens, args.temperature, args.top_k, args.top_p, args.repetition_penalty, args.seed) == \
+        (128, 0.8, 40, 0.95, 1.1, None)
+    args = build_parser().parse_args(["generate", "--model", "m", "--prompt-ids", "1 2;3", "--prompt-ids", "",
+                                      "--max-tokens", "5", "--temperature", "0", "--top-k", "3", "--top-p", "0.5",
+                                      "--repetition-penalty", "1.0", "--seed", "9"])
+    assert parse_prompts(args.prompt_ids) == [[1, 2], [3], []]
+    assert (args.max_tokens, args.temperature, args.top_k, args.top_p, args.repetition_penalty, args.seed) == \
+        (5, 0.0, 3, 0.5, 1.0, 9)
+    with pytest.raises(SystemExit):
+        build_parser().parse_args(["generate", "--prompt-ids", "1"])          # a model is required
+
+
+def test_request_defaults_are_the_references():
+    # crates/xrt-runtime/src/session.rs:25-36 and sampler.rs:15-25
+    request = GenerateRequest([1])
+    assert (request.max_tokens, request.temperature, request.top_k, request.top_p, request.repetition_penalty,
+            request.seed) == (128, 0.8, 40, 0.95, 1.1, None)
+    assert SamplerConfig() == SamplerConfig(0.8, 40, 0.95, 1.1, None)
+    assert SamplerConfig(temperature=1e-5).is_greedy() and not SamplerConfig(temperature=2e-5).is_greedy()
+
+
+def test_python_entry_point_on_the_cpu_stand_in(pair):
+    from xeno_rt_amd import Runtime
+    engine, plain = pair
+    session = Runtime(engine).new_session()
+    request = GenerateRequest([4, 8, 15], max_tokens=5, stop_ids=[], **GREEDY)
+    want = P.generate_greedy(plain, [4, 8, 15], 5, stop_ids=[])
+    assert session.generate(request) == want
+    seen = []
+    assert session.generate_stream(request, seen.append).tokens == want and seen == want
+    session.reset()

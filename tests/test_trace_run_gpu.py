@@ -120,3 +120,24 @@ def test_replay_without_wanted_logits_writes_no_file(tmp_path):
     out = replay(folder, "float32", tmp_path / "out", steps, 64)
     assert list(out) == [1]
     assert_logits(out[1], P.PlainModel(folder).logits([1, 2, 3, 4])[3:], "float32")
+
+
+def test_command_line_generates_what_the_plain_loop_does(tmp_path):
+    folder = make_folder(TINY["qwen3"], tmp_path / "model", seed=21, std=0.2)
+    plain = P.PlainModel(folder)
+    prompts = [[5, 9, 2], [100, 101, 102, 103, 104, 105, 106], []]
+    command = [sys.executable, os.path.join(ROOT, "bin", "xrt"), "generate", "--model", folder, "--dtype", "float32",
+               "--max-tokens", "7", "--temperature", "0", "--repetition-penalty", "1.0", "--stop-ids", "",
+               "--prompt-ids", "5,9,2;100 101 102 103 104 105 106", "--prompt-ids", ""]
+    done = subprocess.run(command, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    lines = [[int(t) for t in line.split()] for line in done.stdout.strip().splitlines()]
+    assert lines == [P.generate_greedy(plain, p, 7, stop_ids=[]) for p in prompts]
+    assert "tokens in" in done.stderr and "decode" in done.stderr and "tok/s" in done.stderr
+    # the repetition penalty of the reference's defaults reaches the kernel: it changes greedy output
+    penalised = subprocess.run(command[:11] + ["--repetition-penalty", "5.0", "--stop-ids", "", "--prompt-ids", "5,9,2"],
+                               capture_output=True, text=True, timeout=300)
+    assert penalised.returncode == 0, penalised.stderr[-2000:]
+    got = [int(t) for t in penalised.stdout.split()]
+    assert got == P.generate_greedy(plain, prompts[0], 7, stop_ids=[], repetition_penalty=5.0)
+    assert len(set(got + prompts[0])) == len(got + prompts[0])        # so strong a penalty never repeats a token
