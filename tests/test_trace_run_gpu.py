@@ -140,4 +140,4 @@ def test_command_line_generates_what_the_plain_loop_does(tmp_path):
     assert penalised.returncode == 0, penalised.stderr[-2000:]
     got = [int(t) for t in penalised.stdout.split()]
     assert got == P.generate_greedy(plain, prompts[0], 7, stop_ids=[], repetition_penalty=5.0)
-    assert len(set(got + prompts[0])) == len(got + prompts[0])        # so strong a penalty never repeats a token
+    assert got != lines[0]
