@@ -6,6 +6,8 @@ from typing import List, Sequence
 
 import torch
 
+from ..staging import staging_for
+
 
 @dataclass
 class StepBatch:
@@ -54,10 +56,7 @@ def build_batch(slots: Sequence[int], tokens: Sequence[Sequence[int]], starts: S
         token_slots.append(-1)
     n_tokens, n_sequences, n_rows = len(token_ids), len(slots), len(rows)
     packed = token_ids + positions + token_slots + list(slots) + offsets + list(starts) + rows
-    host = torch.tensor(packed, dtype=torch.int32)
-    if torch.device(device).type == "cuda":
-        host = host.pin_memory()
-    dev = host.to(device, non_blocking=True)
+    dev = staging_for(device).upload(packed)
     cuts, at = [], 0
     for size in (n_tokens, n_tokens, n_tokens, n_sequences, n_sequences + 1, n_sequences, n_rows):
         cuts.append(dev[at:at + size])

@@ -43,7 +43,7 @@ class StepError(ValueError):
 class Engine:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype="bfloat16",
                  max_tokens: int = 4096, max_slots: Optional[int] = None,
-                 max_context: Optional[int] = None, device="cuda:0", ops=None):
+                 max_context: Optional[int] = None, device="cuda:0", ops=None, graphs: bool = True):
         self.dtype = compute_dtype(dtype)
         self.device = torch.device(device)
         if ops is None:
@@ -67,6 +67,11 @@ class Engine:
         self.cache = SequenceCache(spec.cache_needs(), reads_from, max_tokens, max_slots, limit,
                                    self.dtype, self.device)
         self.vocab_size = spec.head.vocab
+        # decode steps are replayed as HIP graphs where the model allows it
+        self.graphs = None
+        if graphs and self.device.type == "cuda" and spec.capturable():
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self.model, self.cache, self.device)
 
     # -- construction ----------------------------------------------------------
     @classmethod
@@ -111,19 +116,23 @@ class Engine:
         in which their logits are returned (entries first, then want). The sequences of a step either
         all start (length 0) or all continue; their token counts may differ.
         """
-        batch = self.prepare(entries)
+        slots, tokens, wants, starts = self.prepare(entries)
         try:
-            logits = self.model.forward(batch, self.cache)
+            if self.graphs is not None and all(len(ids) == 1 for ids in tokens) and all(w == [0] for w in wants):
+                logits = self.graphs.step(slots, [ids[0] for ids in tokens], starts)
+            else:
+                logits = self.model.forward(build_batch(slots, tokens, starts, wants, self.device), self.cache)
         except Exception:
-            for slot in batch.host_slots:
+            for slot in slots:
                 self.cache.cancel(slot)
             raise
-        for slot, start, count in zip(batch.host_slots, batch.host_starts, batch.host_counts):
-            self.cache.commit(slot, start + count)
+        for slot, start, ids in zip(slots, starts, tokens):
+            self.cache.commit(slot, start + len(ids))
         return logits
 
-    def prepare(self, entries) -> StepBatch:
-        """Check a step, reserve its cache blocks, and pack it. Raises StepError before anything changes."""
+    def prepare(self, entries):
+        """Check a step and reserve its cache blocks; returns (slots, tokens, wants, starts) per sequence.
+        Raises StepError before anything changes."""
         if len(entries) == 0:
             raise StepError("a step needs at least one sequence")
         slots, tokens, wants, starts = [], [], [], []
@@ -162,7 +171,7 @@ class Engine:
                 self.cache.cancel(slot)
             raise StepError(f"the cache cannot hold this step: {error}") from None
         self.cache.sync()
-        return build_batch(slots, tokens, starts, wants, self.device)
+        return slots, tokens, wants, starts
 
 
 class LazyRandom(dict):

@@ -64,6 +64,10 @@ class ModelSpec:
                 specs[name] = spec
         return specs
 
+    def capturable(self) -> bool:
+        """Whether a decode step of this model can be recorded as a graph and replayed."""
+        return all(part.capturable for part in self.parts())
+
     def ignored_names(self) -> List[str]:
         return list(self.head.ignored_names())
 

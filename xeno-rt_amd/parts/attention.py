@@ -24,6 +24,10 @@ from .position import Rotary
 
 
 class Attention(Mixer):
+    @property
+    def capturable(self) -> bool:
+        return self.position is None or self.position.capturable
+
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: Optional[PositionEncoding] = None, qk_norm: bool = False,
                  qk_norm_eps: float = 0.0, scale: Optional[float] = None,

@@ -90,6 +90,12 @@ class Runtime:
 class Part:
     """Base of all parts."""
 
+    # True if `forward` only launches kernels on the current stream with arguments that do not
+    # depend on the step's contents, so that a decode step can be recorded once and replayed.
+    # Parts that look at the batch on the host (loops over sequences, Python arithmetic on
+    # lengths) leave it False; a model with such a part runs every step directly.
+    capturable = False
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         """Full checkpoint name -> WeightSpec of every tensor this part binds."""
         return {}

@@ -21,6 +21,10 @@ class PreNormBlock(Block):
     def parts(self):
         return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
 
+    @property
+    def capturable(self) -> bool:
+        return all(part.capturable for part in self.parts())
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         specs: Dict[str, WeightSpec] = {}
         for part in self.parts():

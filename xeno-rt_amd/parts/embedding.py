@@ -14,6 +14,8 @@ from .base import Part, Runtime, WeightSpec
 
 
 class Embedding(Part):
+    capturable = True
+
     def __init__(self, prefix: str, vocab: int, hidden: int):
         self.prefix = prefix
         self.vocab = vocab
@@ -35,6 +37,8 @@ class Embedding(Part):
 
 
 class OutputHead(Part):
+    capturable = True
+
     def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: Optional[Embedding] = None):
         self.prefix = prefix
         self.vocab = vocab

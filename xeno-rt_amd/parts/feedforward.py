@@ -16,6 +16,8 @@ from .base import FeedForward, Runtime, WeightSpec, register_part
 
 
 class GatedMLP(FeedForward):
+    capturable = True
+
     ACTIVATIONS = ("silu",)
 
     def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):

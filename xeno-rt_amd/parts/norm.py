@@ -13,6 +13,8 @@ from .base import Norm, Runtime, WeightSpec, register_part
 
 
 class RMSNorm(Norm):
+    capturable = True
+
     def __init__(self, prefix: str, dim: int, eps: float):
         self.prefix = prefix
         self.dim = dim

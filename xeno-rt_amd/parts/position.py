@@ -13,6 +13,8 @@ from .base import PositionEncoding, Runtime, register_part
 
 
 class Rotary(PositionEncoding):
+    capturable = True
+
     def __init__(self, rope_dim: int, base: float, scale: float = 1.0):
         if rope_dim <= 0 or rope_dim % 2 != 0:
             raise ValueError(f"rotary width must be positive and even, found {rope_dim}")
@@ -36,6 +38,8 @@ class Rotary(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """Leaves queries and keys as they are."""
+    capturable = True
+
 
     def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch) -> None:
         return None

@@ -22,6 +22,8 @@ from typing import List, Optional, Sequence
 
 import torch
 
+from ..staging import staging_for
+
 GREEDY_BELOW = 1e-5      # sampler.rs:63
 
 
@@ -80,7 +82,7 @@ class Sampler:
         floats = torch.tensor(
             [[c.temperature for c in configs], [c.top_p for c in configs],
              [c.repetition_penalty for c in configs], list(draws)], dtype=torch.float32).to(self.device)
-        ints = torch.tensor([c.top_k for c in configs] + offsets + history, dtype=torch.int32).to(self.device)
+        ints = staging_for(self.device).upload([c.top_k for c in configs] + offsets + history)
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
         self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2],
                         ints[2 * rows + 1:], ints[rows:2 * rows + 1], floats[3])
