@@ -149,10 +149,14 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
     }
 }
 
+// Merges the chunks of one (token, head): out = sum_k w_k O_k / sum_k w_k l_k with
+// w_k = 2^(m_k - max m), in chunk order. One thread per dimension; the weights are worked out
+// once, by the first threads, and shared through LDS; the loads of the sum do not wait on each other.
 template <int HD>
 __global__ void __launch_bounds__(HD) attention_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
     const int* __restrict__ slots, int n_heads, int chunk_blocks, int n_chunks, bf16* __restrict__ out) {
+    extern __shared__ float weights[];                    // n_chunks, then one slot for the sum
     const int token = blockIdx.y, head = blockIdx.x, d = threadIdx.x;
     bf16* dst = out + ((long)token * n_heads + head) * HD;
     if (slots[token] < 0) {
@@ -164,13 +168,20 @@ __global__ void __launch_bounds__(HD) attention_decode_merge_kernel(
     const int chunks = min(n_chunks, (n_keys + chunk_keys - 1) / chunk_keys);
     const long base = ((long)token * n_heads + head) * n_chunks;
     float m = -INFINITY;
-    for (int k = 0; k < chunks; ++k) m = fmaxf(m, part_ml[(base + k) * 2]);
-    float l = 0.f, acc = 0.f;
-    for (int k = 0; k < chunks; ++k) {
-        const float w = __builtin_amdgcn_exp2f(part_ml[(base + k) * 2] - m);
-        l += w * part_ml[(base + k) * 2 + 1];
-        acc += w * part_o[(base + k) * HD + d];
+    for (int k = 0; k < chunks; ++k) m = fmaxf(m, part_ml[(base + k) * 2]);     // same loads in every thread: broadcast
+    for (int k = d; k < chunks; k += HD) weights[k] = __builtin_amdgcn_exp2f(part_ml[(base + k) * 2] - m);
+    __syncthreads();
+    if (d == 0) {
+        float l = 0.f;
+        for (int k = 0; k < chunks; ++k) l += weights[k] * part_ml[(base + k) * 2 + 1];
+        weights[n_chunks] = l;
     }
+    float acc = 0.f;
+    const float* column = part_o + base * HD + d;
+#pragma unroll 8
+    for (int k = 0; k < chunks; ++k) acc = fmaf(weights[k], column[(long)k * HD], acc);
+    __syncthreads();
+    const float l = weights[n_chunks];
     dst[d] = (bf16)(l > 0.f ? acc / l : 0.f);
 }
 
@@ -197,7 +208,7 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
         qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, positions, slots,
         scale, (int)chunk_blocks, n_chunks, q_tiles, part_o, part_ml);
     XRT_LAUNCH_CHECK("attention (decode)");
-    attention_decode_merge_kernel<HD><<<dim3(n_heads, tokens), HD, 0, s>>>(
+    attention_decode_merge_kernel<HD><<<dim3(n_heads, tokens), HD, (n_chunks + 1) * sizeof(float), s>>>(
         part_o, part_ml, positions, slots, n_heads, (int)chunk_blocks, n_chunks, out);
     XRT_LAUNCH_CHECK("attention (decode merge)");
     return 0;

@@ -13,12 +13,14 @@ from typing import Dict
 import torch
 
 from .base import FeedForward, Runtime, WeightSpec, register_part
+from .norm import linear_glu
 
 
 class GatedMLP(FeedForward):
     capturable = True
 
     ACTIVATIONS = ("silu",)
+    takes_normed = True         # h may be a `Normed`: the gate/up product applies the norm
 
     def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):
         if activation not in self.ACTIVATIONS:
@@ -49,7 +51,7 @@ class GatedMLP(FeedForward):
         rt = self.runtime
         tokens = h.shape[0]
         act = rt.empty((tokens, self.intermediate))
-        rt.ops.linear_glu(h, self.w_gate_up, act)
+        linear_glu(rt, h, self.w_gate_up, act)
         rt.ops.linear(act, self.w_down, residual, accumulate=True)
 
 
