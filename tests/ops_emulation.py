@@ -50,15 +50,6 @@ class EmulatedOps:
         gate, up = both[:, :inter], both[:, inter:]
         out.copy_(((gate / (1.0 + torch.exp(-gate))) * up).to(out.dtype))
 
-    def norm_linear(self, x, gamma, eps, w, out, gated=False, rows=None):
-        count = x.shape[0] if rows is None else rows.shape[0]
-        normed = torch.empty((count, x.shape[1]), dtype=w.dtype, device=x.device)
-        self.rmsnorm(x, gamma, eps, normed, rows=rows)
-        if gated:
-            self.linear_glu(normed, w, out)
-        else:
-            self.linear(normed, w, out)
-
     # -- attention --------------------------------------------------------------
     def qkv_prepare(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots,
                     q_norm=None, k_norm=None, norm_eps=0.0, rope_theta=None, rope_dim=0,

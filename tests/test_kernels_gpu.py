@@ -432,25 +432,3 @@ def test_sample_rows_are_independent(ops):
     alone = [sample(ops, logits[r:r + 1].contiguous(), 0.9, 50, 0.9, 1.0, draws=[u[r]])[0] for r in range(5)]
     assert together == alone
 
-
-@pytest.mark.parametrize("gamma_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (8, 1000, 4096), (17, 96, 200), (64, 520, 1032), (5, 12, 96)])
-def test_norm_linear(ops, gamma_dtype, m, n, k):
-    """The product that takes the RMSNorm along, against norm then product; with a row gather and
-    in its gated form."""
-    x = rand(m + 3, k, seed=m, scale=3.0)
-    gamma = (rand(k, seed=1) * 0.3 + 1.0).to(gamma_dtype)
-    w = rand(2 * n, k, dtype=torch.bfloat16, seed=n, scale=0.1)
-    rows = i32([(3 * r + 1) % (m + 3) for r in range(m)])
-    xd = x.double().cpu()[rows.long().cpu()]
-    normed = P.rmsnorm(xd, gamma.double().cpu(), 1e-5)
-    both = normed @ w.double().cpu().t()
-    out = torch.empty(m, 2 * n, device=DEV)
-    ops.norm_linear(x, gamma, 1e-5, w, out, rows=rows)
-    assert rel(out.cpu(), both) < 6e-3                      # one bfloat16 rounding of the normed operand
-    act = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
-    ops.norm_linear(x, gamma, 1e-5, w, act, gated=True, rows=rows)
-    assert rel(act.cpu(), P.swiglu(both[:, :n], both[:, n:])) < 1.2e-2
-    plain = torch.empty(m + 3, 2 * n, device=DEV)
-    ops.norm_linear(x, gamma, 1e-5, w, plain)                 # without a gather
-    assert rel(plain.cpu(), P.rmsnorm(x.double().cpu(), gamma.double().cpu(), 1e-5) @ w.double().cpu().t()) < 6e-3

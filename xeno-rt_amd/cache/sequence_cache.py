@@ -19,6 +19,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Dict, List, Optional
 
+import numpy as np
 import torch
 
 from ..parts.base import CacheNeeds, KVSpec
@@ -50,10 +51,13 @@ class KVGroup:
         self.calls = calls
         self.pool = Pool(n_blocks, "block")
         self.max_blocks_per_sequence = max_blocks_per_sequence
-        # host table: the truth; device table: what kernels read, refreshed before a step
-        self.table = torch.full((max_slots, max_blocks_per_sequence), -1, dtype=torch.int32)
+        # host table: the truth (numpy, so that single entries are cheap to touch; the torch view
+        # shares its memory); device table: what kernels read, refreshed before a step
+        self._table = np.full((max_slots, max_blocks_per_sequence), -1, dtype=np.int32)
+        self.table = torch.from_numpy(self._table)
         self.device_table = self.table.to(device)
         self.dirty = False
+        self._end: Dict[int, int] = {}     # slot -> logical blocks [floor, end) may be held
         self._floor: Dict[int, int] = {}   # slot -> lowest logical block it may still hold
         shape_k = (len(calls), n_blocks, spec.n_kv_heads, BLOCK_TOKENS, spec.head_dim)
         shape_v = (len(calls), n_blocks, spec.n_kv_heads, spec.head_dim, BLOCK_TOKENS)
@@ -67,7 +71,7 @@ class KVGroup:
         return max(0, length + 1 - self.spec.window) // BLOCK_TOKENS
 
     def held(self, slot: int) -> List[int]:
-        row = self.table[slot]
+        row = self._table[slot]
         return [int(b) for b in row[row >= 0]]
 
     def grow(self, slot: int, new_length: int) -> List[int]:
@@ -75,39 +79,45 @@ class KVGroup:
         need = blocks_for(new_length)
         if need > self.max_blocks_per_sequence:
             raise CacheError(f"sequence of {new_length} tokens exceeds the cache's limit per sequence")
+        start = max(self._end.get(slot, 0), self._floor.get(slot, 0))
         added = []
         try:
-            for logical in range(need):
-                if self.table[slot, logical] < 0 and logical >= self._floor.get(slot, 0):
-                    self.table[slot, logical] = self.pool.acquire()
-                    added.append(logical)
+            for logical in range(start, need):
+                self._table[slot, logical] = self.pool.acquire()
+                added.append(logical)
         except CacheFull:
             self.drop(slot, added)
             raise
         if added:
+            self._end[slot] = need
             self.dirty = True
         return added
 
     def drop(self, slot: int, logicals: List[int]) -> None:
         for logical in logicals:
-            self.pool.release(int(self.table[slot, logical]))
-            self.table[slot, logical] = -1
+            self.pool.release(int(self._table[slot, logical]))
+            self._table[slot, logical] = -1
         if logicals:
             self.dirty = True
+            end = self._end.get(slot, 0)
+            while end > 0 and self._table[slot, end - 1] < 0:
+                end -= 1
+            self._end[slot] = end
 
     def shrink_to(self, slot: int, length: int) -> None:
         """Release what a sequence of `length` tokens no longer needs: blocks past its end,
         and blocks that have slid out of the window."""
-        past_end = [l for l in range(blocks_for(length), self.max_blocks_per_sequence)
-                    if self.table[slot, l] >= 0]
+        end = self._end.get(slot, 0)
+        past_end = [l for l in range(blocks_for(length), end) if self._table[slot, l] >= 0]
         floor = self.first_needed_block(length)
-        below = [l for l in range(0, min(floor, self.max_blocks_per_sequence)) if self.table[slot, l] >= 0]
+        below = [l for l in range(self._floor.get(slot, 0), min(floor, end)) if self._table[slot, l] >= 0]
         self._floor[slot] = floor
         self.drop(slot, past_end + below)
 
     def release_all(self, slot: int) -> None:
-        self.drop(slot, [l for l in range(self.max_blocks_per_sequence) if self.table[slot, l] >= 0])
+        self.drop(slot, [l for l in range(self._end.get(slot, 0)) if self._table[slot, l] >= 0])
         self._floor.pop(slot, None)
+        self._end.pop(slot, None)
 
     def sync(self) -> None:
         if self.dirty:

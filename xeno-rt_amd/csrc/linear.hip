@@ -7,8 +7,6 @@ int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out
 bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K);
 int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                       hipStream_t s);
-int xrt_norm_linear_skinny(const float* x, const int* rows, const void* gamma, int gamma_dtype, float eps, const void* w,
-                           void* out, int out_dtype, int M, int N, int K, int mode, hipStream_t s);
 bool xrt_linear_mfma_accepts(const void* a, const void* w, int K);
 int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                     hipStream_t s);
@@ -29,23 +27,4 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
     if (dtype == XRT_BF16 && xrt_linear_mfma_accepts(a, w, K))
         return xrt_linear_mfma(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
     return xrt_linear_plain(a, w, dtype, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
-}
-
-// Whether xrt_norm_linear takes this shape (else the caller normalises first and calls xrt_linear).
-extern "C" int xrt_norm_linear_accepts(const void* x, const void* w, int dtype, int M, int K) {
-    return dtype == XRT_BF16 && M <= 32 && xrt_linear_skinny_accepts(x, w, M, K) ? 1 : 0;
-}
-
-// out[m, n] = sum_k rmsnorm(x[rows ? rows[m] : m, :])[k] * w[n, k]; x float32, w bfloat16; mode 0 store, 2 gated
-extern "C" int xrt_norm_linear(const float* x, const int* rows, const void* gamma, int gamma_dtype, float eps,
-                               const void* w, int dtype, void* out, int out_dtype, int M, int N, int K, int mode,
-                               void* stream) {
-    XRT_REQUIRE(M >= 0 && N > 0 && K > 0, "norm_linear: bad sizes M=%d N=%d K=%d", M, N, K);
-    XRT_REQUIRE(mode == 0 || mode == 2, "norm_linear: mode %d (store and gated only)", mode);
-    XRT_REQUIRE(gamma_dtype == XRT_F32 || gamma_dtype == XRT_BF16, "norm_linear: unknown norm weight dtype %d", gamma_dtype);
-    XRT_REQUIRE(out_dtype == XRT_F32 || out_dtype == XRT_BF16, "norm_linear: unknown output dtype %d", out_dtype);
-    XRT_REQUIRE(x && gamma && w && out, "norm_linear: null operand");
-    XRT_REQUIRE(xrt_norm_linear_accepts(x, w, dtype, M, K), "norm_linear: shape not taken (M=%d K=%d dtype=%d)", M, K, dtype);
-    if (M == 0) return 0;
-    return xrt_norm_linear_skinny(x, rows, gamma, gamma_dtype, eps, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
 }

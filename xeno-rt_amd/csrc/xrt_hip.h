@@ -25,12 +25,6 @@ int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype, float eps,
 int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
                int mode, void* stream);
 
-// the same with the RMSNorm of x taken along: out = rmsnorm(x[rows ? rows[m] : m]) . w^T, x float32.
-// Only for shapes that xrt_norm_linear_accepts (few rows, bfloat16 weights); mode 0 or 2.
-int xrt_norm_linear_accepts(const void* x, const void* w, int dtype, int M, int K);
-int xrt_norm_linear(const float* x, const int* rows, const void* gamma, int gamma_dtype, float eps,
-                    const void* w, int dtype, void* out, int out_dtype, int M, int N, int K, int mode, void* stream);
-
 // per-head RMSNorm of q and k (optional), rotation of q and k (optional), write of k and v
 // into the cache (optional); qkv rows are [q heads | k heads | v heads]
 int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,

@@ -95,6 +95,5 @@ class DecoderModel:
             spec.layers[call.layer].forward(x, batch, cache.layer_cache(index))
         if batch.n_logit_rows == 0:
             return self.runtime.empty((0, spec.head.vocab), torch.float32)
-        norm = spec.final_norm
-        y = norm.lazy(x, rows=batch.logit_rows) if hasattr(norm, "lazy") else norm.forward(x, rows=batch.logit_rows)
+        y = spec.final_norm.forward(x, rows=batch.logit_rows)
         return spec.head.forward(y)

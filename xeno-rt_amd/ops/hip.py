@@ -56,8 +56,8 @@ class HipOps:
             raise KernelError(f"cannot load {path}: {error}") from None
         self.path = path
         self.lib.xrt_last_error.restype = ctypes.c_char_p
-        for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_norm_linear", "xrt_norm_linear_accepts",
-                     "xrt_qkv_prepare", "xrt_attention", "xrt_sample"):
+        for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
+                     "xrt_attention", "xrt_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
     # -- helpers -------------------------------------------------------------
@@ -130,33 +130,6 @@ class HipOps:
         if w_gate_up.shape[0] % 2 != 0:
             raise KernelError("linear_glu: the weight needs gate rows followed by as many up rows")
         self._linear(a, w_gate_up, out, 2, w_gate_up.shape[0] // 2)
-
-    def norm_linear(self, x, gamma, eps, w, out, gated=False, rows=None):
-        """out = rmsnorm(x[rows]) . w^T (gated: silu(. gate rows) * (. up rows)); x float32 [*, k]."""
-        if x.dim() != 2 or w.dim() != 2:
-            raise KernelError("norm_linear: operands must be [rows, k]")
-        k = x.shape[1]
-        m = x.shape[0] if rows is None else rows.shape[0]
-        n = w.shape[0] // 2 if gated else w.shape[0]
-        self._require(x, "norm_linear x", torch.float32)
-        self._require(gamma, "norm_linear weight", None, (k,), x)
-        self._require(w, "norm_linear w", None, None, x)
-        if w.shape[1] != k or (gated and w.shape[0] % 2):
-            raise KernelError(f"norm_linear: x has {k} columns, w is {tuple(w.shape)}")
-        self._require(out, "norm_linear out", None, (m, n), x)
-        if rows is not None:
-            self._require(rows, "norm_linear rows", torch.int32, (m,), x)
-        if m > 0 and self.lib.xrt_norm_linear_accepts(_ptr(x), _ptr(w), _code(w), m, k):
-            self._check(self.lib.xrt_norm_linear(
-                _ptr(x), _ptr(rows), _ptr(gamma), _code(gamma), ctypes.c_float(eps), _ptr(w), _code(w), _ptr(out),
-                _code(out), m, n, k, 2 if gated else 0, self._stream(x)))
-            return
-        normed = torch.empty((m, k), dtype=w.dtype, device=x.device)
-        self.rmsnorm(x, gamma, eps, normed, rows=rows)
-        if gated:
-            self.linear_glu(normed, w, out)
-        else:
-            self.linear(normed, w, out)
 
     def qkv_prepare(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm=None, k_norm=None,
                     norm_eps=0.0, rope_theta=None, rope_dim=0, rope_scale=1.0, kv=None):

@@ -20,13 +20,10 @@ from typing import Dict, Optional
 import torch
 
 from .base import CacheNeeds, KVSpec, Mixer, PositionEncoding, Runtime, WeightSpec, register_part
-from .norm import linear
 from .position import Rotary
 
 
 class Attention(Mixer):
-    takes_normed = True         # h may be a `Normed`: the q/k/v product applies the norm
-
     @property
     def capturable(self) -> bool:
         return self.position is None or self.position.capturable
@@ -91,7 +88,7 @@ class Attention(Mixer):
         tokens = h.shape[0]
         kv = cache.kv
         qkv = rt.empty((tokens, self.q_width + 2 * self.kv_width))
-        linear(rt, h, self.w_qkv, qkv)
+        ops.linear(h, self.w_qkv, qkv)
 
         dims = (self.n_heads, self.n_kv_heads, self.head_dim)
         write_to = kv if cache.writable else None

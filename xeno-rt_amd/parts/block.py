@@ -39,16 +39,11 @@ class PreNormBlock(Block):
         for part in self.parts():
             part.bind(tensors, runtime)
 
-    @staticmethod
-    def _normed(norm, part, x):
-        # a part whose first operation is a product can take the norm along with it
-        if getattr(part, "takes_normed", False) and hasattr(norm, "lazy"):
-            return norm.lazy(x)
-        return norm.forward(x)
-
     def forward(self, x, batch, cache) -> None:
-        self.mixer.forward(self._normed(self.mixer_norm, self.mixer, x), batch, cache, x)
-        self.feed_forward.forward(self._normed(self.feed_forward_norm, self.feed_forward, x), batch, x)
+        h = self.mixer_norm.forward(x)
+        self.mixer.forward(h, batch, cache, x)
+        h = self.feed_forward_norm.forward(x)
+        self.feed_forward.forward(h, batch, x)
 
 
 register_part("block", "pre_norm", PreNormBlock)

@@ -62,9 +62,7 @@ class OutputHead(Part):
         else:
             self.weight = runtime.matrix(tensors[self.prefix + "weight"])
 
-    def forward(self, y) -> torch.Tensor:
-        """float32 logits for the rows of y (a tensor, or rows still to be normalised)."""
-        from .norm import linear
+    def forward(self, y: torch.Tensor) -> torch.Tensor:
         logits = self.runtime.empty((y.shape[0], self.vocab), torch.float32)
-        linear(self.runtime, y, self.weight, logits)
+        self.runtime.ops.linear(y, self.weight, logits)
         return logits

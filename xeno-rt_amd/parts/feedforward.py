@@ -13,14 +13,12 @@ from typing import Dict
 import torch
 
 from .base import FeedForward, Runtime, WeightSpec, register_part
-from .norm import linear_glu
 
 
 class GatedMLP(FeedForward):
     capturable = True
 
     ACTIVATIONS = ("silu",)
-    takes_normed = True         # h may be a `Normed`: the gate/up product applies the norm
 
     def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):
         if activation not in self.ACTIVATIONS:
@@ -51,7 +49,7 @@ class GatedMLP(FeedForward):
         rt = self.runtime
         tokens = h.shape[0]
         act = rt.empty((tokens, self.intermediate))
-        linear_glu(rt, h, self.w_gate_up, act)
+        rt.ops.linear_glu(h, self.w_gate_up, act)
         rt.ops.linear(act, self.w_down, residual, accumulate=True)
 
 
