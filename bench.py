@@ -131,6 +131,8 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    parser.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
+                        help="for profiling: run only the decode steps, or only the prefill (prints a partial record)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this library runs on a single MI355X)")
@@ -143,12 +145,23 @@ def main() -> int:
     config = parse_config(raw)
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     element = 2 if short == "bf16" else 4
+    if args.phase != "all":
+        args.skip_points = True
     largest_batch = args.batch if args.skip_points else max(args.batch, 64)
     engine = Engine.random(config, seed=args.seed, dtype=args.dtype, max_tokens=largest_batch * CONTEXT,
                            max_slots=largest_batch, max_context=CONTEXT)
     bench = Bench(engine, args.seed)
 
+    if args.phase == "prefill":
+        seconds = bench.prefill(PREFILL_TOKENS)
+        print(json.dumps({"phase": "prefill", "tokens": PREFILL_TOKENS, "ms": round(seconds * 1e3, 3),
+                          "frac": round(prefill_flops(config, PREFILL_TOKENS) / seconds / PEAK_FLOPS[short], 4)}), flush=True)
+        return 0
     tokens_per_s, ms_per_step, mean_length = bench.decode(args.batch, args.steps, args.warmup, CONTEXT)
+    if args.phase == "decode":
+        print(json.dumps({"phase": "decode", "batch": args.batch, "ms_per_step": round(ms_per_step, 4),
+                          "tokens_per_s": round(tokens_per_s, 1)}), flush=True)
+        return 0
     step_bytes = weight_bytes(config, element) + args.batch * mean_length * kv_bytes_per_token(config, element)
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
 
