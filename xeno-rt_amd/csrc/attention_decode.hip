@@ -12,9 +12,10 @@
 // O[dim][head] += V^T P, with the transposed value block as A operand (again 16 contiguous
 // bytes per lane) and the probabilities, still in the registers the scores came in, as B
 // operand: key rows are assigned to accumulator rows such that every lane ends up holding
-// eight consecutive keys, exactly the K slots of the next product. Each wavefront leaves an
-// unnormalised partial result (maximum, sum, O); a second kernel merges the chunks of a token
-// in chunk order.
+// eight consecutive keys, exactly the K slots of the next product. All loads of a cache block,
+// keys and values, are issued before anything is computed. The four wavefronts of a workgroup
+// merge their results (maximum, sum, O) through LDS into one partial result; a second kernel
+// merges the partial results of a token, in order.
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -35,31 +36,30 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
     const bf16* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads,
     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
-    float scale, int chunk_blocks, int n_chunks, int q_tiles,
+    float scale, int chunk_blocks, int n_parts, int q_tiles,
     float* __restrict__ part_o, float* __restrict__ part_ml) {
     constexpr int KS = HD / 32;                    // K steps of the score product
     constexpr int DT = HD / 16;                    // 16-row tiles of the value product
+    __shared__ floatx4 merge_o[WAVES][DT][XRT_WAVE];
+    __shared__ float merge_ml[WAVES][2][16];
+
     const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
     const int r = lane % 16, c = lane / 16;
-    const int chunk = blockIdx.x * WAVES + wave;
+    const int part = blockIdx.x;                   // this workgroup's four chunks become one partial result
+    const int chunk = part * WAVES + wave;
     const int kv_head = blockIdx.y / q_tiles, q_tile = blockIdx.y % q_tiles;
     const int token = blockIdx.z;
     const int slot = slots[token];
-    if (slot < 0 || chunk >= n_chunks) return;
+    if (slot < 0) return;                          // padding: the whole workgroup leaves
     const int n_keys = positions[token] + 1;
+    if (part * WAVES * chunk_blocks * XRT_BLOCK_TOKENS >= n_keys) return;      // nothing here for any wavefront
     const int first_block = chunk * chunk_blocks;
-    if (first_block * XRT_BLOCK_TOKENS >= n_keys) return;
+    const bool active = first_block * XRT_BLOCK_TOKENS < n_keys;
     const int last_block = min((n_keys - 1) / XRT_BLOCK_TOKENS, first_block + chunk_blocks - 1);
     const int group = n_heads / n_kv_heads;
     const int head_in_group = q_tile * 16 + r;             // this lane's query head (column of the products)
     const bool head_valid = head_in_group < group;
-    const int head = kv_head * group + head_in_group;
-
-    bf16x8 q[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-        q[ks] = head_valid ? *reinterpret_cast<const bf16x8*>(qkv + (long)token * row_width + (long)head * HD + ks * 32 + c * 8)
-                           : bf16x8{};
+    const int head = kv_head * group + min(head_in_group, group - 1);
 
     const float scale2 = scale * LOG2E;                    // scores are kept in units of log2
     float m = -INFINITY, l = 0.f;
@@ -67,122 +67,189 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (int b = first_block; b <= last_block; ++b) {
-        const int block = block_table[(long)slot * table_stride + b];
-        if (block < 0 || block >= n_blocks) continue;      // the host never lets this happen
-        const bf16* kb = k_cache + ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * HD;
-        const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * XRT_BLOCK_TOKENS;
-        const int valid = min(XRT_BLOCK_TOKENS, n_keys - b * XRT_BLOCK_TOKENS);   // keys of this block that exist
+    if (active) {
+        bf16x8 q[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            q[ks] = *reinterpret_cast<const bf16x8*>(qkv + (long)token * row_width + (long)head * HD + ks * 32 + c * 8);
 
-        // ---- scores of 64 keys: two groups of 32, two tiles of 16 rows each
-        floatx4 s[2][2];
-#pragma unroll
-        for (int g = 0; g < 2; ++g)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                s[g][t] = floatx4{0.f, 0.f, 0.f, 0.f};
-                const bf16* key = kb + (long)(g * 32 + key_of_row(t, r)) * HD + c * 8;
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    s[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(key + ks * 32), q[ks], s[g][t], 0, 0, 0);
-            }
-        // register i of s[g][t] is key g*32 + c*8 + t*4 + i, for query head r
-        float block_max = -INFINITY;
-#pragma unroll
-        for (int g = 0; g < 2; ++g)
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = g * 32 + c * 8 + t * 4 + i;
-                    const float v = key < valid ? s[g][t][i] * scale2 : -INFINITY;   // also drops whatever lies past the end
-                    s[g][t][i] = v;
-                    block_max = fmaxf(block_max, v);
-                }
-        block_max = fmaxf(block_max, __shfl_xor(block_max, 16, XRT_WAVE));
-        block_max = fmaxf(block_max, __shfl_xor(block_max, 32, XRT_WAVE));
-        const float m_new = fmaxf(m, block_max);           // finite: key 0 of the block exists
-        const float correction = __builtin_amdgcn_exp2f(m - m_new);
-        m = m_new;
-        l *= correction;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o[dt] *= correction;
+        for (int b = first_block; b <= last_block; ++b) {
+            int block = block_table[(long)slot * table_stride + b];
+            block = min(max(block, 0), n_blocks - 1);          // the host never hands out anything else
+            const bf16* kb = k_cache + ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * HD;
+            const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * XRT_BLOCK_TOKENS;
+            const int valid = min(XRT_BLOCK_TOKENS, n_keys - b * XRT_BLOCK_TOKENS);   // keys of this block that exist
 
-        // ---- probabilities, and the value product
+            // all loads of the block go out together: the values do not wait for the scores
+            bf16x8 kreg[2][2][KS], vreg[2][DT];
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
-            bf16x8 p;
+            for (int g = 0; g < 2; ++g)
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+                for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float e = __builtin_amdgcn_exp2f(s[g][t][i] - m_new);
-                    l += e;
-                    p[t * 4 + i] = (bf16)e;
+                    for (int ks = 0; ks < KS; ++ks)
+                        kreg[g][t][ks] = *reinterpret_cast<const bf16x8*>(kb + (long)(g * 32 + key_of_row(t, r)) * HD + c * 8 + ks * 32);
+#pragma unroll
+            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    vreg[g][dt] = *reinterpret_cast<const bf16x8*>(vb + (long)(dt * 16 + r) * XRT_BLOCK_TOKENS + g * 32 + c * 8);
+
+            // ---- scores of 64 keys: two groups of 32, two tiles of 16 rows each
+            floatx4 s[2][2];
+#pragma unroll
+            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    s[g][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        s[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[g][t][ks], q[ks], s[g][t], 0, 0, 0);
                 }
+            // register i of s[g][t] is key g*32 + c*8 + t*4 + i, for query head r
+            float block_max = -INFINITY;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                bf16x8 v = *reinterpret_cast<const bf16x8*>(vb + (long)(dt * 16 + r) * XRT_BLOCK_TOKENS + g * 32 + c * 8);
-                if (valid < XRT_BLOCK_TOKENS) {
-                    // the block's tail belongs to nobody: whatever it holds must not meet the zeros of p
+            for (int g = 0; g < 2; ++g)
 #pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (g * 32 + c * 8 + e >= valid) v[e] = (bf16)0.f;
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = g * 32 + c * 8 + t * 4 + i;
+                        const float v = key < valid ? s[g][t][i] * scale2 : -INFINITY;   // also drops whatever lies past the end
+                        s[g][t][i] = v;
+                        block_max = fmaxf(block_max, v);
+                    }
+            block_max = fmaxf(block_max, __shfl_xor(block_max, 16, XRT_WAVE));
+            block_max = fmaxf(block_max, __shfl_xor(block_max, 32, XRT_WAVE));
+            const float m_new = fmaxf(m, block_max);           // finite: key 0 of the block exists
+            const float correction = __builtin_amdgcn_exp2f(m - m_new);
+            m = m_new;
+            l *= correction;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o[dt] *= correction;
+
+            // ---- probabilities, and the value product
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                bf16x8 p;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float e = __builtin_amdgcn_exp2f(s[g][t][i] - m_new);
+                        l += e;
+                        p[t * 4 + i] = (bf16)e;
+                    }
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    bf16x8 v = vreg[g][dt];
+                    if (valid < XRT_BLOCK_TOKENS) {
+                        // the block's tail belongs to nobody: whatever it holds must not meet the zeros of p
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (g * 32 + c * 8 + e >= valid) v[e] = (bf16)0.f;
+                    }
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p, o[dt], 0, 0, 0);
                 }
-                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p, o[dt], 0, 0, 0);
             }
         }
+        l += __shfl_xor(l, 16, XRT_WAVE);
+        l += __shfl_xor(l, 32, XRT_WAVE);
     }
-    l += __shfl_xor(l, 16, XRT_WAVE);
-    l += __shfl_xor(l, 32, XRT_WAVE);
 
-    if (head_valid) {
-        const long slot_index = ((long)token * n_heads + head) * n_chunks + chunk;
-        float* dst = part_o + slot_index * HD;
+    // ---- the four wavefronts' results become one, in wavefront order
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) merge_o[wave][dt][lane] = o[dt];
+    if (c == 0) {
+        merge_ml[wave][0][r] = m;                  // -inf for a wavefront without keys
+        merge_ml[wave][1][r] = l;
+    }
+    __syncthreads();
+    if (wave == 0 && head_valid) {
+        float m_all = merge_ml[0][0][r];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) m_all = fmaxf(m_all, merge_ml[w][0][r]);
+        float l_all = 0.f;
+        floatx4 total[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) total[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float weight = __builtin_amdgcn_exp2f(merge_ml[w][0][r] - m_all);     // 0 for a wavefront without keys
+            l_all += weight * merge_ml[w][1][r];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) total[dt] += merge_o[w][dt][lane] * weight;
+        }
+        const long index = ((long)token * n_heads + head) * n_parts + part;
+        float* dst = part_o + index * HD;
         // accumulator register i of tile dt is dimension dt*16 + c*4 + i, for query head r
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<floatx4*>(dst + dt * 16 + c * 4) = o[dt];
+        for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<floatx4*>(dst + dt * 16 + c * 4) = total[dt];
         if (c == 0) {
-            part_ml[slot_index * 2] = m;
-            part_ml[slot_index * 2 + 1] = l;
+            part_ml[index * 2] = m_all;
+            part_ml[index * 2 + 1] = l_all;
         }
     }
 }
 
-// Merges the chunks of one (token, head): out = sum_k w_k O_k / sum_k w_k l_k with
-// w_k = 2^(m_k - max m), in chunk order. One thread per dimension; the weights are worked out
-// once, by the first threads, and shared through LDS; the loads of the sum do not wait on each other.
+// Merges the partial results of one (token, head): out = sum_k w_k O_k / sum_k w_k l_k with
+// w_k = 2^(m_k - max m), in order. One thread per dimension. The weights are worked out once,
+// by one thread per partial result, and shared through LDS; maximum and sum are wavefront
+// reductions in a fixed order.
 template <int HD>
 __global__ void __launch_bounds__(HD) attention_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
-    const int* __restrict__ slots, int n_heads, int chunk_blocks, int n_chunks, bf16* __restrict__ out) {
-    extern __shared__ float weights[];                    // n_chunks, then one slot for the sum
+    const int* __restrict__ slots, int n_heads, int part_keys, int n_parts, bf16* __restrict__ out) {
+    extern __shared__ float weights[];                    // n_parts
+    __shared__ float reduce[HD / XRT_WAVE][2];
     const int token = blockIdx.y, head = blockIdx.x, d = threadIdx.x;
+    const int lane = d % XRT_WAVE, wave = d / XRT_WAVE;
     bf16* dst = out + ((long)token * n_heads + head) * HD;
     if (slots[token] < 0) {
         dst[d] = (bf16)0.f;
         return;
     }
     const int n_keys = positions[token] + 1;
-    const int chunk_keys = chunk_blocks * XRT_BLOCK_TOKENS;
-    const int chunks = min(n_chunks, (n_keys + chunk_keys - 1) / chunk_keys);
-    const long base = ((long)token * n_heads + head) * n_chunks;
+    const int parts = min(n_parts, (n_keys + part_keys - 1) / part_keys);
+    const long base = ((long)token * n_heads + head) * n_parts;
     float m = -INFINITY;
-    for (int k = 0; k < chunks; ++k) m = fmaxf(m, part_ml[(base + k) * 2]);     // same loads in every thread: broadcast
-    for (int k = d; k < chunks; k += HD) weights[k] = __builtin_amdgcn_exp2f(part_ml[(base + k) * 2] - m);
+    for (int k = d; k < parts; k += HD) m = fmaxf(m, part_ml[(base + k) * 2]);
+    m = wave_max(m);
+    if (lane == 0) reduce[wave][0] = m;
     __syncthreads();
-    if (d == 0) {
-        float l = 0.f;
-        for (int k = 0; k < chunks; ++k) l += weights[k] * part_ml[(base + k) * 2 + 1];
-        weights[n_chunks] = l;
+    m = reduce[0][0];
+#pragma unroll
+    for (int w = 1; w < HD / XRT_WAVE; ++w) m = fmaxf(m, reduce[w][0]);
+    float l = 0.f;
+    for (int k = d; k < parts; k += HD) {
+        const float weight = __builtin_amdgcn_exp2f(part_ml[(base + k) * 2] - m);
+        weights[k] = weight;
+        l = fmaf(weight, part_ml[(base + k) * 2 + 1], l);
     }
+    l = wave_sum(l);
+    if (lane == 0) reduce[wave][1] = l;
+    __syncthreads();
+    l = reduce[0][1];
+#pragma unroll
+    for (int w = 1; w < HD / XRT_WAVE; ++w) l += reduce[w][1];
     float acc = 0.f;
     const float* column = part_o + base * HD + d;
 #pragma unroll 8
-    for (int k = 0; k < chunks; ++k) acc = fmaf(weights[k], column[(long)k * HD], acc);
-    __syncthreads();
-    const float l = weights[n_chunks];
+    for (int k = 0; k < parts; ++k) acc = fmaf(weights[k], column[(long)k * HD], acc);
     dst[d] = (bf16)(l > 0.f ? acc / l : 0.f);
+}
+
+// How the keys of the longest sequence are cut: blocks per wavefront, and partial results
+// (each from the four wavefronts of a workgroup) per (token, head).
+struct Cut { int chunk_blocks, n_parts; };
+
+Cut cut_for(int tokens, int n_kv_heads, int q_tiles, int max_context) {
+    const int max_blocks = (max_context + XRT_BLOCK_TOKENS - 1) / XRT_BLOCK_TOKENS;
+    // enough wavefronts to fill the chip, but chunks as long as that allows
+    long chunk_blocks = ((long)tokens * n_kv_heads * q_tiles * max_blocks) / 4096;
+    chunk_blocks = chunk_blocks < 1 ? 1 : (chunk_blocks > 16 ? 16 : chunk_blocks);
+    const int n_chunks = (int)((max_blocks + chunk_blocks - 1) / chunk_blocks);
+    return Cut{(int)chunk_blocks, (n_chunks + WAVES - 1) / WAVES};
 }
 
 template <int HD>
@@ -191,25 +258,22 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
            float scale, int max_context, float* workspace, long workspace_floats, hipStream_t s) {
     const int group = n_heads / n_kv_heads;
     const int q_tiles = (group + 15) / 16;
-    const int max_blocks = (max_context + XRT_BLOCK_TOKENS - 1) / XRT_BLOCK_TOKENS;
-    // enough wavefronts to fill the chip, but chunks as long as that allows
-    long chunk_blocks = ((long)tokens * n_kv_heads * q_tiles * max_blocks) / 4096;
-    chunk_blocks = chunk_blocks < 1 ? 1 : (chunk_blocks > 16 ? 16 : chunk_blocks);
-    const int n_chunks = (int)((max_blocks + chunk_blocks - 1) / chunk_blocks);
-    const long need = (long)tokens * n_heads * n_chunks * (HD + 2);
+    const Cut cut = cut_for(tokens, n_kv_heads, q_tiles, max_context);
+    const long need = (long)tokens * n_heads * cut.n_parts * (HD + 2);
     XRT_REQUIRE(workspace != nullptr && workspace_floats >= need,
                 "attention (decode): workspace of %ld floats given, %ld needed", workspace_floats, need);
     float* part_o = workspace;
-    float* part_ml = workspace + (long)tokens * n_heads * n_chunks * HD;
+    float* part_ml = workspace + (long)tokens * n_heads * cut.n_parts * HD;
     const int row_width = (n_heads + 2 * n_kv_heads) * HD;
     XRT_REQUIRE(tokens <= 65535 && n_kv_heads * q_tiles <= 65535, "attention (decode): grid too large");
-    const dim3 grid((n_chunks + WAVES - 1) / WAVES, n_kv_heads * q_tiles, tokens);
+    const dim3 grid(cut.n_parts, n_kv_heads * q_tiles, tokens);
     attention_decode_kernel<HD><<<grid, WAVES * XRT_WAVE, 0, s>>>(
         qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, positions, slots,
-        scale, (int)chunk_blocks, n_chunks, q_tiles, part_o, part_ml);
+        scale, cut.chunk_blocks, cut.n_parts, q_tiles, part_o, part_ml);
     XRT_LAUNCH_CHECK("attention (decode)");
-    attention_decode_merge_kernel<HD><<<dim3(n_heads, tokens), HD, (n_chunks + 1) * sizeof(float), s>>>(
-        part_o, part_ml, positions, slots, n_heads, (int)chunk_blocks, n_chunks, out);
+    const int part_keys = cut.chunk_blocks * WAVES * XRT_BLOCK_TOKENS;
+    attention_decode_merge_kernel<HD><<<dim3(n_heads, tokens), HD, cut.n_parts * sizeof(float), s>>>(
+        part_o, part_ml, positions, slots, n_heads, part_keys, cut.n_parts, out);
     XRT_LAUNCH_CHECK("attention (decode merge)");
     return 0;
 }
