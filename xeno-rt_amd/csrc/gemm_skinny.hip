@@ -211,7 +211,9 @@ int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int
     const int mt = (M + 15) / 16;
     // two row tiles per wavefront keep more loads in flight and halve the reads of x, if enough
     // workgroups remain to fill the chip
-    const bool wide = (N / 32) >= 1024 && mode != MODE_GATED;
+    // (with three or four tiles of x the reads of x from L2 outweigh those of w from HBM: then
+    // the wider tile pays as soon as it leaves most compute units a workgroup)
+    const bool wide = mode != MODE_GATED && (N / 32) >= (mt >= 3 ? 160 : 1024);
 #define XRT_SKINNY(MT_) (wide ? launch_mode<MT_, 2, TO>(x, w, out, M, N, K, mode, s) : launch_mode<MT_, 1, TO>(x, w, out, M, N, K, mode, s))
     switch (mt) {
         case 1: return XRT_SKINNY(1);
