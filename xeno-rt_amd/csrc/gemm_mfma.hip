@@ -68,42 +68,57 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
     const int wave_m = wave / WN, wave_n = wave % WN;
 
-    // row of w behind row r of the tile
+    // Row of w behind row r of the tile. Rows beyond the operands are clamped to the last row:
+    // loads then need no guard, and what such a row contributes lands in outputs that are not written.
     auto w_row = [&](int r) -> long {
         if constexpr (MODE == MODE_GATED) {
-            const long n = n0 + (r % BN_OUT);
-            return n < N ? n + (long)(r / BN_OUT) * N : -1;
+            return min(n0 + (r % BN_OUT), (long)N - 1) + (long)(r / BN_OUT) * N;
         } else {
-            const long n = n0 + r;
-            return n < N ? n : -1;
+            return min(n0 + r, (long)N - 1);
         }
     };
+    // element offsets of this thread's chunks from the operands' bases (32 bits: the launcher checks)
+    unsigned off_a[CHUNKS_A], off_b[CHUNKS_B];
+#pragma unroll
+    for (int i = 0; i < CHUNKS_A; ++i) {
+        const int chunk = tid + i * THREADS;
+        off_a[i] = (unsigned)(min(m0 + chunk / 8, (long)M - 1) * K + (chunk % 8) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < CHUNKS_B; ++i) {
+        const int chunk = tid + i * THREADS;
+        off_b[i] = (unsigned)(w_row(chunk / 8) * K + (chunk % 8) * 8);
+    }
 
-    bf16x8 stage_a[CHUNKS_A], stage_b[CHUNKS_B];
-    auto fetch = [&](int k0) {
+    struct Stage { bf16x8 a[CHUNKS_A], b[CHUNKS_B]; };
+    auto fetch = [&](Stage& stage, int k0) {                  // a whole tile of 64 along k, no guards
+#pragma unroll
+        for (int i = 0; i < CHUNKS_A; ++i) stage.a[i] = *reinterpret_cast<const bf16x8*>(a + (off_a[i] + (unsigned)k0));
+#pragma unroll
+        for (int i = 0; i < CHUNKS_B; ++i) stage.b[i] = *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0));
+    };
+    auto fetch_tail = [&](Stage& stage, int k0) {             // the last tile when K is no multiple of 64: zeros beyond K
 #pragma unroll
         for (int i = 0; i < CHUNKS_A; ++i) {
-            const int chunk = tid + i * THREADS, r = chunk / 8, k = k0 + (chunk % 8) * 8;
-            const long m = m0 + r;
-            stage_a[i] = (m < M && k + 8 <= K) ? *reinterpret_cast<const bf16x8*>(a + m * (long)K + k) : bf16x8{};
+            const int k = k0 + ((tid + i * THREADS) % 8) * 8;
+            stage.a[i] = k + 8 <= K ? *reinterpret_cast<const bf16x8*>(a + (off_a[i] + (unsigned)k0)) : bf16x8{};
         }
 #pragma unroll
         for (int i = 0; i < CHUNKS_B; ++i) {
-            const int chunk = tid + i * THREADS, r = chunk / 8, k = k0 + (chunk % 8) * 8;
-            const long n = w_row(r);
-            stage_b[i] = (n >= 0 && k + 8 <= K) ? *reinterpret_cast<const bf16x8*>(w + n * (long)K + k) : bf16x8{};
+            const int k = k0 + ((tid + i * THREADS) % 8) * 8;
+            stage.b[i] = k + 8 <= K ? *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0)) : bf16x8{};
         }
     };
-    auto stash = [&](int buffer) {
+    auto stash = [&](const Stage& stage, int buffer) {
 #pragma unroll
         for (int i = 0; i < CHUNKS_A; ++i) {
             const int chunk = tid + i * THREADS, r = chunk / 8, kc = chunk % 8;
-            *reinterpret_cast<bf16x8*>(lds_a + ((long)buffer * BM + r) * PITCH + kc * 8) = stage_a[i];
+            *reinterpret_cast<bf16x8*>(lds_a + ((long)buffer * BM + r) * PITCH + kc * 8) = stage.a[i];
         }
 #pragma unroll
         for (int i = 0; i < CHUNKS_B; ++i) {
             const int chunk = tid + i * THREADS, r = chunk / 8, kc = chunk % 8;
-            *reinterpret_cast<bf16x8*>(lds_b + ((long)buffer * BN + r) * PITCH + kc * 8) = stage_b[i];
+            *reinterpret_cast<bf16x8*>(lds_b + ((long)buffer * BN + r) * PITCH + kc * 8) = stage.b[i];
         }
     };
 
@@ -115,13 +130,7 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    int buffer = 0;
-    for (int k0 = 0; k0 < K; k0 += BK, buffer ^= 1) {
-        const bool more = k0 + BK < K;
-        if (more) fetch(k0 + BK);
+    auto compute = [&](int buffer) {
         const bf16* tile_a = lds_a + ((long)buffer * BM + wave_m * WAVE_M + lane % 32) * PITCH + (lane / 32) * 8;
         const bf16* tile_b = lds_b + ((long)buffer * BN + wave_n * WAVE_N + lane % 32) * PITCH + (lane / 32) * 8;
 #pragma unroll
@@ -137,9 +146,52 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ra[i], rb[j], acc[i][j], 0, 0, 0);
         }
-        if (more) stash(buffer ^ 1);
+    };
+
+    // Tiles travel global -> registers -> LDS, two tiles ahead of the matrix cores: while tile t is
+    // multiplied from one LDS buffer, tile t+1 moves from registers into the other buffer and the
+    // loads of tile t+2 are in flight (two register stages, used in turn). The steady-state loop
+    // has no branch, so every wait is for exactly the loads it needs.
+    const int whole = K / BK;                                 // tiles of 64 that lie inside K
+    Stage s0, s1;
+    if (whole > 0) {
+        fetch(s0, 0);
+        if (whole > 1) fetch(s1, BK);
+        stash(s0, 0);
         __syncthreads();
+        int t = 0;                                            // LDS buffer 0 holds tile t, stage s1 tile t+1
+        for (; t + 3 < whole; t += 2) {
+            fetch(s0, (t + 2) * BK);
+            compute(0);
+            stash(s1, 1);
+            __syncthreads();
+            fetch(s1, (t + 3) * BK);
+            compute(1);
+            stash(s0, 0);
+            __syncthreads();
+        }
+        const int left = whole - t;                           // 1, 2 or 3
+        if (left == 3) fetch(s0, (t + 2) * BK);
+        compute(0);
+        if (left >= 2) {
+            stash(s1, 1);
+            __syncthreads();
+            compute(1);
+        }
+        if (left == 3) {
+            stash(s0, 0);
+            __syncthreads();
+            compute(0);
+        }
     }
+    if (whole * BK < K) {
+        fetch_tail(s0, whole * BK);
+        __syncthreads();                                      // everyone is done with buffer 0
+        stash(s0, 0);
+        __syncthreads();
+        compute(0);
+    }
+    __syncthreads();                                          // the epilogue may reuse the LDS
 
     // ---- epilogue: accumulator element e of tile (i, j) is row (e/4)*8 + (lane/32)*4 + e%4, column lane%32
     if constexpr (MODE == MODE_GATED) {
@@ -228,8 +280,9 @@ int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
 
 }  // namespace
 
-bool xrt_linear_mfma_accepts(const void* a, const void* w, int K) {
-    return K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
+bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, int mode) {
+    const long rows_w = mode == MODE_GATED ? 2L * N : N;     // operands are addressed with 32-bit element offsets
+    return K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0 && (long)M * K < (1L << 31) && rows_w * K < (1L << 31);
 }
 
 int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,

@@ -7,7 +7,7 @@ int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out
 bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K);
 int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                       hipStream_t s);
-bool xrt_linear_mfma_accepts(const void* a, const void* w, int K);
+bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, int mode);
 int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                     hipStream_t s);
 
@@ -24,7 +24,7 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
     // bfloat16: the matrix-core kernels; float32, and shapes they refuse: the plain kernel
     if (dtype == XRT_BF16 && xrt_linear_skinny_accepts(a, w, M, K))
         return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
-    if (dtype == XRT_BF16 && xrt_linear_mfma_accepts(a, w, K))
+    if (dtype == XRT_BF16 && xrt_linear_mfma_accepts(a, w, M, N, K, mode))
         return xrt_linear_mfma(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
     return xrt_linear_plain(a, w, dtype, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
 }
