@@ -160,3 +160,39 @@ def test_far_keys_among_hundreds(dtype, tmp_path):
     assert_logits(run_whole(engine, ids), want, dtype, "700 tokens whole")
     got = run_tail_decoded(engine, ids)
     assert_logits(got, want, dtype, f"700 tokens, tail decoded, first bad row {first_bad_position(got, want, dtype)}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_replayed_decode_steps_equal_direct_ones(dtype, models):
+    """Decode steps run as recorded graphs; every replay must give the bits of the same step run
+    directly, with other work (a prompt of another sequence, host synchronisation, a batch that
+    shrinks and so changes the graph) between the replays."""
+    from xeno_rt_amd.engine import Engine
+    folder, plain, _ = models["qwen3"]
+    vocab = plain.config.vocab_size
+    recorded = Engine.load(folder, dtype=dtype, max_tokens=64 * 12, max_slots=4)
+    direct = Engine.load(folder, dtype=dtype, max_tokens=64 * 12, max_slots=4, graphs=False)
+    assert recorded.graphs is not None and direct.graphs is None
+    prompts = [token_ids(vocab, n, seed=n) for n in (3, 70, 129)]
+    outputs = []
+    for engine in (recorded, direct):
+        rows = []
+        slots = [engine.alloc_slot() for _ in prompts]
+        rows.append(engine.step([(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)]))
+        live = list(range(3))
+        for step in range(70):
+            tokens = token_ids(vocab, len(live), seed=1000 + step)
+            rows.append(engine.step([(slots[i], [tokens[j]], [0]) for j, i in enumerate(live)]))
+            if step % 9 == 4:                       # other work between replays: a new sequence comes and goes
+                extra = engine.alloc_slot()
+                rows.append(engine.step([(extra, token_ids(vocab, 40, seed=step), [39])]))
+                engine.free_slot(extra)
+                torch.cuda.synchronize()
+            if step == 30:                          # the shortest request ends: the batch, and the graph, change
+                engine.free_slot(slots[live.pop(0)])
+        for i in live:
+            engine.free_slot(slots[i])
+        outputs.append([r.clone() for r in rows])
+    assert len(recorded.graphs.graphs) >= 2
+    for index, (a, b) in enumerate(zip(*outputs)):
+        assert torch.equal(a, b), f"step {index}: a replayed graph differs from the direct step"
