@@ -7,15 +7,18 @@
 // key/value head h / group), computed with the running maximum and sum of its decode loop
 // (:514-574) instead of a stored row of scores.
 //
-// A wavefront owns 32 consecutive query tokens of one sequence and one head; the four
-// wavefronts of a workgroup take four neighbouring heads, which mostly share a key/value head
-// and so hit the same cache lines. Everything is kept transposed so that one lane owns one
-// query: S^T[key][query] = K Q^T and O^T[dim][query] += V^T P^T with
-// v_mfma_f32_32x32x16_bf16. Maximum, sum and rescaling of a query are then private to a lane
-// (plus its partner 32 lanes away), and the probabilities are already in the registers, and
-// the order, that the second product wants as its B operand: key rows are assigned to
-// accumulator rows such that a lane holds eight consecutive keys per K step, which are also
-// 16 contiguous bytes of the transposed value block.
+// A workgroup owns 256 consecutive query tokens of one sequence and one head: eight wavefronts
+// with 32 queries each (two per SIMD, so that one can do its softmax while the other multiplies). It walks the sequence's cache blocks (64 keys) in order; every block
+// travels once from global memory into LDS (keys as they lie, values transposed as they lie),
+// the next block while the current one is used, and all wavefronts read their operands
+// from there. Everything is kept transposed so that one lane owns one query:
+// S^T[key][query] = K Q^T and O^T[dim][query] += V^T P^T with v_mfma_f32_32x32x16_bf16.
+// Maximum, sum and rescaling of a query are then private to a lane (plus its partner 32 lanes
+// away), and the probabilities are already in the registers, and the order, that the second
+// product wants as its B operand: key rows are assigned to accumulator rows such that a lane
+// holds eight consecutive keys per K step, which are also 16 contiguous bytes of the
+// transposed value block. LDS rows are padded by 16 bytes, which spreads the 16-byte operand
+// reads of consecutive rows over the banks.
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -24,8 +27,10 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int WAVES = 4;
+constexpr int WAVES = 8;
 constexpr int QT = 32;                 // query tokens per wavefront
+constexpr int QW = WAVES * QT;         // query tokens per workgroup
+constexpr int BT = XRT_BLOCK_TOKENS;   // keys per cache block
 constexpr float LOG2E = 1.4426950408889634f;
 
 // Key (0..31 within a tile of 32 keys) that row r of the score tile stands for. Accumulator
@@ -40,35 +45,44 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     const int* __restrict__ seq_starts, int n_seqs, bf16* __restrict__ out, float scale) {
     constexpr int KS = HD / 16;            // K steps of the score product
     constexpr int DT = HD / 32;            // 32-row tiles of the value product
-    const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
-    const int col = lane % 32, half = lane / 32;
-    const int head = blockIdx.y * WAVES + wave;
-    if (head >= n_heads) return;
+    constexpr int KP = HD + 8;             // LDS pitch of a key row
+    constexpr int VP = BT + 8;             // LDS pitch of a transposed value row
+    constexpr int CHUNKS = BT * HD / 8 / (WAVES * XRT_WAVE);    // 16-byte chunks per thread for keys (and as many for values)
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    bf16 (*lds_k)[BT * KP] = reinterpret_cast<bf16 (*)[BT * KP]>(lds_raw);                                  // [2][BT * KP]
+    bf16 (*lds_v)[HD * VP] = reinterpret_cast<bf16 (*)[HD * VP]>(lds_raw + 2 * BT * KP * sizeof(bf16));     // [2][HD * VP]
 
-    // which sequence and which of its query tiles this workgroup has
-    int tile = blockIdx.x, seq = 0, count = 0;
+    const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
+    const int col = lane % 32, half = lane / 32;
+    const int head = blockIdx.y;
+
+    // which sequence and which of its query tiles this workgroup has; the grid is walked backwards,
+    // so that the tiles with the most keys before them (the last of a sequence) start first
+    int tile = gridDim.x - 1 - blockIdx.x, seq = 0, count = 0;
     for (; seq < n_seqs; ++seq) {
         count = seq_offsets[seq + 1] - seq_offsets[seq];
-        const int tiles = (count + QT - 1) / QT;
+        const int tiles = (count + QW - 1) / QW;
         if (tile < tiles) break;
         tile -= tiles;
     }
-    if (seq >= n_seqs) return;
+    if (seq >= n_seqs) return;                               // the whole workgroup leaves
     const int slot = seq_slots[seq];
     const int start = seq_starts[seq];                       // tokens in the cache before this step
-    const int q_first = tile * QT;                           // index among the sequence's new tokens
-    const int q_count = min(QT, count - q_first);
+    const int wg_first = tile * QW;                          // index among the sequence's new tokens
+    const int wg_last_key = start + min(count, wg_first + QW) - 1;    // the furthest key any query of the workgroup sees
+    const int q_first = wg_first + wave * QT;
+    const int q_count = max(0, min(QT, count - q_first));    // queries of this wavefront that exist
     const bool q_valid = col < q_count;
-    const long token = (long)seq_offsets[seq] + q_first + col;   // row of qkv and out (if valid)
+    const long token = (long)seq_offsets[seq] + min(q_first + col, count - 1);   // row of qkv and out (clamped: loads need no guard)
     const int q_pos = start + q_first + col;                 // absolute position of this lane's query
-    const int last_key = start + q_first + q_count - 1;      // the furthest key any query of the tile sees
+    const int last_key = start + q_first + q_count - 1;      // the furthest key any query of the wavefront sees
+    const int first_masked = start + q_first;                // key tiles that end at or before this need no mask
     const int kv_head = head / (n_heads / n_kv_heads);
 
     bf16x8 q[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-        q[ks] = q_valid ? *reinterpret_cast<const bf16x8*>(qkv + token * row_width + (long)head * HD + ks * 16 + half * 8)
-                        : bf16x8{};
+        q[ks] = *reinterpret_cast<const bf16x8*>(qkv + token * row_width + (long)head * HD + ks * 16 + half * 8);
 
     const float scale2 = scale * LOG2E;
     float m = -INFINITY, l = 0.f;
@@ -78,22 +92,48 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
 
+    // ---- moving a cache block into LDS: both parts are contiguous in global memory
+    bf16x8 stage_k[CHUNKS], stage_v[CHUNKS];
+    auto fetch = [&](int b) {
+        int block = block_table[(long)slot * table_stride + b];
+        block = min(max(block, 0), n_blocks - 1);            // the host never hands out anything else
+        const bf16* kb = k_cache + ((long)block * n_kv_heads + kv_head) * BT * HD;
+        const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * BT;
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const int chunk = tid + i * WAVES * XRT_WAVE;
+            stage_k[i] = *reinterpret_cast<const bf16x8*>(kb + chunk * 8);
+            stage_v[i] = *reinterpret_cast<const bf16x8*>(vb + chunk * 8);
+        }
+    };
+    auto stash = [&](int buffer) {
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const int chunk = tid + i * WAVES * XRT_WAVE;
+            const int k_row = chunk / (HD / 8), k_at = chunk % (HD / 8);
+            *reinterpret_cast<bf16x8*>(&lds_k[buffer][k_row * KP + k_at * 8]) = stage_k[i];
+            const int v_row = chunk / (BT / 8), v_at = chunk % (BT / 8);
+            *reinterpret_cast<bf16x8*>(&lds_v[buffer][v_row * VP + v_at * 8]) = stage_v[i];
+        }
+    };
+
     const int row_key = key_of_row(col);                     // the key this lane's A-operand row stands for
-    const int first_masked = start + q_first;                // tiles whose keys all lie at or before this need no mask
 
-    for (int k0 = 0; k0 <= last_key; k0 += 32) {
-        const int block = block_table[(long)slot * table_stride + k0 / XRT_BLOCK_TOKENS];
-        if (block < 0 || block >= n_blocks) continue;        // the host never lets this happen
-        const int in_block = k0 % XRT_BLOCK_TOKENS;
-        const bf16* kb = k_cache + (((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS + in_block + row_key) * HD + half * 8;
-        const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * XRT_BLOCK_TOKENS + in_block + half * 8;
-
-        floatx16 s;
+    // one tile of 32 keys (half a block) against this wavefront's 32 queries
+    auto tile32 = [&](int buffer, int k0, int in_block) {
+        const bf16* kb = &lds_k[buffer][(in_block + row_key) * KP + half * 8];
+        const bf16* vb = &lds_v[buffer][in_block + half * 8];
+        // two accumulators, used in turn, so that consecutive products do not wait on each other
+        floatx16 s, s_odd;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+        for (int e = 0; e < 16; ++e) s[e] = s_odd[e] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
+        for (int ks = 0; ks < KS; ks += 2) {
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kb + ks * 16), q[ks], s, 0, 0, 0);
+            s_odd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kb + (ks + 1) * 16), q[ks + 1], s_odd, 0, 0, 0);
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] += s_odd[e];
 
         // register i is key k0 + (i/8)*16 + half*8 + i%8, for this lane's query
         const bool edge = k0 + 31 > first_masked;            // some key of the tile may lie beyond some query
@@ -128,7 +168,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         for (int step = 0; step < 2; ++step)
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                bf16x8 v = *reinterpret_cast<const bf16x8*>(vb + (long)(dt * 32 + col) * XRT_BLOCK_TOKENS + step * 16);
+                bf16x8 v = *reinterpret_cast<const bf16x8*>(vb + (dt * 32 + col) * VP + step * 16);
                 if (edge) {
                     // beyond the sequence's last key the block holds nothing of ours: keep it away from the zeros of p
 #pragma unroll
@@ -137,6 +177,25 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
                 }
                 o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v, p[step], o[dt], 0, 0, 0);
             }
+    };
+
+    // ---- the blocks of the sequence, in order: block b+1 travels while block b is used
+    const int last_block = wg_last_key / BT;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int b = 0; b <= last_block; ++b) {
+        const int buffer = b & 1;
+        if (b < last_block) fetch(b + 1);
+        if (q_count > 0) {
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                const int k0 = b * BT + sub * 32;
+                if (k0 <= last_key) tile32(buffer, k0, sub * 32);        // uniform in the wavefront
+            }
+        }
+        if (b < last_block) stash(buffer ^ 1);
+        __syncthreads();
     }
     l += __shfl_xor(l, 32, XRT_WAVE);
 
@@ -161,10 +220,19 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
            const int* block_table, int table_stride, int n_blocks, const int* seq_offsets, const int* seq_slots,
            const int* seq_starts, int n_seqs, bf16* out, float scale, hipStream_t s) {
     const int row_width = (n_heads + 2 * n_kv_heads) * HD;
-    // every sequence has at most ceil(count/32) tiles; their sum is at most tokens/32 + n_seqs
-    const long tiles = (tokens + QT - 1) / QT + n_seqs;
-    const dim3 grid((unsigned)tiles, (n_heads + WAVES - 1) / WAVES);
-    attention_prefill_kernel<HD><<<grid, WAVES * XRT_WAVE, 0, s>>>(
+    // every sequence has at most ceil(count/256) tiles; their sum is at most tokens/256 + n_seqs
+    const long tiles = (tokens + QW - 1) / QW + n_seqs;
+    XRT_REQUIRE(n_heads <= 65535, "attention (prefill): too many heads for the grid");
+    const dim3 grid((unsigned)tiles, n_heads);
+    constexpr size_t lds = (size_t)2 * (BT * (HD + 8) + HD * (BT + 8)) * sizeof(bf16);
+    static bool configured = false;          // per head size
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        XRT_REQUIRE(e == hipSuccess, "attention (prefill): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        configured = true;
+    }
+    attention_prefill_kernel<HD><<<grid, WAVES * XRT_WAVE, lds, s>>>(
         qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, seq_offsets,
         seq_slots, seq_starts, n_seqs, out, scale);
     XRT_LAUNCH_CHECK("attention (prefill)");
