@@ -3,7 +3,8 @@
 //
 // A workgroup computes a BM x BN tile of the output with v_mfma_f32_32x32x16_bf16. Tiles of
 // a and w, 64 wide in k, are staged through LDS: while the matrix cores work on one buffer,
-// the next tile travels global -> registers -> the other buffer (one barrier per step). LDS
+// the next tile is written into the other and the one after that is on its way from global
+// memory into registers (one barrier per step). LDS
 // rows are padded by 16 bytes so that the 16-byte operand reads of 16 consecutive rows fall
 // into different banks. Each wavefront owns a (BM/WM) x (BN/WN) part of the tile and keeps
 // its accumulators in registers for the whole K loop.
@@ -130,11 +131,15 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    auto compute = [&](int buffer) {
+    // The products of one LDS buffer. `between` runs ahead of them: it writes the next tile to the
+    // other LDS buffer and requests the tile after it. (Placing it halfway through the products
+    // was measured slower: the fetched registers then stay live across all of them.)
+    auto compute = [&](int buffer, auto between) {
         const bf16* tile_a = lds_a + ((long)buffer * BM + wave_m * WAVE_M + lane % 32) * PITCH + (lane / 32) * 8;
         const bf16* tile_b = lds_b + ((long)buffer * BN + wave_n * WAVE_N + lane % 32) * PITCH + (lane / 32) * 8;
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
+            if (ks == 0) between();
             bf16x8 ra[TM], rb[TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i) ra[i] = *reinterpret_cast<const bf16x8*>(tile_a + i * 32 * PITCH + ks * 16);
@@ -147,41 +152,34 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ra[i], rb[j], acc[i][j], 0, 0, 0);
         }
     };
+    auto nothing = [] {};
 
-    // Tiles travel global -> registers -> LDS, two tiles ahead of the matrix cores: while tile t is
-    // multiplied from one LDS buffer, tile t+1 moves from registers into the other buffer and the
-    // loads of tile t+2 are in flight (two register stages, used in turn). The steady-state loop
-    // has no branch, so every wait is for exactly the loads it needs.
+    // Tiles travel global -> registers -> LDS ahead of the matrix cores. During step t the
+    // registers hold tile t+1 (fetched a step ago): it is written into the LDS buffer that step t-1
+    // has finished with, the registers are refilled with tile t+2, and tile t is multiplied. The steady-state loop has no branch.
     const int whole = K / BK;                                 // tiles of 64 that lie inside K
-    Stage s0, s1;
+    Stage s0;
     if (whole > 0) {
         fetch(s0, 0);
-        if (whole > 1) fetch(s1, BK);
         stash(s0, 0);
+        if (whole > 1) fetch(s0, BK);
         __syncthreads();
-        int t = 0;                                            // LDS buffer 0 holds tile t, stage s1 tile t+1
+        int t = 0;                                            // LDS buffer 0 holds tile t, the registers tile t+1
         for (; t + 3 < whole; t += 2) {
-            fetch(s0, (t + 2) * BK);
-            compute(0);
-            stash(s1, 1);
+            compute(0, [&] { stash(s0, 1); fetch(s0, (t + 2) * BK); });
             __syncthreads();
-            fetch(s1, (t + 3) * BK);
-            compute(1);
-            stash(s0, 0);
+            compute(1, [&] { stash(s0, 0); fetch(s0, (t + 3) * BK); });
             __syncthreads();
         }
         const int left = whole - t;                           // 1, 2 or 3
-        if (left == 3) fetch(s0, (t + 2) * BK);
-        compute(0);
+        compute(0, [&] { if (left >= 2) stash(s0, 1); if (left == 3) fetch(s0, (t + 2) * BK); });
         if (left >= 2) {
-            stash(s1, 1);
             __syncthreads();
-            compute(1);
+            compute(1, [&] { if (left == 3) stash(s0, 0); });
         }
         if (left == 3) {
-            stash(s0, 0);
             __syncthreads();
-            compute(0);
+            compute(0, nothing);
         }
     }
     if (whole * BK < K) {
@@ -189,7 +187,7 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
         __syncthreads();                                      // everyone is done with buffer 0
         stash(s0, 0);
         __syncthreads();
-        compute(0);
+        compute(0, nothing);
     }
     __syncthreads();                                          // the epilogue may reuse the LDS
 
