@@ -2,12 +2,12 @@
 // matrix cores: out[m, n] = sum_k a[m, k] * w[n, k]; both operands are contiguous along k.
 //
 // A workgroup computes a BM x BN tile of the output with v_mfma_f32_32x32x16_bf16. Tiles of
-// a and w, 64 wide in k, are staged through LDS: while the matrix cores work on one buffer,
-// the next tile is written into the other and the one after that is on its way from global
-// memory into registers (one barrier per step). LDS
-// rows are padded by 16 bytes so that the 16-byte operand reads of 16 consecutive rows fall
-// into different banks. Each wavefront owns a (BM/WM) x (BN/WN) part of the tile and keeps
-// its accumulators in registers for the whole K loop.
+// a and w travel through LDS, several steps ahead of the matrix cores, with one barrier per
+// step. When K is a multiple of 64 they are loaded from global memory straight into LDS, in a
+// swizzled layout; otherwise they pass through registers into rows padded by 16 bytes (64 wide
+// in k, the last tile filled with zeros). Either layout keeps the 16-byte operand reads of
+// consecutive rows in different banks. Each wavefront owns a (BM/WM) x (BN/WN) part of the
+// tile and keeps its accumulators in registers for the whole K loop.
 //
 // Workgroup ids are remapped so that the workgroups that run on one XCD (ids are dealt
 // round-robin to the 8 XCDs) work on neighbouring tiles and share their operands in that
@@ -15,7 +15,7 @@
 //
 // Epilogues: store (bfloat16 or float32), accumulate into float32, or the gated pair
 // silu(gate) * up: then the w tile holds BN/2 gate rows and the BN/2 up rows that belong to
-// them (rows n and n + N of w), and the two halves meet through LDS after the K loop.
+// them (rows n and n + N of w), arranged so that each wavefront holds both of a pair.
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -28,9 +28,29 @@ constexpr int BK = 64;
 constexpr int PITCH = BK + 8;          // bf16 elements per LDS row
 enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
 
+// 16 bytes per lane from global memory into LDS without passing registers: lane l of the
+// wavefront writes LDS byte address lds_base + 16 * l (lds_base is the same for the whole
+// wavefront and travels in M0) with the 16 bytes at base + byte_offset (of that lane). Written
+// as assembly so that the waits for these loads are the explicit ones in the kernel: the
+// compiler, when it knows of such a load, waits for all of them at every barrier.
+__device__ __forceinline__ void load_to_lds(const bf16* base, unsigned byte_offset, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base), "v"(byte_offset), "s"(base) : "memory");
+}
+// Waits until at most `pending` of this wavefront's loads (the newest ones) are outstanding and
+// its LDS reads are done, then meets the workgroup's other wavefronts. __syncthreads() cannot
+// stand here: its release fence waits for every load, also those meant to stay in flight.
+template <int pending>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(pending) : "memory");
+}
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    return (unsigned)(unsigned long)(const __attribute__((address_space(3))) void*)p;
+}
+
 __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 
-template <int BM, int BN, int WM, int WN, int MODE, typename TO>
+template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
     int tiles_m, int tiles_n) {
@@ -42,7 +62,7 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     static_assert(BM * BK / 8 % THREADS == 0 && BN * BK / 8 % THREADS == 0, "tile does not divide among the threads");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    bf16* lds_a = reinterpret_cast<bf16*>(lds_raw);                    // [2][BM][PITCH]
+    bf16* lds_a = reinterpret_cast<bf16*>(lds_raw);                    // [2][BM][PITCH]; laid out differently on the direct path
     bf16* lds_b = lds_a + 2 * BM * PITCH;                              // [2][BN][PITCH]
 
     // ---- which tile: ids are dealt to XCDs round-robin; give each XCD a contiguous run of tiles,
@@ -69,60 +89,20 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
     const int wave_m = wave / WN, wave_n = wave % WN;
 
-    // Row of w behind row r of the tile. Rows beyond the operands are clamped to the last row:
-    // loads then need no guard, and what such a row contributes lands in outputs that are not written.
+    // Row of w behind row r of the tile. In the gated mode the rows that one wavefront owns are
+    // half gate rows and half the up rows of the same outputs (rows n and n + N of w), so that the
+    // pair meets in that wavefront's registers. Rows beyond the operands are clamped to the last
+    // row: loads then need no guard, and what such a row contributes lands in outputs that are
+    // not written.
     auto w_row = [&](int r) -> long {
         if constexpr (MODE == MODE_GATED) {
-            return min(n0 + (r % BN_OUT), (long)N - 1) + (long)(r / BN_OUT) * N;
+            constexpr int HALF = WAVE_N / 2;
+            const int within = r % WAVE_N;
+            return min(n0 + (r / WAVE_N) * HALF + within % HALF, (long)N - 1) + (long)(within / HALF) * N;
         } else {
             return min(n0 + r, (long)N - 1);
         }
     };
-    // element offsets of this thread's chunks from the operands' bases (32 bits: the launcher checks)
-    unsigned off_a[CHUNKS_A], off_b[CHUNKS_B];
-#pragma unroll
-    for (int i = 0; i < CHUNKS_A; ++i) {
-        const int chunk = tid + i * THREADS;
-        off_a[i] = (unsigned)(min(m0 + chunk / 8, (long)M - 1) * K + (chunk % 8) * 8);
-    }
-#pragma unroll
-    for (int i = 0; i < CHUNKS_B; ++i) {
-        const int chunk = tid + i * THREADS;
-        off_b[i] = (unsigned)(w_row(chunk / 8) * K + (chunk % 8) * 8);
-    }
-
-    struct Stage { bf16x8 a[CHUNKS_A], b[CHUNKS_B]; };
-    auto fetch = [&](Stage& stage, int k0) {                  // a whole tile of 64 along k, no guards
-#pragma unroll
-        for (int i = 0; i < CHUNKS_A; ++i) stage.a[i] = *reinterpret_cast<const bf16x8*>(a + (off_a[i] + (unsigned)k0));
-#pragma unroll
-        for (int i = 0; i < CHUNKS_B; ++i) stage.b[i] = *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0));
-    };
-    auto fetch_tail = [&](Stage& stage, int k0) {             // the last tile when K is no multiple of 64: zeros beyond K
-#pragma unroll
-        for (int i = 0; i < CHUNKS_A; ++i) {
-            const int k = k0 + ((tid + i * THREADS) % 8) * 8;
-            stage.a[i] = k + 8 <= K ? *reinterpret_cast<const bf16x8*>(a + (off_a[i] + (unsigned)k0)) : bf16x8{};
-        }
-#pragma unroll
-        for (int i = 0; i < CHUNKS_B; ++i) {
-            const int k = k0 + ((tid + i * THREADS) % 8) * 8;
-            stage.b[i] = k + 8 <= K ? *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0)) : bf16x8{};
-        }
-    };
-    auto stash = [&](const Stage& stage, int buffer) {
-#pragma unroll
-        for (int i = 0; i < CHUNKS_A; ++i) {
-            const int chunk = tid + i * THREADS, r = chunk / 8, kc = chunk % 8;
-            *reinterpret_cast<bf16x8*>(lds_a + ((long)buffer * BM + r) * PITCH + kc * 8) = stage.a[i];
-        }
-#pragma unroll
-        for (int i = 0; i < CHUNKS_B; ++i) {
-            const int chunk = tid + i * THREADS, r = chunk / 8, kc = chunk % 8;
-            *reinterpret_cast<bf16x8*>(lds_b + ((long)buffer * BN + r) * PITCH + kc * 8) = stage.b[i];
-        }
-    };
-
     floatx16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -131,96 +111,218 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    // The products of one LDS buffer. `between` runs ahead of them: it writes the next tile to the
-    // other LDS buffer and requests the tile after it. (Placing it halfway through the products
-    // was measured slower: the fetched registers then stay live across all of them.)
-    auto compute = [&](int buffer, auto between) {
-        const bf16* tile_a = lds_a + ((long)buffer * BM + wave_m * WAVE_M + lane % 32) * PITCH + (lane / 32) * 8;
-        const bf16* tile_b = lds_b + ((long)buffer * BN + wave_n * WAVE_N + lane % 32) * PITCH + (lane / 32) * 8;
+    if constexpr (DK != 0) {
+        // Tiles go from global memory straight into LDS (global_load_lds_dwordx4): no registers and
+        // no LDS write instructions in between. Tiles are DK wide in k and LDS holds STAGES of
+        // them: while one is multiplied, the next is complete and STAGES - 2 more are on their
+        // way. One load instruction of a wavefront fills 64 consecutive 16-byte places of LDS,
+        // lane by lane, which is 64 / CHUNKS whole rows; rows can therefore not be padded. Instead
+        // the chunks of a row are stored in permuted places, place = chunk ^ swizzle(row), and
+        // each lane fetches the chunk that belongs in its place. The swizzles are chosen so that
+        // the operand reads of 8 and of 16 consecutive rows at one chunk fall into different
+        // 16-byte bank groups.
+        constexpr int CHUNKS = DK / 8;                             // 16-byte chunks per row: 4 or 8
+        constexpr int ROWS = 64 / CHUNKS;                          // rows that one load instruction fills
+        constexpr int WAVES = WM * WN;
+        constexpr int LOADS_A = BM / ROWS / WAVES, LOADS_B = BN / ROWS / WAVES;   // instructions per wavefront and tile
+        constexpr int SLICES = DK / 16;
+        static_assert(DK == 32 || DK == 64, "swizzles exist for rows of 4 and of 8 chunks");
+        static_assert(BM % (ROWS * WAVES) == 0 && BN % (ROWS * WAVES) == 0, "tile rows do not divide among the wavefronts");
+        bf16* stage_a = lds_a;                                     // [STAGES][BM][DK]
+        bf16* stage_b = lds_a + STAGES * BM * DK;                  // [STAGES][BN][DK]
+        auto swizzle_of = [](int r) { return CHUNKS == 4 ? (r / 2 % 4) ^ (r / 8 % 2) : (r % 8) ^ (r / 8 % 2); };
+        const int sub = lane / CHUNKS;                             // row within the rows of one instruction
+        auto chunk_of = [&](int row) { return ((lane % CHUNKS) ^ swizzle_of(row)) * 8; };   // what belongs in this lane's place
+        unsigned off_a[LOADS_A], off_b[LOADS_B];                   // bytes
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            if (ks == 0) between();
-            bf16x8 ra[TM], rb[TN];
+        for (int i = 0; i < LOADS_A; ++i) {
+            const int r = (i * WAVES + wave) * ROWS + sub;
+            off_a[i] = (unsigned)(min(m0 + r, (long)M - 1) * K + chunk_of(r)) * 2u;
+        }
 #pragma unroll
-            for (int i = 0; i < TM; ++i) ra[i] = *reinterpret_cast<const bf16x8*>(tile_a + i * 32 * PITCH + ks * 16);
+        for (int i = 0; i < LOADS_B; ++i) {
+            const int r = (i * WAVES + wave) * ROWS + sub;
+            off_b[i] = (unsigned)(w_row(r) * K + chunk_of(r)) * 2u;
+        }
+        const unsigned wave_uniform = __builtin_amdgcn_readfirstlane(wave);
+        const unsigned lds_rows_a = lds_address(stage_a) + wave_uniform * ROWS * DK * 2;   // first rows this wavefront fills
+        const unsigned lds_rows_b = lds_address(stage_b) + wave_uniform * ROWS * DK * 2;
+        auto issue = [&](int stage, int k0) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) rb[j] = *reinterpret_cast<const bf16x8*>(tile_b + j * 32 * PITCH + ks * 16);
+            for (int i = 0; i < LOADS_A; ++i)
+                load_to_lds(a, off_a[i] + (unsigned)k0 * 2u, lds_rows_a + (unsigned)((stage * BM + i * WAVES * ROWS) * DK * 2));
+#pragma unroll
+            for (int i = 0; i < LOADS_B; ++i)
+                load_to_lds(w, off_b[i] + (unsigned)k0 * 2u, lds_rows_b + (unsigned)((stage * BN + i * WAVES * ROWS) * DK * 2));
+        };
+        const int swizzle = swizzle_of(lane % 16);                 // of every row this lane reads: they differ by multiples of 32
+        // operands of one 16-wide slice of k: TM row blocks of a, TN row blocks of w
+        struct Operands { bf16x8 a[TM], b[TN]; };
+        auto read = [&](Operands& r, int stage, int slice) {
+            const int place = ((slice * 2 + lane / 32) ^ swizzle) * 8;
+            const bf16* tile_a = stage_a + ((long)stage * BM + wave_m * WAVE_M + lane % 32) * DK + place;
+            const bf16* tile_b = stage_b + ((long)stage * BN + wave_n * WAVE_N + lane % 32) * DK + place;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) r.a[i] = *reinterpret_cast<const bf16x8*>(tile_a + i * 32 * DK);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) r.b[j] = *reinterpret_cast<const bf16x8*>(tile_b + j * 32 * DK);
+        };
+        auto multiply = [&](const Operands& r) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ra[i], rb[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(r.a[i], r.b[j], acc[i][j], 0, 0, 0);
+        };
+        // The launcher sends only K that is a multiple of DK here. Every step issues the loads of
+        // the tile STAGES - 1 steps ahead; beyond the end of k it repeats the last tile (into a
+        // stage nobody uses any more), so that the number of loads in flight is the same at every
+        // wait. The operands of each slice are read from LDS while the matrix cores work on the
+        // slice before it, across the barrier too: the first slice of the next tile is read right
+        // after the barrier, under the products of the last slice of this one.
+        constexpr int AHEAD = STAGES - 1;
+        constexpr int IN_FLIGHT = (AHEAD - 1) * (LOADS_A + LOADS_B);   // loads that may be outstanding when the next tile is needed
+        const int steps = K / DK;
+        const int last_k = (steps - 1) * DK;
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i) issue(i, min(i * DK, last_k));
+        wait_loads_and_barrier<IN_FLIGHT>();                      // tile 0 is in LDS
+        Operands operands[2];
+        read(operands[0], 0, 0);
+        for (int t = 0; t < steps; ++t) {
+            issue((t + AHEAD) % STAGES, min((t + AHEAD) * DK, last_k));   // that stage was read in step t-1, before the last barrier
+#pragma unroll
+            for (int slice = 0; slice + 1 < SLICES; ++slice) {
+                read(operands[(slice + 1) % 2], t % STAGES, slice + 1);
+                __builtin_amdgcn_sched_barrier(0);                // keeps the reads ahead of the products that hide them
+                multiply(operands[slice % 2]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            wait_loads_and_barrier<IN_FLIGHT>();                  // tile t+1 has arrived from every wavefront, tile t has been read by all
+            read(operands[0], (t + 1) % STAGES, 0);               // after the last step: a repeated tile, not used
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(operands[(SLICES - 1) % 2]);
         }
-    };
-    auto nothing = [] {};
+        wait_loads_and_barrier<0>();                              // nothing lands in LDS after this
+    } else {
+        // element offsets of this thread's chunks from the operands' bases (32 bits: the launcher checks)
+        unsigned off_a[CHUNKS_A], off_b[CHUNKS_B];
+    #pragma unroll
+        for (int i = 0; i < CHUNKS_A; ++i) {
+            const int chunk = tid + i * THREADS;
+            off_a[i] = (unsigned)(min(m0 + chunk / 8, (long)M - 1) * K + (chunk % 8) * 8);
+        }
+    #pragma unroll
+        for (int i = 0; i < CHUNKS_B; ++i) {
+            const int chunk = tid + i * THREADS;
+            off_b[i] = (unsigned)(w_row(chunk / 8) * K + (chunk % 8) * 8);
+        }
 
-    // Tiles travel global -> registers -> LDS ahead of the matrix cores. During step t the
-    // registers hold tile t+1 (fetched a step ago): it is written into the LDS buffer that step t-1
-    // has finished with, the registers are refilled with tile t+2, and tile t is multiplied. The steady-state loop has no branch.
-    const int whole = K / BK;                                 // tiles of 64 that lie inside K
-    Stage s0;
-    if (whole > 0) {
-        fetch(s0, 0);
-        stash(s0, 0);
-        if (whole > 1) fetch(s0, BK);
-        __syncthreads();
-        int t = 0;                                            // LDS buffer 0 holds tile t, the registers tile t+1
-        for (; t + 3 < whole; t += 2) {
-            compute(0, [&] { stash(s0, 1); fetch(s0, (t + 2) * BK); });
+        struct Stage { bf16x8 a[CHUNKS_A], b[CHUNKS_B]; };
+        auto fetch = [&](Stage& stage, int k0) {                  // a whole tile of 64 along k, no guards
+    #pragma unroll
+            for (int i = 0; i < CHUNKS_A; ++i) stage.a[i] = *reinterpret_cast<const bf16x8*>(a + (off_a[i] + (unsigned)k0));
+    #pragma unroll
+            for (int i = 0; i < CHUNKS_B; ++i) stage.b[i] = *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0));
+        };
+        auto fetch_tail = [&](Stage& stage, int k0) {             // the last tile when K is no multiple of 64: zeros beyond K
+    #pragma unroll
+            for (int i = 0; i < CHUNKS_A; ++i) {
+                const int k = k0 + ((tid + i * THREADS) % 8) * 8;
+                stage.a[i] = k + 8 <= K ? *reinterpret_cast<const bf16x8*>(a + (off_a[i] + (unsigned)k0)) : bf16x8{};
+            }
+    #pragma unroll
+            for (int i = 0; i < CHUNKS_B; ++i) {
+                const int k = k0 + ((tid + i * THREADS) % 8) * 8;
+                stage.b[i] = k + 8 <= K ? *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0)) : bf16x8{};
+            }
+        };
+        auto stash = [&](const Stage& stage, int buffer) {
+    #pragma unroll
+            for (int i = 0; i < CHUNKS_A; ++i) {
+                const int chunk = tid + i * THREADS, r = chunk / 8, kc = chunk % 8;
+                *reinterpret_cast<bf16x8*>(lds_a + ((long)buffer * BM + r) * PITCH + kc * 8) = stage.a[i];
+            }
+    #pragma unroll
+            for (int i = 0; i < CHUNKS_B; ++i) {
+                const int chunk = tid + i * THREADS, r = chunk / 8, kc = chunk % 8;
+                *reinterpret_cast<bf16x8*>(lds_b + ((long)buffer * BN + r) * PITCH + kc * 8) = stage.b[i];
+            }
+        };
+
+        // The products of one LDS buffer. `between` runs ahead of them: it writes the next tile to the
+        // other LDS buffer and requests the tile after it. (Placing it halfway through the products
+        // was measured slower: the fetched registers then stay live across all of them.)
+        auto compute = [&](int buffer, auto between) {
+            const bf16* tile_a = lds_a + ((long)buffer * BM + wave_m * WAVE_M + lane % 32) * PITCH + (lane / 32) * 8;
+            const bf16* tile_b = lds_b + ((long)buffer * BN + wave_n * WAVE_N + lane % 32) * PITCH + (lane / 32) * 8;
+    #pragma unroll
+            for (int ks = 0; ks < BK / 16; ++ks) {
+                if (ks == 0) between();
+                bf16x8 ra[TM], rb[TN];
+    #pragma unroll
+                for (int i = 0; i < TM; ++i) ra[i] = *reinterpret_cast<const bf16x8*>(tile_a + i * 32 * PITCH + ks * 16);
+    #pragma unroll
+                for (int j = 0; j < TN; ++j) rb[j] = *reinterpret_cast<const bf16x8*>(tile_b + j * 32 * PITCH + ks * 16);
+    #pragma unroll
+                for (int i = 0; i < TM; ++i)
+    #pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ra[i], rb[j], acc[i][j], 0, 0, 0);
+            }
+        };
+        auto nothing = [] {};
+
+        // Tiles travel global -> registers -> LDS ahead of the matrix cores. During step t the
+        // registers hold tile t+1 (fetched a step ago): it is written into the LDS buffer that step t-1
+        // has finished with, the registers are refilled with tile t+2, and tile t is multiplied. The steady-state loop has no branch.
+        const int whole = K / BK;                                 // tiles of 64 that lie inside K
+        Stage s0;
+        if (whole > 0) {
+            fetch(s0, 0);
+            stash(s0, 0);
+            if (whole > 1) fetch(s0, BK);
             __syncthreads();
-            compute(1, [&] { stash(s0, 0); fetch(s0, (t + 3) * BK); });
-            __syncthreads();
+            int t = 0;                                            // LDS buffer 0 holds tile t, the registers tile t+1
+            for (; t + 3 < whole; t += 2) {
+                compute(0, [&] { stash(s0, 1); fetch(s0, (t + 2) * BK); });
+                __syncthreads();
+                compute(1, [&] { stash(s0, 0); fetch(s0, (t + 3) * BK); });
+                __syncthreads();
+            }
+            const int left = whole - t;                           // 1, 2 or 3
+            compute(0, [&] { if (left >= 2) stash(s0, 1); if (left == 3) fetch(s0, (t + 2) * BK); });
+            if (left >= 2) {
+                __syncthreads();
+                compute(1, [&] { if (left == 3) stash(s0, 0); });
+            }
+            if (left == 3) {
+                __syncthreads();
+                compute(0, nothing);
+            }
         }
-        const int left = whole - t;                           // 1, 2 or 3
-        compute(0, [&] { if (left >= 2) stash(s0, 1); if (left == 3) fetch(s0, (t + 2) * BK); });
-        if (left >= 2) {
-            __syncthreads();
-            compute(1, [&] { if (left == 3) stash(s0, 0); });
-        }
-        if (left == 3) {
+        if (whole * BK < K) {
+            fetch_tail(s0, whole * BK);
+            __syncthreads();                                      // everyone is done with buffer 0
+            stash(s0, 0);
             __syncthreads();
             compute(0, nothing);
         }
     }
-    if (whole * BK < K) {
-        fetch_tail(s0, whole * BK);
-        __syncthreads();                                      // everyone is done with buffer 0
-        stash(s0, 0);
-        __syncthreads();
-        compute(0, nothing);
-    }
-    __syncthreads();                                          // the epilogue may reuse the LDS
 
     // ---- epilogue: accumulator element e of tile (i, j) is row (e/4)*8 + (lane/32)*4 + e%4, column lane%32
     if constexpr (MODE == MODE_GATED) {
-        // wavefronts of the right half (up) hand their accumulators to the wavefront that holds
-        // the gate values of the same rows and columns: wave_n and wave_n + WN/2
-        static_assert(WN % 2 == 0, "a gated tile needs an even number of wavefront columns");
-        float* exchange = reinterpret_cast<float*>(lds_raw);           // [pairs][TM*TN*16][64]
-        const int pair = wave_m * (WN / 2) + wave_n % (WN / 2);
-        float* mine = exchange + (long)pair * (TM * TN * 16) * XRT_WAVE;
-        if (wave_n >= WN / 2) {
+        static_assert(TN % 2 == 0, "a wavefront holds as many gate blocks as up blocks");
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN / 2; ++j)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) mine[((i * TN + j) * 16 + e) * XRT_WAVE + lane] = acc[i][j][e];
-        }
-        __syncthreads();
-        if (wave_n < WN / 2) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
-                        const long n = n0 + wave_n * WAVE_N + j * 32 + lane % 32;
-                        const float up = mine[((i * TN + j) * 16 + e) * XRT_WAVE + lane];
-                        if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(silu(acc[i][j][e]) * up);
-                    }
-        }
+                for (int e = 0; e < 16; ++e) {
+                    const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
+                    const long n = n0 + wave_n * (WAVE_N / 2) + j * 32 + lane % 32;
+                    if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(silu(acc[i][j][e]) * acc[i][j + TN / 2][e]);
+                }
     } else {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -239,15 +341,14 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     }
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, typename TO>
-int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
+int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
     constexpr int BN_OUT = MODE == MODE_GATED ? BN / 2 : BN;
     constexpr int THREADS = WM * WN * XRT_WAVE;
-    constexpr size_t staging = (size_t)2 * (BM + BN) * PITCH * sizeof(bf16);
-    constexpr size_t exchange = MODE == MODE_GATED ? (size_t)(WM * WN / 2) * (BM / WM / 32) * (BN / WN / 32) * 16 * XRT_WAVE * sizeof(float) : 0;
-    constexpr size_t lds = staging > exchange ? staging : exchange;
+    constexpr size_t staging = DK != 0 ? (size_t)STAGES * (BM + BN) * DK * sizeof(bf16) : (size_t)2 * (BM + BN) * PITCH * sizeof(bf16);
+    constexpr size_t lds = staging;
     static_assert(lds <= 160 * 1024, "tile does not fit the LDS of a compute unit");
-    auto kernel = gemm_mfma_kernel<BM, BN, WM, WN, MODE, TO>;
+    auto kernel = gemm_mfma_kernel<BM, BN, WM, WN, MODE, DK, STAGES, TO>;
     static bool configured = false;          // per instantiation
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -260,6 +361,19 @@ int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream
     kernel<<<grid, THREADS, lds, s>>>(a, w, out, M, N, K, tiles_m, tiles_n);
     XRT_LAUNCH_CHECK("linear (mfma)");
     return 0;
+}
+
+template <int BM, int BN, int WM, int WN, int MODE, typename TO>
+int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+    // Whole tiles along k go straight into LDS; a ragged last tile needs the path through
+    // registers. The large tile fills LDS with four narrow stages and keeps two tiles in flight;
+    // two workgroups of the small tile share a compute unit and cover each other's waits, and do
+    // better with fewer, wider steps.
+    if (K % 64 == 0) {
+        if constexpr (BM * BN >= 256 * 256) return launch_kernel<BM, BN, WM, WN, MODE, 32, 4, TO>(a, w, out, M, N, K, s);
+        else return launch_kernel<BM, BN, WM, WN, MODE, 64, 2, TO>(a, w, out, M, N, K, s);
+    }
+    return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, s);
 }
 
 template <typename TO>
