@@ -4,9 +4,10 @@
 // Such a product is bound by reading w once from HBM, so the kernel is built around that
 // stream. A workgroup of 8 wavefronts owns 16 (or 32) rows of w. Each wavefront takes one
 // eighth of K and streams its part of those rows straight from global memory into the A
-// operand of v_mfma_f32_16x16x32_bf16: lane (r, c) reads 64 contiguous bytes of row r per
-// 128-wide K step (four 16-byte loads), so a row is read in 256-byte runs. The B operand holds
-// the activations x (16 rows of m per tile), read with the same K permutation. Loads carry no
+// operand of v_mfma_f32_16x16x32_bf16: a 128-wide K step is four load instructions, and in each
+// the four lanes (r, 0..3) of a row read 64 contiguous bytes of it, so that one instruction
+// asks for 16 half cache lines and a row is read in 256-byte runs. The B operand holds the
+// activations x (16 rows of m per tile), read with the same K permutation. Loads carry no
 // branches (addresses are clamped into the operands instead), run one step ahead of the
 // matrix cores, and the products of a step go to accumulators that do not wait on each other:
 // all three matter, because a wavefront that stalls stops issuing its next loads.
@@ -62,23 +63,23 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     for (int t = 0; t < WT; ++t) {
         const int rt = t % RT, half = t / RT;                   // half 1: the "up" rows of a gated product
         const long n = min(n0 + rt * 16 + r, (long)N - 1);
-        w_ptr[t] = w + (n + (long)half * N) * K + c * 32;
+        w_ptr[t] = w + (n + (long)half * N) * K + c * 8;
     }
     const bf16* x_ptr[MT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) x_ptr[m] = x + (long)min(m * 16 + r, M - 1) * K + c * 32;
+    for (int m = 0; m < MT; ++m) x_ptr[m] = x + (long)min(m * 16 + r, M - 1) * K + c * 8;
 
     auto load_w = [&](bf16x8 (&regs)[WT][4], int kb) {
 #pragma unroll
         for (int t = 0; t < WT; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) regs[t][j] = *reinterpret_cast<const bf16x8*>(w_ptr[t] + kb + j * 8);
+            for (int j = 0; j < 4; ++j) regs[t][j] = *reinterpret_cast<const bf16x8*>(w_ptr[t] + kb + j * 32);
     };
     auto load_x = [&](bf16x8 (&regs)[MT][4], int kb) {
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) regs[m][j] = *reinterpret_cast<const bf16x8*>(x_ptr[m] + kb + j * 8);
+            for (int j = 0; j < 4; ++j) regs[m][j] = *reinterpret_cast<const bf16x8*>(x_ptr[m] + kb + j * 32);
     };
     auto multiply = [&](const bf16x8 (&wregs)[WT][4], const bf16x8 (&xregs)[MT][4]) {
 #pragma unroll
@@ -122,14 +123,14 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     if (tail_begin < k_end) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const bool inside = tail_begin + c * 32 + j * 8 + 8 <= K;       // K is a multiple of 8
+            const bool inside = tail_begin + j * 32 + c * 8 + 8 <= K;       // K is a multiple of 8
             bf16x8 b[MT];
 #pragma unroll
             for (int m = 0; m < MT; ++m)
-                b[m] = inside ? *reinterpret_cast<const bf16x8*>(x_ptr[m] + tail_begin + j * 8) : bf16x8{};
+                b[m] = inside ? *reinterpret_cast<const bf16x8*>(x_ptr[m] + tail_begin + j * 32) : bf16x8{};
 #pragma unroll
             for (int t = 0; t < WT; ++t) {
-                const bf16x8 a = inside ? *reinterpret_cast<const bf16x8*>(w_ptr[t] + tail_begin + j * 8) : bf16x8{};
+                const bf16x8 a = inside ? *reinterpret_cast<const bf16x8*>(w_ptr[t] + tail_begin + j * 32) : bf16x8{};
 #pragma unroll
                 for (int m = 0; m < MT; ++m)
                     chain[0][t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[m], chain[0][t][m], 0, 0, 0);
