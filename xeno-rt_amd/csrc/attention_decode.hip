@@ -205,15 +205,26 @@ __global__ void __launch_bounds__(HD) attention_decode_merge_kernel(
     const int token = blockIdx.y, head = blockIdx.x, d = threadIdx.x;
     const int lane = d % XRT_WAVE, wave = d / XRT_WAVE;
     bf16* dst = out + ((long)token * n_heads + head) * HD;
-    if (slots[token] < 0) {
+    const long base = ((long)token * n_heads + head) * n_parts;
+    const float* column = part_o + base * HD + d;
+    // Everything this thread may need is asked for at once, before it is known how many partial
+    // results count: the loads then cost one trip to memory instead of one after the other.
+    // What lies beyond the partial results that count is read (it is inside the workspace) and
+    // never used.
+    constexpr int EARLY = 16;
+    float early_o[EARLY];
+#pragma unroll
+    for (int k = 0; k < EARLY; ++k) early_o[k] = k < n_parts ? column[(long)k * HD] : 0.f;
+    const float2 early_ml = d < n_parts ? *reinterpret_cast<const float2*>(part_ml + (base + d) * 2) : make_float2(0.f, 0.f);
+    const int slot = slots[token];
+    const int n_keys = positions[token] + 1;
+    if (slot < 0) {
         dst[d] = (bf16)0.f;
         return;
     }
-    const int n_keys = positions[token] + 1;
     const int parts = min(n_parts, (n_keys + part_keys - 1) / part_keys);
-    const long base = ((long)token * n_heads + head) * n_parts;
-    float m = -INFINITY;
-    for (int k = d; k < parts; k += HD) m = fmaxf(m, part_ml[(base + k) * 2]);
+    float m = d < parts ? early_ml.x : -INFINITY;
+    for (int k = d + HD; k < parts; k += HD) m = fmaxf(m, part_ml[(base + k) * 2]);
     m = wave_max(m);
     if (lane == 0) reduce[wave][0] = m;
     __syncthreads();
@@ -221,7 +232,12 @@ __global__ void __launch_bounds__(HD) attention_decode_merge_kernel(
 #pragma unroll
     for (int w = 1; w < HD / XRT_WAVE; ++w) m = fmaxf(m, reduce[w][0]);
     float l = 0.f;
-    for (int k = d; k < parts; k += HD) {
+    if (d < parts) {
+        const float weight = __builtin_amdgcn_exp2f(early_ml.x - m);
+        weights[d] = weight;
+        l = weight * early_ml.y;
+    }
+    for (int k = d + HD; k < parts; k += HD) {
         const float weight = __builtin_amdgcn_exp2f(part_ml[(base + k) * 2] - m);
         weights[k] = weight;
         l = fmaf(weight, part_ml[(base + k) * 2 + 1], l);
@@ -233,9 +249,11 @@ __global__ void __launch_bounds__(HD) attention_decode_merge_kernel(
 #pragma unroll
     for (int w = 1; w < HD / XRT_WAVE; ++w) l += reduce[w][1];
     float acc = 0.f;
-    const float* column = part_o + base * HD + d;
+#pragma unroll
+    for (int k = 0; k < EARLY; ++k)
+        if (k < parts) acc = fmaf(weights[k], early_o[k], acc);
 #pragma unroll 8
-    for (int k = 0; k < parts; ++k) acc = fmaf(weights[k], column[(long)k * HD], acc);
+    for (int k = EARLY; k < parts; ++k) acc = fmaf(weights[k], column[(long)k * HD], acc);
     dst[d] = (bf16)(l > 0.f ? acc / l : 0.f);
 }
 

@@ -41,11 +41,13 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
         const int quads = hidden / 4;
         const float4* row4 = reinterpret_cast<const float4*>(row);
         float4 kept[CACHED];
+        Vec4<TW> gain[CACHED];                                  // asked for now, so that they arrive under the sum
         float sum = 0.f;
 #pragma unroll
         for (int i = 0; i < CACHED; ++i) {
             const int q = threadIdx.x + i * 256;
             kept[i] = q < quads ? row4[q] : make_float4(0.f, 0.f, 0.f, 0.f);
+            gain[i] = q < quads ? *reinterpret_cast<const Vec4<TW>*>(weight + 4 * q) : Vec4<TW>{};
         }
 #pragma unroll
         for (int i = 0; i < CACHED; ++i)
@@ -56,8 +58,7 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
         }
         sum = block_sum(sum, scratch);
         const float inv_rms = 1.0f / sqrtf(sum / (float)hidden + eps);
-        auto emit = [&](int q, const float4& v) {
-            const Vec4<TW> w = *reinterpret_cast<const Vec4<TW>*>(weight + 4 * q);
+        auto emit = [&](int q, const float4& v, const Vec4<TW>& w) {
             Vec4<TO> r;
             r.e[0] = from_float<TO>((v.x * inv_rms) * to_float(w.e[0]));
             r.e[1] = from_float<TO>((v.y * inv_rms) * to_float(w.e[1]));
@@ -68,9 +69,9 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
 #pragma unroll
         for (int i = 0; i < CACHED; ++i) {
             const int q = threadIdx.x + i * 256;
-            if (q < quads) emit(q, kept[i]);
+            if (q < quads) emit(q, kept[i], gain[i]);
         }
-        for (int q = threadIdx.x + CACHED * 256; q < quads; q += 256) emit(q, row4[q]);
+        for (int q = threadIdx.x + CACHED * 256; q < quads; q += 256) emit(q, row4[q], *reinterpret_cast<const Vec4<TW>*>(weight + 4 * q));
         return;
     }
     float sum = 0.f;
