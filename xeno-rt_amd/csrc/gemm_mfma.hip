@@ -16,6 +16,7 @@
 // Epilogues: store (bfloat16 or float32), accumulate into float32, or the gated pair
 // silu(gate) * up: then the w tile holds BN/2 gate rows and the BN/2 up rows that belong to
 // them (rows n and n + N of w), arranged so that each wavefront holds both of a pair.
+#include <climits>
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -59,7 +60,6 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;        // 32x32 accumulator tiles of a wavefront
     constexpr int CHUNKS_A = BM * BK / 8 / THREADS;          // 16-byte chunks each thread moves per step
     constexpr int CHUNKS_B = BN * BK / 8 / THREADS;
-    static_assert(BM * BK / 8 % THREADS == 0 && BN * BK / 8 % THREADS == 0, "tile does not divide among the threads");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     bf16* lds_a = reinterpret_cast<bf16*>(lds_raw);                    // [2][BM][PITCH]; laid out differently on the direct path
@@ -124,10 +124,13 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
         constexpr int CHUNKS = DK / 8;                             // 16-byte chunks per row: 4 or 8
         constexpr int ROWS = 64 / CHUNKS;                          // rows that one load instruction fills
         constexpr int WAVES = WM * WN;
-        constexpr int LOADS_A = BM / ROWS / WAVES, LOADS_B = BN / ROWS / WAVES;   // instructions per wavefront and tile
+        // load instructions per wavefront and tile; where the row blocks do not divide among the
+        // wavefronts, the spare instructions fetch the last block once more (same bytes, same place)
+        constexpr int BLOCKS_A = BM / ROWS, BLOCKS_B = BN / ROWS;
+        constexpr int LOADS_A = (BLOCKS_A + WAVES - 1) / WAVES, LOADS_B = (BLOCKS_B + WAVES - 1) / WAVES;
         constexpr int SLICES = DK / 16;
         static_assert(DK == 32 || DK == 64, "swizzles exist for rows of 4 and of 8 chunks");
-        static_assert(BM % (ROWS * WAVES) == 0 && BN % (ROWS * WAVES) == 0, "tile rows do not divide among the wavefronts");
+        static_assert(BM % ROWS == 0 && BN % ROWS == 0, "tile rows do not divide into load instructions");
         bf16* stage_a = lds_a;                                     // [STAGES][BM][DK]
         bf16* stage_b = lds_a + STAGES * BM * DK;                  // [STAGES][BN][DK]
         auto swizzle_of = [](int r) { return CHUNKS == 4 ? (r / 2 % 4) ^ (r / 8 % 2) : (r % 8) ^ (r / 8 % 2); };
@@ -136,24 +139,27 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
         unsigned off_a[LOADS_A], off_b[LOADS_B];                   // bytes
 #pragma unroll
         for (int i = 0; i < LOADS_A; ++i) {
-            const int r = (i * WAVES + wave) * ROWS + sub;
+            const int r = min(i * WAVES + wave, BLOCKS_A - 1) * ROWS + sub;
             off_a[i] = (unsigned)(min(m0 + r, (long)M - 1) * K + chunk_of(r)) * 2u;
         }
 #pragma unroll
         for (int i = 0; i < LOADS_B; ++i) {
-            const int r = (i * WAVES + wave) * ROWS + sub;
+            const int r = min(i * WAVES + wave, BLOCKS_B - 1) * ROWS + sub;
             off_b[i] = (unsigned)(w_row(r) * K + chunk_of(r)) * 2u;
         }
-        const unsigned wave_uniform = __builtin_amdgcn_readfirstlane(wave);
-        const unsigned lds_rows_a = lds_address(stage_a) + wave_uniform * ROWS * DK * 2;   // first rows this wavefront fills
-        const unsigned lds_rows_b = lds_address(stage_b) + wave_uniform * ROWS * DK * 2;
+        const int wave_uniform = __builtin_amdgcn_readfirstlane(wave);
+        const unsigned lds_a0 = lds_address(stage_a), lds_b0 = lds_address(stage_b);
         auto issue = [&](int stage, int k0) {
 #pragma unroll
-            for (int i = 0; i < LOADS_A; ++i)
-                load_to_lds(a, off_a[i] + (unsigned)k0 * 2u, lds_rows_a + (unsigned)((stage * BM + i * WAVES * ROWS) * DK * 2));
+            for (int i = 0; i < LOADS_A; ++i) {
+                const int block = min(i * WAVES + wave_uniform, BLOCKS_A - 1);
+                load_to_lds(a, off_a[i] + (unsigned)k0 * 2u, lds_a0 + (unsigned)((stage * BM + block * ROWS) * DK * 2));
+            }
 #pragma unroll
-            for (int i = 0; i < LOADS_B; ++i)
-                load_to_lds(w, off_b[i] + (unsigned)k0 * 2u, lds_rows_b + (unsigned)((stage * BN + i * WAVES * ROWS) * DK * 2));
+            for (int i = 0; i < LOADS_B; ++i) {
+                const int block = min(i * WAVES + wave_uniform, BLOCKS_B - 1);
+                load_to_lds(w, off_b[i] + (unsigned)k0 * 2u, lds_b0 + (unsigned)((stage * BN + block * ROWS) * DK * 2));
+            }
         };
         const int swizzle = swizzle_of(lane % 16);                 // of every row this lane reads: they differ by multiples of 32
         // operands of one 16-wide slice of k: TM row blocks of a, TN row blocks of w
@@ -366,28 +372,48 @@ int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hi
 template <int BM, int BN, int WM, int WN, int MODE, typename TO>
 int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
     // Whole tiles along k go straight into LDS; a ragged last tile needs the path through
-    // registers. The large tile fills LDS with four narrow stages and keeps two tiles in flight;
+    // registers. The large tiles fill LDS with four narrow stages and keep two tiles in flight;
     // two workgroups of the small tile share a compute unit and cover each other's waits, and do
     // better with fewer, wider steps.
     if (K % 64 == 0) {
-        if constexpr (BM * BN >= 256 * 256) return launch_kernel<BM, BN, WM, WN, MODE, 32, 4, TO>(a, w, out, M, N, K, s);
+        if constexpr (BM * BN > 128 * 128) return launch_kernel<BM, BN, WM, WN, MODE, 32, 4, TO>(a, w, out, M, N, K, s);
         else return launch_kernel<BM, BN, WM, WN, MODE, 64, 2, TO>(a, w, out, M, N, K, s);
     }
-    return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, s);
+    if constexpr (BN % 128 != 0) {
+        XRT_REQUIRE(false, "linear (mfma): the 192-wide tile takes only K that is a multiple of 64 (K=%d)", K);
+    } else {
+        return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, s);
+    }
+}
+
+// Time of a product with BM x BN tiles, in units of tile elements per compute unit: the tiles
+// run in rounds over the 256 compute units (`share` workgroups of that tile fit one unit and
+// share its matrix cores), and a partly filled last round costs a whole one. `penalty` is what a
+// tile shape loses against the largest, in percent, from reading its operands more often.
+long rounds_cost(long tiles, int tile_elements, int share, int penalty) {
+    const long rounds = (tiles + 256L * share - 1) / (256L * share);
+    return rounds * share * tile_elements * (100 + penalty) / 100;
+}
+
+template <int MODE, typename TO>
+int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+    // output columns per tile are half the tile's w rows in the gated mode
+    constexpr int DIV = MODE == MODE_GATED ? 2 : 1;
+    auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn / DIV - 1) / (bn / DIV)); };
+    const long large = rounds_cost(tiles(256, 256), 256 * 256, 1, 0);
+    const long medium = K % 64 == 0 && MODE != MODE_GATED ? rounds_cost(tiles(256, 192), 256 * 192, 1, 5) : LONG_MAX;
+    const long small = rounds_cost(tiles(128, 128), 128 * 128, 2, 18);
+    if (large <= medium && large <= small) return launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, s);
+    if constexpr (MODE != MODE_GATED)
+        if (medium <= small) return launch<256, 192, 4, 2, MODE, TO>(a, w, out, M, N, K, s);
+    return launch<128, 128, 2, 2, MODE, TO>(a, w, out, M, N, K, s);
 }
 
 template <typename TO>
 int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, hipStream_t s) {
-    // large tiles when they still fill the chip's 256 compute units, else smaller ones
-    const long big_tiles = (long)((M + 255) / 256) * ((N + 255) / 256);
-    const bool big = big_tiles >= 192;
-    if (mode == MODE_STORE) return big ? launch<256, 256, 2, 4, MODE_STORE, TO>(a, w, out, M, N, K, s)
-                                       : launch<128, 128, 2, 2, MODE_STORE, TO>(a, w, out, M, N, K, s);
-    if (mode == MODE_ACCUMULATE) return big ? launch<256, 256, 2, 4, MODE_ACCUMULATE, TO>(a, w, out, M, N, K, s)
-                                            : launch<128, 128, 2, 2, MODE_ACCUMULATE, TO>(a, w, out, M, N, K, s);
-    const long big_gated = (long)((M + 255) / 256) * ((N + 127) / 128);
-    return big_gated >= 192 ? launch<256, 256, 2, 4, MODE_GATED, TO>(a, w, out, M, N, K, s)
-                            : launch<128, 128, 2, 2, MODE_GATED, TO>(a, w, out, M, N, K, s);
+    if (mode == MODE_STORE) return launch_mode<MODE_STORE, TO>(a, w, out, M, N, K, s);
+    if (mode == MODE_ACCUMULATE) return launch_mode<MODE_ACCUMULATE, TO>(a, w, out, M, N, K, s);
+    return launch_mode<MODE_GATED, TO>(a, w, out, M, N, K, s);
 }
 
 }  // namespace
