@@ -7,8 +7,10 @@
 // key/value head h / group), computed with the running maximum and sum of its decode loop
 // (:514-574) instead of a stored row of scores.
 //
-// A workgroup owns 256 consecutive query tokens of one sequence and one head: eight wavefronts
-// with 32 queries each (two per SIMD, so that one can do its softmax while the other multiplies). It walks the sequence's cache blocks (64 keys) in order; every block
+// A workgroup owns 256 (or 128) consecutive query tokens of one sequence and one head: eight (or
+// four) wavefronts with 32 queries each; a compute unit then holds eight wavefronts, two per
+// SIMD, so that one can do its softmax while the other multiplies. The workgroup walks the
+// sequence's cache blocks (64 keys) in order; every block
 // travels once from global memory into LDS (keys as they lie, values transposed as they lie),
 // the next block while the current one is used, and all wavefronts read their operands
 // from there. Everything is kept transposed so that one lane owns one query:
@@ -27,9 +29,7 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int WAVES = 8;
 constexpr int QT = 32;                 // query tokens per wavefront
-constexpr int QW = WAVES * QT;         // query tokens per workgroup
 constexpr int BT = XRT_BLOCK_TOKENS;   // keys per cache block
 constexpr float LOG2E = 1.4426950408889634f;
 
@@ -37,12 +37,14 @@ constexpr float LOG2E = 1.4426950408889634f;
 // register i of lane half h is row (i/4)*8 + h*4 + i%4 and must be key (i/8)*16 + h*8 + i%8.
 __device__ __forceinline__ int key_of_row(int r) { return (r / 16) * 16 + ((r % 8) / 4) * 8 + ((r / 8) % 2) * 4 + r % 4; }
 
-template <int HD>
+// WAVES wavefronts of 32 queries each share the cache blocks that the workgroup moves through LDS.
+template <int HD, int WAVES>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     const bf16* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads,
     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ seq_offsets, const int* __restrict__ seq_slots,
     const int* __restrict__ seq_starts, int n_seqs, bf16* __restrict__ out, float scale) {
+    constexpr int QW = WAVES * QT;         // query tokens per workgroup
     constexpr int KS = HD / 16;            // K steps of the score product
     constexpr int DT = HD / 32;            // 32-row tiles of the value product
     constexpr int KP = HD + 8;             // LDS pitch of a key row
@@ -54,11 +56,12 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 
     const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
     const int col = lane % 32, half = lane / 32;
-    const int head = blockIdx.y;
+    const int head = blockIdx.x;
 
-    // which sequence and which of its query tiles this workgroup has; the grid is walked backwards,
-    // so that the tiles with the most keys before them (the last of a sequence) start first
-    int tile = gridDim.x - 1 - blockIdx.x, seq = 0, count = 0;
+    // which sequence and which of its query tiles this workgroup has; tiles are walked backwards
+    // and heads change fastest, so that the tiles with the most keys before them (the last of a
+    // sequence) start first, for all heads
+    int tile = gridDim.y - 1 - blockIdx.y, seq = 0, count = 0;
     for (; seq < n_seqs; ++seq) {
         count = seq_offsets[seq + 1] - seq_offsets[seq];
         const int tiles = (count + QW - 1) / QW;
@@ -137,30 +140,36 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 
         // register i is key k0 + (i/8)*16 + half*8 + i%8, for this lane's query
         const bool edge = k0 + 31 > first_masked;            // some key of the tile may lie beyond some query
-        float tile_max = -INFINITY;
+        float tile_max = -INFINITY;                          // of the raw products: the scale is positive
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int key = k0 + (i / 8) * 16 + half * 8 + i % 8;
-            float v = s[i] * scale2;
-            if (edge && key > q_pos) v = -INFINITY;           // causal: keys after the query do not exist for it
-            s[i] = v;
-            tile_max = fmaxf(tile_max, v);
+            if (edge && key > q_pos) s[i] = -INFINITY;        // causal: keys after the query do not exist for it
+            tile_max = fmaxf(tile_max, s[i]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, XRT_WAVE));
-        const float m_new = fmaxf(m, tile_max);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // a query that sees none of these keys yet
-        const float correction = __builtin_amdgcn_exp2f(m - m_safe);
-        m = m_new;
-        l *= correction;
+        // m is the exponent that the sums so far are relative to: the largest score seen when it was
+        // last moved, not necessarily the largest seen. It moves, and the sums are scaled down,
+        // only when some query of the wavefront meets a score more than 8 (in log2) above its m;
+        // until then the probabilities are at most 2^8 and the quotient at the end is the same.
+        // After the first tiles that is rare.
+        const float tile_top = tile_max * scale2;
+        if (__builtin_amdgcn_ballot_w64(tile_top > m + 8.0f) != 0) {
+            const float m_new = fmaxf(m, tile_top);
+            const float correction = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.f : m_new));
+            l *= correction;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) o[dt][e] *= correction;
+                for (int e = 0; e < 16; ++e) o[dt][e] *= correction;
+            m = m_new;
+        }
+        const float m_safe = m == -INFINITY ? 0.f : m;        // a query that sees none of these keys yet
 
         bf16x8 p[2];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float e = __builtin_amdgcn_exp2f(s[i] - m_safe);
+            const float e = __builtin_amdgcn_exp2f(fmaf(s[i], scale2, -m_safe));
             l += e;
             p[i / 8][i % 8] = (bf16)e;
         }
@@ -215,28 +224,41 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     }
 }
 
-template <int HD>
-int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
-           const int* block_table, int table_stride, int n_blocks, const int* seq_offsets, const int* seq_slots,
-           const int* seq_starts, int n_seqs, bf16* out, float scale, hipStream_t s) {
+template <int HD, int WAVES>
+int launch_waves(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
+                 const int* block_table, int table_stride, int n_blocks, const int* seq_offsets, const int* seq_slots,
+                 const int* seq_starts, int n_seqs, bf16* out, float scale, hipStream_t s) {
+    constexpr int QW = WAVES * QT;
     const int row_width = (n_heads + 2 * n_kv_heads) * HD;
-    // every sequence has at most ceil(count/256) tiles; their sum is at most tokens/256 + n_seqs
+    // every sequence has at most ceil(count / QW) tiles; their sum is at most tokens / QW + n_seqs
     const long tiles = (tokens + QW - 1) / QW + n_seqs;
-    XRT_REQUIRE(n_heads <= 65535, "attention (prefill): too many heads for the grid");
-    const dim3 grid((unsigned)tiles, n_heads);
+    XRT_REQUIRE(tiles <= 65535, "attention (prefill): too many query tiles for the grid");
+    const dim3 grid(n_heads, (unsigned)tiles);
     constexpr size_t lds = (size_t)2 * (BT * (HD + 8) + HD * (BT + 8)) * sizeof(bf16);
-    static bool configured = false;          // per head size
+    static bool configured = false;          // per instantiation
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD, WAVES>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         XRT_REQUIRE(e == hipSuccess, "attention (prefill): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
         configured = true;
     }
-    attention_prefill_kernel<HD><<<grid, WAVES * XRT_WAVE, lds, s>>>(
+    attention_prefill_kernel<HD, WAVES><<<grid, WAVES * XRT_WAVE, lds, s>>>(
         qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, seq_offsets,
         seq_slots, seq_starts, n_seqs, out, scale);
     XRT_LAUNCH_CHECK("attention (prefill)");
     return 0;
+}
+
+template <int HD>
+int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
+           const int* block_table, int table_stride, int n_blocks, const int* seq_offsets, const int* seq_slots,
+           const int* seq_starts, int n_seqs, bf16* out, float scale, hipStream_t s) {
+    // Tiles of 128 queries (four wavefronts, two workgroups to a compute unit) would spread the
+    // uneven work of causal tiles better, but were measured slower at 2048 tokens (121 against
+    // 101 us): every workgroup moves all its cache blocks through LDS, and with half the
+    // wavefronts per block that work doubles.
+    return launch_waves<HD, 8>(qkv, tokens, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks,
+                               seq_offsets, seq_slots, seq_starts, n_seqs, out, scale, s);
 }
 
 }  // namespace
