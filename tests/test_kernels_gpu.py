@@ -186,6 +186,35 @@ def test_qkv_prepare(ops, dtype, nh, nkv, hd, rope_dim):
         assert int((kv_got.k != 0).any(-1).sum()) == 8 * nkv      # eight tokens cached, padding not
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,rope_dim", [(4, 2, 128, 128), (3, 3, 64, 64), (2, 1, 256, 256), (4, 2, 48, 48),
+                                                (4, 2, 64, 16)])
+def test_qkv_prepare_of_many_tokens(ops, dtype, nh, nkv, hd, rope_dim):
+    """A prefill step: three sequences, one of which continues in the middle of a cache block, one padding
+    token between them; the values reach their transposed blocks through the kernel that turns tiles."""
+    runs = [(0, 0, 70), (1, 37, 100), (-1, 0, 1), (2, 64, 30)]          # slot, first position, tokens
+    slots = [slot for slot, _, count in runs for _ in range(count)]
+    positions = [first + i for _, first, count in runs for i in range(count)]
+    tokens = len(slots)
+    qkv = rand(tokens, (nh + 2 * nkv) * hd, dtype=DT[dtype], seed=hd + 1)
+    kv = make_cache(40, nkv, hd, DT[dtype], 3, 4)
+    kv.block_table[0, :4] = i32([7, 3, 11, 2])
+    kv.block_table[1, :4] = i32([30, 31, 5, 6])
+    kv.block_table[2, :4] = i32([20, 19, 18, 17])
+    theta = (torch.tensor(10000.0) ** (torch.arange(rope_dim // 2) * 2.0 / rope_dim)).to(DEV)
+    qn, kn = rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0
+    got, want = qkv.clone(), qkv.clone()
+    kv_got, kv_want = clone_cache(kv), clone_cache(kv)
+    args = dict(q_norm=qn, k_norm=kn, norm_eps=1e-4, rope_theta=theta, rope_dim=rope_dim, rope_scale=1.0)
+    ops.qkv_prepare(got, nh, nkv, hd, i32(positions), i32(slots), kv=kv_got, **args)
+    REF.qkv_prepare(want, nh, nkv, hd, i32(positions), i32(slots), kv=kv_want, **args)
+    tol = 3e-5 if dtype == "float32" else ULP[dtype]
+    assert rel(got.float(), want.float()) < tol
+    assert rel(kv_got.k.float(), kv_want.k.float()) < tol
+    assert torch.equal(kv_got.v, kv_want.v)
+    assert int((kv_got.k != 0).any(-1).sum()) == (tokens - 1) * nkv
+
+
 def test_rope_reference_vector_and_pairing(ops):
     # tests/kernels_test.rs:94-108: one head of 4, position 2, base 1e4 -> pairs (0,2), (1,3)
     qkv = torch.zeros(1, 3 * 16, device=DEV)
