@@ -54,7 +54,7 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int tiles_m, int tiles_n) {
+    int tiles_m, int tiles_n, int n_first) {
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr int WAVE_M = BM / WM, WAVE_N = BN / WN;        // part of the tile owned by one wavefront
     constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;        // 32x32 accumulator tiles of a wavefront
@@ -84,7 +84,7 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     const int tile_m = in_panel / panel_width;
     const long m0 = (long)tile_m * BM;
     constexpr int BN_OUT = MODE == MODE_GATED ? BN / 2 : BN;          // output columns of a tile
-    const long n0 = (long)tile_n * BN_OUT;
+    const long n0 = n_first + (long)tile_n * BN_OUT;      // this launch covers output columns from n_first on
 
     const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
     const int wave_m = wave / WN, wave_n = wave % WN;
@@ -347,8 +347,9 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     }
 }
 
+// Launches the tiles of output columns [n_first, n_first + n_count).
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
-int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, hipStream_t s) {
     constexpr int BN_OUT = MODE == MODE_GATED ? BN / 2 : BN;
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr size_t staging = DK != 0 ? (size_t)STAGES * (BM + BN) * DK * sizeof(bf16) : (size_t)2 * (BM + BN) * PITCH * sizeof(bf16);
@@ -361,32 +362,34 @@ int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hi
         XRT_REQUIRE(e == hipSuccess, "linear (mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
         configured = true;
     }
-    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN_OUT - 1) / BN_OUT;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (n_count + BN_OUT - 1) / BN_OUT;
     const int total = tiles_m * tiles_n;
     const unsigned grid = (unsigned)(((total + 7) / 8) * 8);           // a whole number of rounds over the XCDs
-    kernel<<<grid, THREADS, lds, s>>>(a, w, out, M, N, K, tiles_m, tiles_n);
+    kernel<<<grid, THREADS, lds, s>>>(a, w, out, M, N, K, tiles_m, tiles_n, n_first);
     XRT_LAUNCH_CHECK("linear (mfma)");
     return 0;
 }
 
 template <int BM, int BN, int WM, int WN, int MODE, typename TO>
-int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, hipStream_t s) {
     // Whole tiles along k go straight into LDS; a ragged last tile needs the path through
     // registers. The large tiles fill LDS with four narrow stages and keep two tiles in flight;
     // two workgroups of the small tile share a compute unit and cover each other's waits, and do
     // better with fewer, wider steps.
     if (K % 64 == 0) {
-        if constexpr (BM * BN > 128 * 128) return launch_kernel<BM, BN, WM, WN, MODE, 32, 4, TO>(a, w, out, M, N, K, s);
-        else return launch_kernel<BM, BN, WM, WN, MODE, 64, 2, TO>(a, w, out, M, N, K, s);
+        if constexpr (BM * BN > 128 * 128)
+            return launch_kernel<BM, BN, WM, WN, MODE, 32, 4, TO>(a, w, out, M, N, K, n_first, n_count, s);
+        else
+            return launch_kernel<BM, BN, WM, WN, MODE, 64, 2, TO>(a, w, out, M, N, K, n_first, n_count, s);
     }
-    if constexpr (BN % 128 != 0) {
-        XRT_REQUIRE(false, "linear (mfma): the 192-wide tile takes only K that is a multiple of 64 (K=%d)", K);
+    if constexpr (BM == 256 && BN == 256 || BM == 128 && BN == 128) {
+        return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, n_first, n_count, s);
     } else {
-        return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, s);
+        XRT_REQUIRE(false, "linear (mfma): this tile takes only K that is a multiple of 64 (K=%d)", K);
     }
 }
 
-// Time of a product with BM x BN tiles, in units of tile elements per compute unit: the tiles
+// Time of tiles of `tile_elements` outputs, in units of tile elements per compute unit: the tiles
 // run in rounds over the 256 compute units (`share` workgroups of that tile fit one unit and
 // share its matrix cores), and a partly filled last round costs a whole one. `penalty` is what a
 // tile shape loses against the largest, in percent, from reading its operands more often.
@@ -400,13 +403,29 @@ int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipS
     // output columns per tile are half the tile's w rows in the gated mode
     constexpr int DIV = MODE == MODE_GATED ? 2 : 1;
     auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn / DIV - 1) / (bn / DIV)); };
+    const bool whole_k = K % 64 == 0;
     const long large = rounds_cost(tiles(256, 256), 256 * 256, 1, 0);
-    const long medium = K % 64 == 0 && MODE != MODE_GATED ? rounds_cost(tiles(256, 192), 256 * 192, 1, 5) : LONG_MAX;
+    const long medium = whole_k && MODE != MODE_GATED ? rounds_cost(tiles(256, 192), 256 * 192, 1, 5) : LONG_MAX;
     const long small = rounds_cost(tiles(128, 128), 128 * 128, 2, 18);
-    if (large <= medium && large <= small) return launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, s);
+    // Large tiles for as many columns as make whole rounds, and tiles of half the height for the
+    // rest, if those then fit one round: the last round is full of half-sized work instead of
+    // half empty.
+    const int tiles_m = (M + 255) / 256, tiles_n = (N + 256 / DIV - 1) / (256 / DIV);
+    const int whole_columns = (int)((long)tiles_m * tiles_n / 256 * 256 / tiles_m);     // n-tiles that run in full rounds
+    const long rest_tiles = (long)((M + 127) / 128) * (tiles_n - whole_columns);
+    long mixed = LONG_MAX;
+    if (whole_k && whole_columns > 0 && whole_columns < tiles_n && rest_tiles <= 256)
+        mixed = rounds_cost((long)tiles_m * whole_columns, 256 * 256, 1, 0) + rounds_cost(rest_tiles, 128 * 256, 1, 8);
+    if (mixed < large && mixed <= medium && mixed <= small) {
+        const int split = whole_columns * (256 / DIV);
+        const int status = launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, 0, split, s);
+        if (status != 0) return status;
+        return launch<128, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, split, N - split, s);
+    }
+    if (large <= medium && large <= small) return launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, 0, N, s);
     if constexpr (MODE != MODE_GATED)
-        if (medium <= small) return launch<256, 192, 4, 2, MODE, TO>(a, w, out, M, N, K, s);
-    return launch<128, 128, 2, 2, MODE, TO>(a, w, out, M, N, K, s);
+        if (medium <= small) return launch<256, 192, 4, 2, MODE, TO>(a, w, out, M, N, K, 0, N, s);
+    return launch<128, 128, 2, 2, MODE, TO>(a, w, out, M, N, K, 0, N, s);
 }
 
 template <typename TO>
