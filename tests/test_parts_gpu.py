@@ -153,7 +153,7 @@ def define_toy():
     from dataclasses import dataclass
     from xeno_rt_amd.config import register_architecture
     from xeno_rt_amd.models import LayerCall, ModelSpec
-    from xeno_rt_amd.parts import (Attention, CacheNeeds, Embedding, GatedMLP, Mixer, OutputHead,
+    from xeno_rt_amd.parts import (Attention, CacheNeeds, Embedding, FeedForward, GatedMLP, Mixer, OutputHead,
                                    PositionEncoding, PreNormBlock, RMSNorm, StateSpec, WeightSpec,
                                    register_part)
 
@@ -200,8 +200,41 @@ def define_toy():
             for head in range(n_heads + n_kv_heads):
                 qkv[:, head * head_dim] += bump
 
+    class MixtureMLP(FeedForward):
+        """Several gated MLPs, each weighted by the softmax of a router's logits (float32): a
+        feed-forward made of the framework's own part, several times, behind a router. Every expert
+        gets every token, so that a rounding error cannot flip a choice and the comparison with
+        the plain model stays one of tolerances."""
+
+        def __init__(self, prefix, hidden, inner, experts, sharpness):
+            self.prefix, self.hidden, self.sharpness = prefix, hidden, sharpness
+            self.experts = [GatedMLP(f"{prefix}experts.{e}.", hidden, inner) for e in range(experts)]
+
+        def weight_specs(self):
+            specs = {self.prefix + "router.weight": WeightSpec((len(self.experts), self.hidden))}
+            for expert in self.experts:
+                specs.update(expert.weight_specs())
+            return specs
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.router = runtime.matrix(tensors[self.prefix + "router.weight"])
+            for expert in self.experts:
+                expert.bind(tensors, runtime)
+
+        def forward(self, h, batch, residual):
+            rt = self.runtime
+            logits = rt.empty((h.shape[0], len(self.experts)), torch.float32)
+            rt.ops.linear(h, self.router, logits)
+            weights = torch.softmax(logits * self.sharpness, dim=-1)
+            for e, expert in enumerate(self.experts):
+                share = torch.zeros_like(residual)
+                expert.forward(h, batch, share)
+                residual.addcmul_(share, weights[:, e:e + 1])
+
     register_part("mixer", "toy_decay", DecayMixer)
     register_part("position", "toy_shift", ShiftPosition)
+    register_part("feed_forward", "toy_mixture", MixtureMLP)
 
     @dataclass(frozen=True)
     class ToyConfig:
@@ -236,8 +269,10 @@ def define_toy():
                                                    position=create_part("position", "toy_shift", step=0.01)),
                          norm("l1.n2."), GatedMLP("l1.mlp.", h, 2 * h + 8)),
             # layer 2: attention without position encoding, reading the cache of the first call of layer 1
+            # ... and with a feed-forward of three experts behind a router
             PreNormBlock(norm("l2.n1."), Attention("l2.attn.", h, 4, 2, 16, qk_norm=True, qk_norm_eps=1e-5),
-                         norm("l2.n2."), GatedMLP("l2.mlp.", h, 2 * h + 8)),
+                         norm("l2.n2."), create_part("feed_forward", "toy_mixture", prefix="l2.moe.", hidden=h,
+                                                     inner=h + 24, experts=3, sharpness=4.0)),
         ]
         emb = Embedding("emb.", c.vocab_size, h)
         schedule = [LayerCall(0), LayerCall(1), LayerCall(1), LayerCall(2, reads_cache_of=1)]
@@ -288,7 +323,9 @@ def plain_toy(w, config, ids):
     # layer 2 reads the keys and values that the first call of layer 1 cached
     out, _ = attend("l2.attn.", P.rmsnorm(x, w["l2.n1.weight"], 1e-5), 0.0, shared=first_kv)
     x = x + out
-    x = x + mlp("l2.mlp.", P.rmsnorm(x, w["l2.n2.weight"], 1e-5))
+    y = P.rmsnorm(x, w["l2.n2.weight"], 1e-5)
+    share = torch.softmax(P.linear(y, w["l2.moe.router.weight"]) * 4.0, dim=-1)
+    x = x + sum(share[:, e:e + 1] * mlp(f"l2.moe.experts.{e}.", y) for e in range(3))
     return P.linear(P.rmsnorm(x, w["final.weight"], 1e-5), w["head.weight"])
 
 
