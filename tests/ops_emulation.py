@@ -53,7 +53,7 @@ class EmulatedOps:
     # -- attention --------------------------------------------------------------
     def qkv_prepare(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots,
                     q_norm=None, k_norm=None, norm_eps=0.0, rope_theta=None, rope_dim=0,
-                    rope_scale=1.0, kv=None):
+                    rope_scale=1.0, kv=None, longest_run=0):
         tokens = qkv.shape[0]
         qw, kw = n_heads * head_dim, n_kv_heads * head_dim
         work = qkv.to(torch.float32)

@@ -207,7 +207,7 @@ def test_qkv_prepare_of_many_tokens(ops, dtype, nh, nkv, hd, rope_dim):
     got, want = qkv.clone(), qkv.clone()
     kv_got, kv_want = clone_cache(kv), clone_cache(kv)
     args = dict(q_norm=qn, k_norm=kn, norm_eps=1e-4, rope_theta=theta, rope_dim=rope_dim, rope_scale=1.0)
-    ops.qkv_prepare(got, nh, nkv, hd, i32(positions), i32(slots), kv=kv_got, **args)
+    ops.qkv_prepare(got, nh, nkv, hd, i32(positions), i32(slots), kv=kv_got, longest_run=100, **args)
     REF.qkv_prepare(want, nh, nkv, hd, i32(positions), i32(slots), kv=kv_want, **args)
     tol = 3e-5 if dtype == "float32" else ULP[dtype]
     assert rel(got.float(), want.float()) < tol

@@ -246,7 +246,7 @@ extern "C" int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, in
                                const int* positions, const int* slots, const void* q_norm, const void* k_norm,
                                int norm_dtype, float norm_eps, const float* rope_theta, int rope_dim,
                                float rope_scale, void* k_cache, void* v_cache, const int* block_table,
-                               int table_stride, int n_blocks, void* stream) {
+                               int table_stride, int n_blocks, int longest_run, void* stream) {
     XRT_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0, "qkv_prepare: bad head counts %d/%d", n_heads, n_kv_heads);
     XRT_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= MAX_HEAD_DIM,
                 "qkv_prepare: head_dim %d must be even and at most %d", head_dim, MAX_HEAD_DIM);
@@ -268,8 +268,9 @@ extern "C" int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, in
                         (rope_theta == nullptr || rope_dim == head_dim) && (uintptr_t)qkv % 16 == 0 &&
                         (k_cache == nullptr || ((uintptr_t)k_cache % 16 == 0));
     if (vector) {
-        // many tokens: their values go through the transposing kernel; few: element by element from this one
-        const bool values_apart = v_cache != nullptr && tokens >= XRT_WAVE;
+        // sequences that bring many tokens: their values go through the transposing kernel;
+        // otherwise element by element from this one
+        const bool values_apart = v_cache != nullptr && longest_run >= XRT_WAVE / 2;
         const unsigned grid = (unsigned)tokens;
 #define XRT_VEC(T, TW, L)                                                                                  \
     qkv_prepare_vector_kernel<T, TW, L><<<grid, WAVES * XRT_WAVE, 0, s>>>(                                 \

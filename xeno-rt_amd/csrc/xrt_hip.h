@@ -26,13 +26,15 @@ int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype
                int mode, void* stream);
 
 // per-head RMSNorm of q and k (optional), rotation of q and k (optional), write of k and v
-// into the cache (optional); qkv rows are [q heads | k heads | v heads]
+// into the cache (optional); qkv rows are [q heads | k heads | v heads]. longest_run: the most
+// consecutive tokens that one sequence brings (0 if unknown); it only picks the faster way to
+// write the values
 int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                     const int* positions, const int* slots,
                     const void* q_norm, const void* k_norm, int norm_dtype, float norm_eps,
                     const float* rope_theta, int rope_dim, float rope_scale,
                     void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks,
-                    void* stream);
+                    int longest_run, void* stream);
 
 // causal attention of every token of a step over its sequence's cache. The sequences of the
 // step may be described (seq_* arrays, n_seqs, the largest token count of a sequence and the

@@ -132,7 +132,7 @@ class HipOps:
         self._linear(a, w_gate_up, out, 2, w_gate_up.shape[0] // 2)
 
     def qkv_prepare(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm=None, k_norm=None,
-                    norm_eps=0.0, rope_theta=None, rope_dim=0, rope_scale=1.0, kv=None):
+                    norm_eps=0.0, rope_theta=None, rope_dim=0, rope_scale=1.0, kv=None, longest_run=0):
         tokens = qkv.shape[0]
         width = (n_heads + 2 * n_kv_heads) * head_dim
         self._require(qkv, "qkv", None, (tokens, width))
@@ -155,7 +155,7 @@ class HipOps:
             _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(positions), _ptr(slots),
             _ptr(q_norm), _ptr(k_norm), norm_code, ctypes.c_float(norm_eps), _ptr(rope_theta), int(rope_dim),
             ctypes.c_float(rope_scale), _ptr(k_cache), _ptr(v_cache), _ptr(table), stride, n_blocks,
-            self._stream(qkv)))
+            int(longest_run), self._stream(qkv)))
 
     def _kv(self, kv, like, n_kv_heads, head_dim):
         from ..cache import BLOCK_TOKENS

@@ -92,6 +92,7 @@ class Attention(Mixer):
 
         dims = (self.n_heads, self.n_kv_heads, self.head_dim)
         write_to = kv if cache.writable else None
+        longest_run = int(getattr(batch, "max_count", 0) or 0)      # picks how the values are written; 0: unknown
         rotary = self.position if isinstance(self.position, Rotary) else None
         if rotary is not None or self.position is None:
             # one pass: head norms, rotation, cache write
@@ -100,7 +101,7 @@ class Attention(Mixer):
                             rope_theta=None if rotary is None else rotary.theta,
                             rope_dim=0 if rotary is None else rotary.rope_dim,
                             rope_scale=1.0 if rotary is None else rotary.scale,
-                            kv=write_to)
+                            kv=write_to, longest_run=longest_run)
         else:
             # any other position encoding: norms, then the encoding, then the cache write
             if self.qk_norm:
@@ -108,7 +109,7 @@ class Attention(Mixer):
                                 q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.qk_norm_eps)
             self.position.apply(qkv, *dims, batch)
             if write_to is not None:
-                ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots, kv=write_to)
+                ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots, kv=write_to, longest_run=longest_run)
 
         out = rt.empty((tokens, self.q_width))
         ops.attention(qkv, *dims, kv, batch, out, scale=self.scale, window=self.window)
