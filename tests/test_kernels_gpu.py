@@ -82,7 +82,7 @@ def test_rmsnorm_reference_vector(ops):
 SHAPES = [(1, 64, 64), (3, 200, 96), (8, 1000, 176), (17, 96, 192), (64, 333, 520), (130, 257, 72),
           (300, 520, 1032), (1, 3, 5), (5, 7, 13), (33, 4100, 264), (64, 40, 4096), (65, 40, 4096),
           (2048, 6144, 128), (2000, 6200, 136), (70, 300, 64), (300, 520, 1024), (2100, 6100, 320),
-          (2100, 8300, 128)]
+          (2100, 8300, 128), (40, 4100, 1024), (64, 333, 640), (33, 130, 128), (17, 700, 192)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -105,7 +105,8 @@ def test_linear(ops, dtype, m, n, k):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("m,n,k", [(1, 176, 64), (9, 100, 96), (64, 520, 200), (200, 1000, 72), (48, 2000, 520),
-                                   (2048, 3100, 64), (300, 130, 1032), (2048, 3072, 128), (2000, 3000, 192), (2048, 4224, 64)])
+                                   (2048, 3100, 64), (300, 130, 1032), (2048, 3072, 128), (2000, 3000, 192), (2048, 4224, 64),
+                                   (64, 520, 256), (50, 1000, 1024)])
 def test_linear_glu(ops, dtype, m, n, k):
     a = rand(m, k, dtype=DT[dtype], seed=1)
     w = rand(2 * n, k, dtype=DT[dtype], seed=2, scale=0.3)

@@ -54,7 +54,7 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int tiles_m, int tiles_n, int n_first) {
+    int tiles_m, int tiles_n, int n_first, int k_per_split) {
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr int WAVE_M = BM / WM, WAVE_N = BN / WN;        // part of the tile owned by one wavefront
     constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;        // 32x32 accumulator tiles of a wavefront
@@ -188,15 +188,19 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
         // after the barrier, under the products of the last slice of this one.
         constexpr int AHEAD = STAGES - 1;
         constexpr int IN_FLIGHT = (AHEAD - 1) * (LOADS_A + LOADS_B);   // loads that may be outstanding when the next tile is needed
-        const int steps = K / DK;
-        const int last_k = (steps - 1) * DK;
+        // a launch with several grid rows splits k among them: row y takes k_per_split from
+        // y * k_per_split on (less at the end) and writes its sums to the y-th copy of out
+        const int k_begin = blockIdx.y * k_per_split;
+        const int steps = min(k_per_split, K - k_begin) / DK;
+        const int last_k = k_begin + (steps - 1) * DK;
+        out += (long)blockIdx.y * M * N;
 #pragma unroll
-        for (int i = 0; i < AHEAD; ++i) issue(i, min(i * DK, last_k));
+        for (int i = 0; i < AHEAD; ++i) issue(i, min(k_begin + i * DK, last_k));
         wait_loads_and_barrier<IN_FLIGHT>();                      // tile 0 is in LDS
         Operands operands[2];
         read(operands[0], 0, 0);
         for (int t = 0; t < steps; ++t) {
-            issue((t + AHEAD) % STAGES, min((t + AHEAD) * DK, last_k));   // that stage was read in step t-1, before the last barrier
+            issue((t + AHEAD) % STAGES, min(k_begin + (t + AHEAD) * DK, last_k));   // that stage was read in step t-1, before the last barrier
 #pragma unroll
             for (int slice = 0; slice + 1 < SLICES; ++slice) {
                 read(operands[(slice + 1) % 2], t % STAGES, slice + 1);
@@ -349,7 +353,8 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
 
 // Launches the tiles of output columns [n_first, n_first + n_count).
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
-int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, hipStream_t s) {
+int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, hipStream_t s,
+                  int splits = 1, int k_per_split = 0) {
     constexpr int BN_OUT = MODE == MODE_GATED ? BN / 2 : BN;
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr size_t staging = DK != 0 ? (size_t)STAGES * (BM + BN) * DK * sizeof(bf16) : (size_t)2 * (BM + BN) * PITCH * sizeof(bf16);
@@ -365,7 +370,9 @@ int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, in
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (n_count + BN_OUT - 1) / BN_OUT;
     const int total = tiles_m * tiles_n;
     const unsigned grid = (unsigned)(((total + 7) / 8) * 8);           // a whole number of rounds over the XCDs
-    kernel<<<grid, THREADS, lds, s>>>(a, w, out, M, N, K, tiles_m, tiles_n, n_first);
+    XRT_REQUIRE(splits == 1 || DK != 0, "linear (mfma): only whole tiles along k can be split");
+    kernel<<<dim3(grid, splits), THREADS, lds, s>>>(a, w, out, M, N, K, tiles_m, tiles_n, n_first,
+                                                    splits == 1 ? K : k_per_split);
     XRT_LAUNCH_CHECK("linear (mfma)");
     return 0;
 }
@@ -435,6 +442,60 @@ int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
     return launch_mode<MODE_GATED, TO>(a, w, out, M, N, K, s);
 }
 
+// ---- 17 to 64 rows of x: too many for the kernel that streams w through registers (it would read
+// x from L2 up to four times as often as w from HBM), too few for the tiles above to fill the chip.
+// Tiles of 64 x 128 take their x through LDS; k is split among workgroups until there are enough
+// of them to pull w at the rate of HBM; each writes float32 sums of its part of k to a workspace,
+// and a second kernel adds the parts in order and applies the epilogue.
+constexpr int SPLIT_BM = 64, SPLIT_BN = 128;
+
+struct SplitPlan { int splits, k_per_split; long rows_w; };
+
+SplitPlan split_plan(int N, int K, int mode) {
+    const long rows_w = mode == MODE_GATED ? 2L * N : N;
+    const long tiles = (rows_w + SPLIT_BN - 1) / SPLIT_BN;
+    const int units = K / 64;                                  // k is dealt out in pieces of 64
+    int splits = (int)((384 + tiles - 1) / tiles);             // about one and a half workgroups per compute unit
+    splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
+    splits = splits > units ? units : splits;
+    const int per = (units + splits - 1) / splits;
+    splits = (units + per - 1) / per;                          // no empty part
+    return SplitPlan{splits, per * 64, rows_w};
+}
+
+template <int MODE, typename TO>
+__global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restrict__ parts, int splits, int M, int N,
+                                                            TO* __restrict__ out) {
+    const long rows_w = MODE == MODE_GATED ? 2L * N : N;
+    const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= (long)M * N) return;
+    const long m = index / N, n = index % N;
+    float sum = 0.f, up = 0.f;
+    for (int p = 0; p < splits; ++p) {
+        const float* part = parts + ((long)p * M + m) * rows_w;
+        sum += part[n];
+        if constexpr (MODE == MODE_GATED) up += part[N + n];
+    }
+    if constexpr (MODE == MODE_STORE) out[index] = from_float<TO>(sum);
+    else if constexpr (MODE == MODE_ACCUMULATE) out[index] = from_float<TO>(to_float(out[index]) + sum);
+    else out[index] = from_float<TO>(silu(sum) * up);
+}
+
+template <typename TO>
+int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, float* workspace, hipStream_t s) {
+    const SplitPlan plan = split_plan(N, K, mode);
+    // the product of all rows of w, ungated, into the workspace: [splits][M][rows_w]
+    const int status = launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 32, 4, float>(
+        a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split);
+    if (status != 0) return status;
+    const unsigned blocks = (unsigned)(((long)M * N + 255) / 256);
+    if (mode == MODE_STORE) split_reduce_kernel<MODE_STORE, TO><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out);
+    else if (mode == MODE_ACCUMULATE) split_reduce_kernel<MODE_ACCUMULATE, TO><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out);
+    else split_reduce_kernel<MODE_GATED, TO><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out);
+    XRT_LAUNCH_CHECK("linear (split reduce)");
+    return 0;
+}
+
 }  // namespace
 
 bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, int mode) {
@@ -446,4 +507,19 @@ int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int 
                     hipStream_t s) {
     if (out_dtype == XRT_F32) return launch_shape<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, s);
     return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, s);
+}
+
+// Floats of workspace with which a product of 17 to 64 rows of x runs split along k; 0 if this
+// product does not take that path.
+long xrt_linear_split_workspace(const void* a, const void* w, int M, int N, int K, int mode) {
+    if (M <= 16 || M > SPLIT_BM || K % 64 != 0 || K < 128 || !xrt_linear_mfma_accepts(a, w, M, N, K, mode)) return 0;
+    const SplitPlan plan = split_plan(N, K, mode);
+    if (plan.rows_w * (long)M >= (1L << 31)) return 0;
+    return (long)plan.splits * M * plan.rows_w;
+}
+
+int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+                     float* workspace, hipStream_t s) {
+    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, workspace, s);
+    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, workspace, s);
 }

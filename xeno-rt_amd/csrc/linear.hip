@@ -11,8 +11,17 @@ bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, 
 int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                     hipStream_t s);
 
+long xrt_linear_split_workspace(const void* a, const void* w, int M, int N, int K, int mode);
+int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+                     float* workspace, hipStream_t s);
+
+extern "C" long xrt_linear_workspace(const void* a, const void* w, int dtype, int M, int N, int K, int mode) {
+    if (dtype != XRT_BF16 || M <= 0 || N <= 0 || K <= 0 || mode < 0 || mode > 2) return 0;
+    return xrt_linear_split_workspace(a, w, M, N, K, mode);
+}
+
 extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N,
-                          int K, int mode, void* stream) {
+                          int K, int mode, float* workspace, long workspace_floats, void* stream) {
     XRT_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
     XRT_REQUIRE(mode >= 0 && mode <= 2, "linear: unknown mode %d", mode);
     XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "linear: unknown dtype %d", dtype);
@@ -22,6 +31,11 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
     XRT_REQUIRE(a && w && out, "linear: null operand");
     if (M == 0) return 0;
     // bfloat16: the matrix-core kernels; float32, and shapes they refuse: the plain kernel
+    if (dtype == XRT_BF16 && workspace != nullptr) {
+        const long need = xrt_linear_split_workspace(a, w, M, N, K, mode);
+        if (need > 0 && workspace_floats >= need)
+            return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, workspace, (hipStream_t)stream);
+    }
     if (dtype == XRT_BF16 && xrt_linear_skinny_accepts(a, w, M, K))
         return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
     if (dtype == XRT_BF16 && xrt_linear_mfma_accepts(a, w, M, N, K, mode))

@@ -59,6 +59,7 @@ class HipOps:
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
                      "xrt_attention", "xrt_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
+        self.lib.xrt_linear_workspace.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
     def _check(self, status: int) -> None:
@@ -120,8 +121,10 @@ class HipOps:
         if w.shape[1] != k:
             raise KernelError(f"linear: a has {k} columns, w has {w.shape[1]}")
         self._require(out, "linear out", None, (m, n), a)
+        need = int(self.lib.xrt_linear_workspace(_ptr(a), _ptr(w), _code(a), m, n, k, mode))
+        workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
         self._check(self.lib.xrt_linear(_ptr(a), _ptr(w), _code(a), _ptr(out), _code(out), m, n, k, mode,
-                                        self._stream(a)))
+                                        _ptr(workspace), ctypes.c_long(need), self._stream(a)))
 
     def linear(self, a, w, out, accumulate=False):
         self._linear(a, w, out, 1 if accumulate else 0, w.shape[0])
