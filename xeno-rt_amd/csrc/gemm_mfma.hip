@@ -447,17 +447,27 @@ int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
 // Tiles of 64 x 128 take their x through LDS; k is split among workgroups until there are enough
 // of them to pull w at the rate of HBM; each writes float32 sums of its part of k to a workspace,
 // and a second kernel adds the parts in order and applies the epilogue.
+// With more rows of x (up to a few hundred) the tiles of 128 x 128 do the same when they are too
+// few to fill the chip: such products are still bound by reading w.
 constexpr int SPLIT_BM = 64, SPLIT_BN = 128;
 
 struct SplitPlan { int splits, k_per_split; long rows_w; };
 
-SplitPlan split_plan(int N, int K, int mode) {
+SplitPlan split_plan(int M, int N, int K, int mode) {
     const long rows_w = mode == MODE_GATED ? 2L * N : N;
-    const long tiles = (rows_w + SPLIT_BN - 1) / SPLIT_BN;
+    const long tiles_n = (rows_w + SPLIT_BN - 1) / SPLIT_BN;
     const int units = K / 64;                                  // k is dealt out in pieces of 64
-    int splits = (int)((384 + tiles - 1) / tiles);             // about one and a half workgroups per compute unit
+    int splits, least;                                         // least: pieces of k that a part should have
+    if (M <= SPLIT_BM) {
+        splits = (int)((384 + tiles_n - 1) / tiles_n);         // about one and a half workgroups per compute unit
+        least = 1;
+    } else {
+        const long tiles = (long)((M + 127) / 128) * tiles_n;  // two of these workgroups share a compute unit
+        splits = tiles >= 384 ? 1 : (int)((512 + tiles - 1) / tiles);
+        least = 4;
+    }
     splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
-    splits = splits > units ? units : splits;
+    splits = splits > units / least ? (units / least < 1 ? 1 : units / least) : splits;
     const int per = (units + splits - 1) / splits;
     splits = (units + per - 1) / per;                          // no empty part
     return SplitPlan{splits, per * 64, rows_w};
@@ -483,10 +493,13 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restri
 
 template <typename TO>
 int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, float* workspace, hipStream_t s) {
-    const SplitPlan plan = split_plan(N, K, mode);
+    const SplitPlan plan = split_plan(M, N, K, mode);
     // the product of all rows of w, ungated, into the workspace: [splits][M][rows_w]
-    const int status = launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 32, 4, float>(
-        a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split);
+    const int status = M <= SPLIT_BM
+        ? launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 32, 4, float>(
+              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split)
+        : launch_kernel<128, 128, 2, 2, MODE_STORE, 64, 2, float>(
+              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split);
     if (status != 0) return status;
     const unsigned blocks = (unsigned)(((long)M * N + 255) / 256);
     if (mode == MODE_STORE) split_reduce_kernel<MODE_STORE, TO><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out);
@@ -509,11 +522,12 @@ int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int 
     return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, s);
 }
 
-// Floats of workspace with which a product of 17 to 64 rows of x runs split along k; 0 if this
-// product does not take that path.
+// Floats of workspace with which a product runs split along k (17 to 64 rows of x, or more rows
+// and few tiles); 0 if this product does not take that path.
 long xrt_linear_split_workspace(const void* a, const void* w, int M, int N, int K, int mode) {
-    if (M <= 16 || M > SPLIT_BM || K % 64 != 0 || K < 128 || !xrt_linear_mfma_accepts(a, w, M, N, K, mode)) return 0;
-    const SplitPlan plan = split_plan(N, K, mode);
+    if (M <= 16 || K % 64 != 0 || K < 128 || !xrt_linear_mfma_accepts(a, w, M, N, K, mode)) return 0;
+    const SplitPlan plan = split_plan(M, N, K, mode);
+    if (M > SPLIT_BM && plan.splits == 1) return 0;            // enough tiles without a split: the kernels above
     if (plan.rows_w * (long)M >= (1L << 31)) return 0;
     return (long)plan.splits * M * plan.rows_w;
 }

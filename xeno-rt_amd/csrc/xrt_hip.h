@@ -22,7 +22,7 @@ int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype, float eps,
 
 // out[m, n] (+)= sum_k a[m, k] * w[n, k]   (mode 0 store, 1 accumulate into float32 out,
 // 2 gated: out[m, n] = silu(a.w[n]) * (a.w[n + N]) with w of 2N rows)
-// Some products (17 to 64 rows of a) run faster split along k, through a workspace of float32
+// Some products (17 to 64 rows of a, or more rows and a narrow w) run faster split along k, through a workspace of float32
 // sums: xrt_linear_workspace says how many floats that takes (0: none); without it the product
 // takes another kernel.
 int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
