@@ -210,3 +210,14 @@ def test_python_entry_point_on_the_cpu_stand_in(pair):
     seen = []
     assert session.generate_stream(request, seen.append).tokens == want and seen == want
     session.reset()
+
+
+def test_engine_conveniences(pair):
+    engine, plain = pair
+    prompts = [[4, 8, 15], [42, 7]]
+    got = engine.generate(prompts, max_tokens=4, stop_ids=[])           # greedy unless told otherwise
+    assert got == [P.generate_greedy(plain, p, 4, stop_ids=[]) for p in prompts]
+    table = engine.get_tensor("model.embed_tokens.weight")
+    assert table.device.type == "cpu" and tuple(table.shape) == (engine.config.vocab_size, engine.config.hidden_size)
+    with pytest.raises(KeyError):
+        engine.get_tensor("model.no_such.weight")

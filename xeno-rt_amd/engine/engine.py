@@ -52,6 +52,7 @@ class Engine:
         self.ops = ops
         self.runtime = Runtime(ops, self.dtype, self.device)
         self.config = spec.config
+        self.tensors = tensors          # by checkpoint name, as loaded (or made on demand): see get_tensor
         self.model = DecoderModel(spec, tensors, self.runtime)
         model_context = getattr(spec.config, "max_position_embeddings", None)
         limit = max_context if max_context is not None else model_context
@@ -107,6 +108,26 @@ class Engine:
     @property
     def max_context(self) -> int:
         return self.cache.max_context
+
+    # -- conveniences ------------------------------------------------------------
+    def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 128, temperature: float = 0.0,
+                 top_k: int = 0, top_p: float = 1.0, repetition_penalty: float = 1.0, seed: Optional[int] = 0,
+                 stop_ids: Optional[Sequence[int]] = None, batch_size: Optional[int] = None) -> List[List[int]]:
+        """The generated token ids of every prompt, with one set of sampling options for all
+        (greedy unless told otherwise). `generate()` of this package takes a request per prompt
+        with options of its own and returns finish reasons and timings as well."""
+        from .generate import GenerateRequest, generate
+        requests = [GenerateRequest(list(ids), max_tokens=max_tokens, temperature=temperature, top_k=top_k,
+                                    top_p=top_p, repetition_penalty=repetition_penalty, seed=seed,
+                                    stop_ids=None if stop_ids is None else tuple(stop_ids)) for ids in prompts]
+        return [list(result.tokens) for result in generate(self, requests, batch_size=batch_size)]
+
+    def get_tensor(self, name: str) -> torch.Tensor:
+        """A weight by its checkpoint name, as the file (or the random-weights mode) gives it,
+        on the host: what a reference computation outside this library needs."""
+        if name not in self.tensors:
+            raise KeyError(f"no tensor named '{name}'")
+        return self.tensors[name].detach().to("cpu")
 
     # -- the step ----------------------------------------------------------------
     def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> torch.Tensor:
