@@ -335,7 +335,21 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
                 }
     } else {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i) {
+            // When accumulating, what the outputs of one row block hold is read in one go, from
+            // addresses clamped into the matrix, before any of them is written: guarded, each
+            // read would wait for the one before it.
+            float before[TN][16];
+            if constexpr (MODE == MODE_ACCUMULATE) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const long m = min(m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4, (long)M - 1);
+                        const long n = min(n0 + wave_n * WAVE_N + j * 32 + lane % 32, (long)N - 1);
+                        before[j][e] = to_float(out[m * (long)N + n]);
+                    }
+            }
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -343,11 +357,11 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
                     const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
                     const long n = n0 + wave_n * WAVE_N + j * 32 + lane % 32;
                     if (m < M && n < N) {
-                        TO* dst = out + m * (long)N + n;
-                        if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(acc[i][j][e]);
-                        else *dst = from_float<TO>(to_float(*dst) + acc[i][j][e]);
+                        if constexpr (MODE == MODE_STORE) out[m * (long)N + n] = from_float<TO>(acc[i][j][e]);
+                        else out[m * (long)N + n] = from_float<TO>(before[j][e] + acc[i][j][e]);
                     }
                 }
+        }
     }
 }
 
