@@ -196,3 +196,34 @@ def test_replayed_decode_steps_equal_direct_ones(dtype, models):
     assert len(recorded.graphs.graphs) >= 2
     for index, (a, b) in enumerate(zip(*outputs)):
         assert torch.equal(a, b), f"step {index}: a replayed graph differs from the direct step"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decoding_across_a_thousand_tokens(dtype, tmp_path):
+    """Two sequences decode from just under 1024 tokens to beyond it, one of them from a block edge:
+    the recorded decode steps change their context size on the way (head size 64: in bfloat16 the
+    matrix-core decode kernel with its split over key chunks and its merge). Every step must equal
+    the same step run directly, and the last logits must be the plain model's."""
+    from xeno_rt_amd.engine import Engine
+    raw = dict(TINY["llama"], max_position_embeddings=1200, num_hidden_layers=2, num_attention_heads=4,
+               num_key_value_heads=1, head_dim=64, rope_theta=50000.0)
+    folder = make_folder(raw, tmp_path / "long", seed=9, std=0.25)
+    plain = P.PlainModel(folder)
+    vocab = plain.config.vocab_size
+    starts, steps = (1000, 960), 70
+    sequences = [token_ids(vocab, n + steps, seed=n) for n in starts]
+    rows = []
+    for graphs in (True, False):
+        engine = Engine.load(folder, dtype=dtype, max_tokens=64 * 40, max_slots=2, graphs=graphs)
+        slots = [engine.alloc_slot() for _ in starts]
+        engine.step([(s, ids[:n], []) for s, ids, n in zip(slots, sequences, starts)])
+        out = [engine.step([(s, [ids[n + t]], [0]) for s, ids, n in zip(slots, sequences, starts)]).clone()
+               for t in range(steps)]
+        rows.append(out)
+        if graphs:
+            assert engine.graphs is not None and len(engine.graphs.graphs) >= 2     # two context sizes
+    for t, (a, b) in enumerate(zip(*rows)):
+        assert torch.equal(a, b), f"decode step {t}: the recorded step differs from the direct one"
+    for i, (ids, n) in enumerate(zip(sequences, starts)):
+        want = plain.logits(ids)[-1:]
+        assert_logits(rows[0][-1][i:i + 1], want, dtype, f"sequence {i}, last decoded token")
