@@ -227,3 +227,26 @@ def test_decoding_across_a_thousand_tokens(dtype, tmp_path):
     for i, (ids, n) in enumerate(zip(sequences, starts)):
         want = plain.logits(ids)[-1:]
         assert_logits(rows[0][-1][i:i + 1], want, dtype, f"sequence {i}, last decoded token")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_batch_of_forty_sequences(dtype, tmp_path):
+    """Forty sequences of unequal lengths start together and end one after the other: the step's
+    token count runs through 300-odd (prompts), 40 and down to 1, and with a width of 128 the
+    bfloat16 products take every kernel there is on the way: the tiled one and the one split along
+    k for the prompts, the split one for 17 to 40 rows, the streaming one below."""
+    from xeno_rt_amd.engine import Engine
+    raw = dict(TINY["qwen3"], hidden_size=128, intermediate_size=320, num_attention_heads=4, num_key_value_heads=2,
+               head_dim=64, num_hidden_layers=2, max_position_embeddings=128)
+    folder = make_folder(raw, tmp_path / "wide", seed=13, std=0.15)
+    plain = P.PlainModel(folder)
+    vocab = plain.config.vocab_size
+    lengths = [6 + (7 * i) % 45 for i in range(40)]
+    prompts = [1 + (3 * i) % 5 + (i % 7) * 2 for i in range(40)]
+    requests = [token_ids(vocab, n, seed=200 + i) for i, n in enumerate(lengths)]
+    engine = Engine.load(folder, dtype=dtype, max_tokens=64 * 40, max_slots=40)
+    got = run_batched(engine, requests, [min(p, n) for p, n in zip(prompts, lengths)])
+    for i, (ids, rows) in enumerate(zip(requests, got)):
+        assert_logits(rows, plain.logits(ids), dtype, f"request {i} of 40")
+    engine.cache.check()
+    assert engine.cache.slots.n_held == 0
