@@ -52,10 +52,12 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 
 __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 
+// One tile of the product, by one workgroup: `id` is the workgroup's number among those that work
+// on the output columns from n_first on, tiles_m x tiles_n of them.
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
-__global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
+__device__ __forceinline__ void gemm_tile(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int tiles_m, int tiles_n, int n_first, int k_per_split) {
+    int id, int tiles_m, int tiles_n, int n_first, int k_per_split) {
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr int WAVE_M = BM / WM, WAVE_N = BN / WN;        // part of the tile owned by one wavefront
     constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;        // 32x32 accumulator tiles of a wavefront
@@ -69,7 +71,6 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     // ---- which tile: ids are dealt to XCDs round-robin; give each XCD a contiguous run of tiles,
     // and walk a run m-fastest inside panels of 8 n-tiles so that concurrent tiles share w
     const int total = tiles_m * tiles_n;
-    int id = blockIdx.x;
     {
         const int xcds = 8;
         const int per = (total + xcds - 1) / xcds;
@@ -366,6 +367,29 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     }
 }
 
+template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
+__global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
+    const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
+    int tiles_m, int tiles_n, int n_first, int k_per_split) {
+    gemm_tile<BM, BN, WM, WN, MODE, DK, STAGES, TO>(a, w, out, M, N, K, blockIdx.x, tiles_m, tiles_n, n_first, k_per_split);
+}
+
+// Two tile shapes in one launch: the first `large_blocks` workgroups take 256 x 256 tiles of the
+// output columns below `split`, the others 128 x 256 tiles of the columns from `split` on. The
+// large tiles are handed out first and fill whole rounds over the compute units; the small ones
+// follow as compute units become free, so the last round is full of half-sized work and there is
+// no gap between the two.
+template <int MODE, typename TO>
+__global__ void __launch_bounds__(8 * XRT_WAVE) gemm_mfma_mixed_kernel(
+    const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
+    int large_blocks, int large_tiles_m, int large_tiles_n, int split, int small_tiles_m, int small_tiles_n) {
+    if ((int)blockIdx.x < large_blocks)
+        gemm_tile<256, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x, large_tiles_m, large_tiles_n, 0, K);
+    else
+        gemm_tile<128, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x - large_blocks, small_tiles_m,
+                                                   small_tiles_n, split, K);
+}
+
 // Launches the tiles of output columns [n_first, n_first + n_count).
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, hipStream_t s,
@@ -434,9 +458,21 @@ int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipS
         mixed = rounds_cost((long)tiles_m * whole_columns, 256 * 256, 1, 0) + rounds_cost(rest_tiles, 128 * 256, 1, 8);
     if (mixed < large && mixed <= medium && mixed <= small) {
         const int split = whole_columns * (256 / DIV);
-        const int status = launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, 0, split, s);
-        if (status != 0) return status;
-        return launch<128, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, split, N - split, s);
+        const int small_tiles_m = (M + 127) / 128, small_tiles_n = tiles_n - whole_columns;
+        const int large_blocks = (tiles_m * whole_columns + 7) / 8 * 8;      // whole rounds over the XCDs
+        const int small_blocks = (small_tiles_m * small_tiles_n + 7) / 8 * 8;
+        constexpr size_t lds = (size_t)2 * (256 + 256) * 64 * sizeof(bf16);
+        auto kernel = gemm_mfma_mixed_kernel<MODE, TO>;
+        static bool configured = false;      // per instantiation
+        if (!configured) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            XRT_REQUIRE(e == hipSuccess, "linear (mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+            configured = true;
+        }
+        kernel<<<large_blocks + small_blocks, 8 * XRT_WAVE, lds, s>>>(a, w, out, M, N, K, large_blocks, tiles_m, whole_columns,
+                                                                      split, small_tiles_m, small_tiles_n);
+        XRT_LAUNCH_CHECK("linear (mfma, two tile shapes)");
+        return 0;
     }
     if (large <= medium && large <= small) return launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, 0, N, s);
     if constexpr (MODE != MODE_GATED)
