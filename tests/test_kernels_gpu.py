@@ -455,6 +455,31 @@ def test_sample_matches_the_plain_distribution(ops, vocab):
         assert greedy == [P.greedy(adjusted)] * 2
 
 
+def test_sample_with_ties_by_the_thousand_and_a_large_top_k(ops):
+    """What top-k leaves is kept in a short list on the chip when it fits; ties that do not fit, and a
+    top-k of thousands, take the path over the whole row. Either way only kept tokens are drawn, and an
+    even sweep of draws meets every kept token in proportion."""
+    vocab, draws = 5000, 400
+    u = ((torch.arange(draws) + 0.5) / draws).tolist()
+    flat = torch.zeros(vocab)
+    flat[[17, 4000]] = 1.0                                         # two tokens above 4998 that tie
+    for top_k, allowed in ((2, {17, 4000}), (3, set(range(vocab)))):    # the third place is a tie of 4998
+        picks = sample(ops, flat.to(DEV)[None, :].expand(draws, vocab).contiguous(), 1.0, top_k, 1.0, draws=u)
+        assert set(picks) <= allowed
+        if top_k == 2:
+            assert abs(picks.count(17) - draws / 2) <= 1 and abs(picks.count(4000) - draws / 2) <= 1
+        else:
+            assert len(set(picks)) > 300                            # spread over the tie, not stuck on the top two
+    g = torch.Generator().manual_seed(5)
+    row = torch.randn(vocab, generator=g) * 2.0
+    for top_k in (1500, 2500):                                      # fits the list narrowly, or not at all
+        dist = P.sampling_distribution(row, 1.0, top_k, 0.9)
+        picks = sample(ops, row.to(DEV)[None, :].expand(draws, vocab).contiguous(), 1.0, top_k, 0.9, draws=u)
+        counts = torch.bincount(torch.tensor(picks), minlength=vocab).double() / draws
+        assert float((counts - dist).abs().max()) <= 1.5 / draws + 1e-6
+        assert set(torch.nonzero(counts).flatten().tolist()) <= set(torch.nonzero(dist).flatten().tolist())
+
+
 def test_sample_rows_are_independent(ops):
     g = torch.Generator().manual_seed(1)
     logits = (torch.randn(5, 777, generator=g) * 3).to(DEV)
