@@ -38,9 +38,11 @@ struct Row {
     float penalty;
     bool penalised;
     int vocab;
+    // without branches: a pass makes this choice a hundred times per thread
     __device__ __forceinline__ float adjusted(int i, float v) const {
-        if (penalised && ((seen[i >> 5] >> (i & 31)) & 1u)) v = v > 0.f ? v / penalty : v * penalty;
-        return v;
+        const unsigned word = penalised ? seen[i >> 5] : 0u;
+        const float changed = v > 0.f ? v / penalty : v * penalty;
+        return (word >> (i & 31)) & 1u ? changed : v;
     }
     // f(i, value) for this thread's tokens i = tid, tid + THREADS, ..., in ascending order
     template <typename F>
@@ -360,21 +362,29 @@ __global__ void __launch_bounds__(THREADS) sample_kernel(
         const float target = target_in_wave;
         float running = 0.f;                            // mass of the ids before the current 64
         int pick = -1, last_kept = -1;
-        for (int base = begin; base < end && pick < 0; base += XRT_WAVE) {
-            const int i = base + lane;
-            const float w = i < end ? kept(i, row.logits[min(i, vocab - 1)]) : 0.f;
-            float through = w;                          // inclusive sum over the lanes, in lane order
+        for (int outer = begin; outer < end && pick < 0; outer += IN_FLIGHT * XRT_WAVE) {
+            float v[IN_FLIGHT];
 #pragma unroll
-            for (int offset = 1; offset < XRT_WAVE; offset <<= 1) {
-                const float below = __shfl_up(through, offset, XRT_WAVE);
-                if (lane >= offset) through += below;
+            for (int u = 0; u < IN_FLIGHT; ++u) v[u] = row.logits[min(outer + u * XRT_WAVE + lane, vocab - 1)];
+#pragma unroll
+            for (int u = 0; u < IN_FLIGHT; ++u) {
+                const int base = outer + u * XRT_WAVE;
+                if (base >= end || pick >= 0) continue;     // uniform in the wavefront
+                const int i = base + lane;
+                const float w = i < end ? kept(i, v[u]) : 0.f;
+                float through = w;                      // inclusive sum over the lanes, in lane order
+#pragma unroll
+                for (int offset = 1; offset < XRT_WAVE; offset <<= 1) {
+                    const float below = __shfl_up(through, offset, XRT_WAVE);
+                    if (lane >= offset) through += below;
+                }
+                const bool hit = w > 0.f && running + through > target;
+                const unsigned long long hits = __ballot(hit);
+                const unsigned long long kepts = __ballot(w > 0.f);
+                if (hits != 0ull) pick = base + __builtin_ctzll(hits);
+                if (kepts != 0ull) last_kept = base + 63 - __builtin_clzll(kepts);
+                running += __shfl(through, XRT_WAVE - 1, XRT_WAVE);
             }
-            const bool hit = w > 0.f && running + through > target;
-            const unsigned long long hits = __ballot(hit);
-            const unsigned long long kepts = __ballot(w > 0.f);
-            if (hits != 0ull) pick = base + __builtin_ctzll(hits);
-            if (kepts != 0ull) last_kept = base + 63 - __builtin_clzll(kepts);
-            running += __shfl(through, XRT_WAVE - 1, XRT_WAVE);
         }
         if (pick < 0) pick = last_kept;                 // rounding at the run's end: its last kept token
         if (lane == 0) chosen = pick;
