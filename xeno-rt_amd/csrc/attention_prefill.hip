@@ -47,12 +47,18 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     constexpr int QW = WAVES * QT;         // query tokens per workgroup
     constexpr int KS = HD / 16;            // K steps of the score product
     constexpr int DT = HD / 32;            // 32-row tiles of the value product
-    constexpr int KP = HD + 8;             // LDS pitch of a key row
-    constexpr int VP = BT + 8;             // LDS pitch of a transposed value row
-    constexpr int CHUNKS = BT * HD / 8 / (WAVES * XRT_WAVE);    // 16-byte chunks per thread for keys (and as many for values)
+    constexpr int K_CHUNKS = HD / 8;       // 16-byte chunks of a key row (16 or 8)
+    constexpr int V_CHUNKS = BT / 8;       // of a transposed value row (8)
+    constexpr int LOADS = BT * HD * 2 / 1024 / WAVES;           // load instructions per wavefront for a block's keys (and as many for its values)
+    static_assert(BT * HD * 2 % (1024 * WAVES) == 0, "a cache block does not divide among the wavefronts");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    bf16 (*lds_k)[BT * KP] = reinterpret_cast<bf16 (*)[BT * KP]>(lds_raw);                                  // [2][BT * KP]
-    bf16 (*lds_v)[HD * VP] = reinterpret_cast<bf16 (*)[HD * VP]>(lds_raw + 2 * BT * KP * sizeof(bf16));     // [2][HD * VP]
+    bf16 (*lds_k)[BT * HD] = reinterpret_cast<bf16 (*)[BT * HD]>(lds_raw);                                  // [2][BT * HD]
+    bf16 (*lds_v)[HD * BT] = reinterpret_cast<bf16 (*)[HD * BT]>(lds_raw + 2 * BT * HD * sizeof(bf16));     // [2][HD * BT]
+    // Rows are not padded (a load instruction fills 1024 consecutive bytes of LDS); instead the
+    // 16-byte chunks of a row lie in permuted places, place = chunk ^ swizzle(row), chosen so
+    // that the operand reads of consecutive rows at one chunk fall into different banks.
+    auto k_swizzle = [](int row) { return K_CHUNKS == 16 ? row % 16 : (row % 8) ^ (row / 8 % 2); };
+    auto v_swizzle = [](int row) { return (row % 8) ^ (row / 8 % 2); };
 
     const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
     const int col = lane % 32, half = lane / 32;
@@ -95,28 +101,29 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
 
-    // ---- moving a cache block into LDS: both parts are contiguous in global memory
-    bf16x8 stage_k[CHUNKS], stage_v[CHUNKS];
-    auto fetch = [&](int b) {
+    // ---- moving a cache block into LDS: both parts are contiguous in global memory, and go
+    // straight there (global_load_lds_dwordx4): lane l of an instruction fills the l-th 16 bytes
+    // of a 1024-byte stretch with the chunk that belongs in that place
+    const int wave_uniform = __builtin_amdgcn_readfirstlane(wave);
+    unsigned k_from[LOADS], v_from[LOADS];                   // byte offsets of this lane's chunks within a block
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int place = ((i * WAVES + wave) * XRT_WAVE + lane);          // 16-byte place within the block's LDS image
+        const int k_row = place / K_CHUNKS, v_row = place / V_CHUNKS;
+        k_from[i] = (unsigned)((k_row * K_CHUNKS + ((place % K_CHUNKS) ^ k_swizzle(k_row))) * 16);
+        v_from[i] = (unsigned)((v_row * V_CHUNKS + ((place % V_CHUNKS) ^ v_swizzle(v_row))) * 16);
+    }
+    const unsigned lds_k0 = lds_address(lds_raw), lds_v0 = lds_k0 + 2 * BT * HD * (unsigned)sizeof(bf16);
+    auto fetch = [&](int b, int buffer) {
         int block = block_table[(long)slot * table_stride + b];
         block = min(max(block, 0), n_blocks - 1);            // the host never hands out anything else
         const bf16* kb = k_cache + ((long)block * n_kv_heads + kv_head) * BT * HD;
         const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * BT;
 #pragma unroll
-        for (int i = 0; i < CHUNKS; ++i) {
-            const int chunk = tid + i * WAVES * XRT_WAVE;
-            stage_k[i] = *reinterpret_cast<const bf16x8*>(kb + chunk * 8);
-            stage_v[i] = *reinterpret_cast<const bf16x8*>(vb + chunk * 8);
-        }
-    };
-    auto stash = [&](int buffer) {
-#pragma unroll
-        for (int i = 0; i < CHUNKS; ++i) {
-            const int chunk = tid + i * WAVES * XRT_WAVE;
-            const int k_row = chunk / (HD / 8), k_at = chunk % (HD / 8);
-            *reinterpret_cast<bf16x8*>(&lds_k[buffer][k_row * KP + k_at * 8]) = stage_k[i];
-            const int v_row = chunk / (BT / 8), v_at = chunk % (BT / 8);
-            *reinterpret_cast<bf16x8*>(&lds_v[buffer][v_row * VP + v_at * 8]) = stage_v[i];
+        for (int i = 0; i < LOADS; ++i) {
+            const unsigned at = (unsigned)((buffer * BT * HD) * 2 + (i * WAVES + wave_uniform) * 1024);
+            load_to_lds(kb, k_from[i], lds_k0 + at);
+            load_to_lds(vb, v_from[i], lds_v0 + at);
         }
     };
 
@@ -124,16 +131,19 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 
     // one tile of 32 keys (half a block) against this wavefront's 32 queries
     auto tile32 = [&](int buffer, int k0, int in_block) {
-        const bf16* kb = &lds_k[buffer][(in_block + row_key) * KP + half * 8];
-        const bf16* vb = &lds_v[buffer][in_block + half * 8];
+        const bf16* kb = &lds_k[buffer][(in_block + row_key) * HD];
+        const int k_turn = k_swizzle(in_block + row_key);     // in_block is 0 or 32: the swizzle of this lane's key row
+        const bf16* vb = &lds_v[buffer][0];
+        const int v_first = in_block / 8 + half;              // chunk of a value row that step 0 reads
+        auto k_at = [&](int ks) { return kb + ((ks * 2 + half) ^ k_turn) * 8; };
         // two accumulators, used in turn, so that consecutive products do not wait on each other
         floatx16 s, s_odd;
 #pragma unroll
         for (int e = 0; e < 16; ++e) s[e] = s_odd[e] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ks += 2) {
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kb + ks * 16), q[ks], s, 0, 0, 0);
-            s_odd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kb + (ks + 1) * 16), q[ks + 1], s_odd, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(k_at(ks)), q[ks], s, 0, 0, 0);
+            s_odd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(k_at(ks + 1)), q[ks + 1], s_odd, 0, 0, 0);
         }
 #pragma unroll
         for (int e = 0; e < 16; ++e) s[e] += s_odd[e];
@@ -177,7 +187,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         for (int step = 0; step < 2; ++step)
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                bf16x8 v = *reinterpret_cast<const bf16x8*>(vb + (dt * 32 + col) * VP + step * 16);
+                const int v_row = dt * 32 + col;
+                bf16x8 v = *reinterpret_cast<const bf16x8*>(vb + v_row * BT + ((v_first + step * 2) ^ v_swizzle(v_row)) * 8);
                 if (edge) {
                     // beyond the sequence's last key the block holds nothing of ours: keep it away from the zeros of p
 #pragma unroll
@@ -190,12 +201,11 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 
     // ---- the blocks of the sequence, in order: block b+1 travels while block b is used
     const int last_block = wg_last_key / BT;
-    fetch(0);
-    stash(0);
-    __syncthreads();
+    fetch(0, 0);
+    wait_loads_and_barrier<0>();
     for (int b = 0; b <= last_block; ++b) {
         const int buffer = b & 1;
-        if (b < last_block) fetch(b + 1);
+        if (b < last_block) fetch(b + 1, buffer ^ 1);          // that buffer was read in step b-1, before the last barrier
         if (q_count > 0) {
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub) {
@@ -203,8 +213,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
                 if (k0 <= last_key) tile32(buffer, k0, sub * 32);        // uniform in the wavefront
             }
         }
-        if (b < last_block) stash(buffer ^ 1);
-        __syncthreads();
+        wait_loads_and_barrier<0>();                         // block b+1 has arrived from every wavefront, block b has been read by all
     }
     l += __shfl_xor(l, 32, XRT_WAVE);
 
@@ -234,7 +243,7 @@ int launch_waves(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const
     const long tiles = (tokens + QW - 1) / QW + n_seqs;
     XRT_REQUIRE(tiles <= 65535, "attention (prefill): too many query tiles for the grid");
     const dim3 grid(n_heads, (unsigned)tiles);
-    constexpr size_t lds = (size_t)2 * (BT * (HD + 8) + HD * (BT + 8)) * sizeof(bf16);
+    constexpr size_t lds = (size_t)2 * (BT * HD + HD * BT) * sizeof(bf16);
     static bool configured = false;          // per instantiation
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD, WAVES>),

@@ -77,3 +77,25 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     for (int w = 0; w < waves; ++w) total += scratch[w];
     return total;
 }
+// ---- global memory -> LDS without passing registers (gfx950) ----------------------------------
+// 16 bytes per lane from global memory into LDS without passing registers: lane l of the
+// wavefront writes LDS byte address lds_base + 16 * l (lds_base is the same for the whole
+// wavefront and travels in M0) with the 16 bytes at base + byte_offset (of that lane). Written
+// as assembly so that the waits for these loads are the explicit ones in the kernel: the
+// compiler, when it knows of such a load, waits for all of them at every barrier.
+__device__ __forceinline__ void load_to_lds(const void* base, unsigned byte_offset, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base), "v"(byte_offset), "s"(base) : "memory");
+}
+// Waits until at most `pending` of this wavefront's loads (the newest ones) are outstanding and
+// its LDS reads are done, then meets the workgroup's other wavefronts. __syncthreads() cannot
+// stand here: its release fence waits for every load, also those meant to stay in flight.
+template <int pending>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(pending) : "memory");
+}
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    return (unsigned)(unsigned long)(const __attribute__((address_space(3))) void*)p;
+}
+
+
