@@ -31,6 +31,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int QT = 32;                 // query tokens per wavefront
 constexpr int BT = XRT_BLOCK_TOKENS;   // keys per cache block
+constexpr int PER_STAGE = 2;           // cache blocks between two barriers
 constexpr float LOG2E = 1.4426950408889634f;
 
 // Key (0..31 within a tile of 32 keys) that row r of the score tile stands for. Accumulator
@@ -52,8 +53,9 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     constexpr int LOADS = BT * HD * 2 / 1024 / WAVES;           // load instructions per wavefront for a block's keys (and as many for its values)
     static_assert(BT * HD * 2 % (1024 * WAVES) == 0, "a cache block does not divide among the wavefronts");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    bf16 (*lds_k)[BT * HD] = reinterpret_cast<bf16 (*)[BT * HD]>(lds_raw);                                  // [2][BT * HD]
-    bf16 (*lds_v)[HD * BT] = reinterpret_cast<bf16 (*)[HD * BT]>(lds_raw + 2 * BT * HD * sizeof(bf16));     // [2][HD * BT]
+    // two buffers of PER_STAGE cache blocks each: one barrier per PER_STAGE blocks
+    bf16 (*lds_k)[BT * HD] = reinterpret_cast<bf16 (*)[BT * HD]>(lds_raw);                                  // [2 * PER_STAGE][BT * HD]
+    bf16 (*lds_v)[HD * BT] = reinterpret_cast<bf16 (*)[HD * BT]>(lds_raw + 2 * PER_STAGE * BT * HD * sizeof(bf16));   // [2 * PER_STAGE][HD * BT]
     // Rows are not padded (a load instruction fills 1024 consecutive bytes of LDS); instead the
     // 16-byte chunks of a row lie in permuted places, place = chunk ^ swizzle(row), chosen so
     // that the operand reads of consecutive rows at one chunk fall into different banks.
@@ -113,7 +115,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         k_from[i] = (unsigned)((k_row * K_CHUNKS + ((place % K_CHUNKS) ^ k_swizzle(k_row))) * 16);
         v_from[i] = (unsigned)((v_row * V_CHUNKS + ((place % V_CHUNKS) ^ v_swizzle(v_row))) * 16);
     }
-    const unsigned lds_k0 = lds_address(lds_raw), lds_v0 = lds_k0 + 2 * BT * HD * (unsigned)sizeof(bf16);
+    const unsigned lds_k0 = lds_address(lds_raw), lds_v0 = lds_k0 + 2 * PER_STAGE * BT * HD * (unsigned)sizeof(bf16);
     auto fetch = [&](int b, int buffer) {
         int block = block_table[(long)slot * table_stride + b];
         block = min(max(block, 0), n_blocks - 1);            // the host never hands out anything else
@@ -201,11 +203,20 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 
     // ---- the blocks of the sequence, in order: block b+1 travels while block b is used
     const int last_block = wg_last_key / BT;
-    fetch(0, 0);
+#pragma unroll
+    for (int i = 0; i < PER_STAGE; ++i)
+        if (i <= last_block) fetch(i, i);
     wait_loads_and_barrier<0>();
-    for (int b = 0; b <= last_block; ++b) {
-        const int buffer = b & 1;
-        if (b < last_block) fetch(b + 1, buffer ^ 1);          // that buffer was read in step b-1, before the last barrier
+    for (int first = 0; first <= last_block; first += PER_STAGE) {
+        const int stage = (first / PER_STAGE) & 1;
+        // the other stage's buffers were read in the step before, ahead of the last barrier
+#pragma unroll
+        for (int i = 0; i < PER_STAGE; ++i)
+            if (first + PER_STAGE + i <= last_block) fetch(first + PER_STAGE + i, (stage ^ 1) * PER_STAGE + i);
+#pragma unroll
+        for (int i = 0; i < PER_STAGE; ++i) {
+        const int b = first + i, buffer = stage * PER_STAGE + i;
+        if (b > last_block) continue;
         if (q_count > 0) {
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub) {
@@ -213,7 +224,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
                 if (k0 <= last_key) tile32(buffer, k0, sub * 32);        // uniform in the wavefront
             }
         }
-        wait_loads_and_barrier<0>();                         // block b+1 has arrived from every wavefront, block b has been read by all
+        }
+        wait_loads_and_barrier<0>();                         // the next blocks have arrived from every wavefront, these have been read by all
     }
     l += __shfl_xor(l, 32, XRT_WAVE);
 
@@ -243,7 +255,7 @@ int launch_waves(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const
     const long tiles = (tokens + QW - 1) / QW + n_seqs;
     XRT_REQUIRE(tiles <= 65535, "attention (prefill): too many query tiles for the grid");
     const dim3 grid(n_heads, (unsigned)tiles);
-    constexpr size_t lds = (size_t)2 * (BT * HD + HD * BT) * sizeof(bf16);
+    constexpr size_t lds = (size_t)2 * PER_STAGE * (BT * HD + HD * BT) * sizeof(bf16);
     static bool configured = false;          // per instantiation
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD, WAVES>),
