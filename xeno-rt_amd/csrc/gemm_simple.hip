@@ -12,7 +12,7 @@
 
 namespace {
 
-constexpr int BM = 64, BN = 64, BK = 16, PAD = 4;
+constexpr int BN = 64, BK = 16, PAD = 4;
 enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
 
 template <typename T>
@@ -38,10 +38,13 @@ __device__ __forceinline__ void load4(const T* __restrict__ base, long row, int 
 
 __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }   // silu.rs:1-3
 
-template <typename TI, typename TO, int MODE>
+// RM rows of the output per thread: a tile is 16 RM x 64. With few rows of a (a decode step) the
+// small tile does a quarter of the arithmetic; an element's sum is the same either way.
+template <typename TI, typename TO, int MODE, int RM>
 __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__ a, const TI* __restrict__ w,
                                                           TO* __restrict__ out, int M, int N, int K,
                                                           int vector_ok) {
+    constexpr int BM = 16 * RM;
     __shared__ __attribute__((aligned(16))) float As[BK][BM + PAD];
     __shared__ __attribute__((aligned(16))) float Ws[BK][BN + PAD];
     __shared__ __attribute__((aligned(16))) float Us[MODE == MODE_GATED ? BK : 1][BN + PAD];
@@ -50,40 +53,42 @@ __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__
     const long m0 = (long)blockIdx.y * BM, n0 = (long)blockIdx.x * BN;
     const int load_row = tid / 4, load_k = (tid % 4) * 4;
 
-    float acc[4][4] = {}, acc_up[MODE == MODE_GATED ? 4 : 1][4] = {};
+    float acc[RM][4] = {}, acc_up[MODE == MODE_GATED ? RM : 1][4] = {};
 
-    for (int k0 = 0; k0 < K; k0 += BK) {
-        float va[4], vw[4];
-        load4(a, m0 + load_row, M, k0 + load_k, K, vector_ok, va);
+    // the tile after the one being multiplied is on its way from global memory meanwhile
+    float va[4], vw[4], vu[4] = {0.f, 0.f, 0.f, 0.f};
+    auto fetch = [&](int k0) {
+        if (load_row < BM) load4(a, m0 + load_row, M, k0 + load_k, K, vector_ok, va);
         load4(w, n0 + load_row, N, k0 + load_k, K, vector_ok, vw);
+        // rows of the "up" half follow the N rows of the "gate" half
+        if constexpr (MODE == MODE_GATED) load4(w + (long)N * K, n0 + load_row, N, k0 + load_k, K, vector_ok, vu);
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += BK) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            As[load_k + i][load_row] = va[i];
+            if (load_row < BM) As[load_k + i][load_row] = va[i];
             Ws[load_k + i][load_row] = vw[i];
+            if constexpr (MODE == MODE_GATED) Us[load_k + i][load_row] = vu[i];
         }
-        if constexpr (MODE == MODE_GATED) {
-            float vu[4];
-            // rows of the "up" half follow the N rows of the "gate" half
-            load4(w + (long)N * K, n0 + load_row, N, k0 + load_k, K, vector_ok, vu);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) Us[load_k + i][load_row] = vu[i];
-        }
+        if (k0 + BK < K) fetch(k0 + BK);
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < BK; ++kk) {
-            const float4 av = *reinterpret_cast<const float4*>(&As[kk][ty * 4]);
+            float ar[RM];
+#pragma unroll
+            for (int i = 0; i < RM; ++i) ar[i] = As[kk][ty * RM + i];
             const float4 wv = *reinterpret_cast<const float4*>(&Ws[kk][tx * 4]);
-            const float ar[4] = {av.x, av.y, av.z, av.w};
             const float wr[4] = {wv.x, wv.y, wv.z, wv.w};
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < RM; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
             if constexpr (MODE == MODE_GATED) {
                 const float4 uv = *reinterpret_cast<const float4*>(&Us[kk][tx * 4]);
                 const float ur[4] = {uv.x, uv.y, uv.z, uv.w};
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < RM; ++i)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) acc_up[i][j] = fmaf(ar[i], ur[j], acc_up[i][j]);
             }
@@ -91,32 +96,48 @@ __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__
         __syncthreads();
     }
 
+    // when accumulating, the old values are read in one go (from addresses clamped into
+    // the matrix) before any is written: guarded one by one, each read would wait for the last
+    float before[RM][4] = {};
+    if constexpr (MODE == MODE_ACCUMULATE) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const long m = m0 + ty * 4 + i;
-        if (m >= M) continue;
+        for (int i = 0; i < RM; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                before[i][j] = to_float(out[min(m0 + ty * RM + i, (long)M - 1) * N + min(n0 + tx * 4 + j, (long)N - 1)]);
+    }
+#pragma unroll
+    for (int i = 0; i < RM; ++i) {
+        const long m = m0 + ty * RM + i;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const long n = n0 + tx * 4 + j;
-            if (n >= N) continue;
+            if (m >= M || n >= N) continue;
             TO* dst = out + m * (long)N + n;
             if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(acc[i][j]);
-            if constexpr (MODE == MODE_ACCUMULATE) *dst = from_float<TO>(to_float(*dst) + acc[i][j]);
+            if constexpr (MODE == MODE_ACCUMULATE) *dst = from_float<TO>(before[i][j] + acc[i][j]);
             if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(silu(acc[i][j]) * acc_up[i][j]);
         }
     }
 }
 
-template <typename TI, typename TO>
-int launch(const void* a, const void* w, void* out, int M, int N, int K, int mode, hipStream_t s) {
+template <typename TI, typename TO, int RM>
+void launch_rows(const void* a, const void* w, void* out, int M, int N, int K, int mode, hipStream_t s) {
+    constexpr int BM = 16 * RM;
     const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
     const int vector_ok = (K % 4 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
     if (mode == MODE_STORE)
-        gemm_simple_kernel<TI, TO, MODE_STORE><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+        gemm_simple_kernel<TI, TO, MODE_STORE, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
     else if (mode == MODE_ACCUMULATE)
-        gemm_simple_kernel<TI, TO, MODE_ACCUMULATE><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+        gemm_simple_kernel<TI, TO, MODE_ACCUMULATE, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
     else
-        gemm_simple_kernel<TI, TO, MODE_GATED><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+        gemm_simple_kernel<TI, TO, MODE_GATED, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+}
+
+template <typename TI, typename TO>
+int launch(const void* a, const void* w, void* out, int M, int N, int K, int mode, hipStream_t s) {
+    if (M <= 16) launch_rows<TI, TO, 1>(a, w, out, M, N, K, mode, s);
+    else launch_rows<TI, TO, 4>(a, w, out, M, N, K, mode, s);
     XRT_LAUNCH_CHECK("linear (plain)");
     return 0;
 }
