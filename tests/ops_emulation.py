@@ -37,16 +37,39 @@ class EmulatedOps:
         out.copy_(((src * inv) * weight.to(torch.float32)).to(out.dtype))
 
     # -- products ---------------------------------------------------------------
-    def linear(self, a, w, out, accumulate=False):
-        result = a.to(torch.float32) @ w.to(torch.float32).t()
+    # An RMSNorm between two products may be done by the two of them (the kernels do so for steps
+    # of few rows): the first returns the updated rows times the gain with their sums of squares,
+    # the second divides by the rms.
+    norms_between_products = True
+
+    class Prescaled:
+        def __init__(self, values, squares, eps):
+            self.values, self.squares, self.eps = values, squares, eps
+            self.shape = values.shape
+
+    def _rows(self, a):
+        if isinstance(a, self.Prescaled):
+            inv = 1.0 / torch.sqrt(a.squares / a.values.shape[-1] + a.eps)
+            return a.values.to(torch.float32), inv[:, None]
+        return a.to(torch.float32), 1.0
+
+    def linear(self, a, w, out, accumulate=False, then_norm=None):
+        rows, inv = self._rows(a)
+        result = (rows @ w.to(torch.float32).t()) * inv
         if accumulate:
             out.add_(result.to(out.dtype))
         else:
             out.copy_(result.to(out.dtype))
+        if then_norm is not None and accumulate and self.norms_between_products:
+            gain, eps = then_norm
+            fresh = out.to(torch.float32)
+            return self.Prescaled((fresh * gain.to(torch.float32)).to(w.dtype), (fresh * fresh).sum(-1), eps)
+        return None
 
     def linear_glu(self, a, w_gate_up, out):
         inter = w_gate_up.shape[0] // 2
-        both = a.to(torch.float32) @ w_gate_up.to(torch.float32).t()
+        rows, inv = self._rows(a)
+        both = (rows @ w_gate_up.to(torch.float32).t()) * inv
         gate, up = both[:, :inter], both[:, inter:]
         out.copy_(((gate / (1.0 + torch.exp(-gate))) * up).to(out.dtype))
 

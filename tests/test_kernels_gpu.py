@@ -128,6 +128,59 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(one[0], whole[row])                  # same bits: same order of the sum
 
 
+@pytest.mark.parametrize("m,hidden,k,n", [(1, 4096, 512, 1024), (8, 4096, 14336, 6144), (16, 200, 96, 72),
+                                          (5, 1000, 136, 333), (13, 8200, 64, 48)])
+def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n):
+    # x += a w^T; y = rmsnorm(x) * gain; z = y v^T (and the gated pair), the norm without a kernel of its own
+    a = rand(m, k, dtype=torch.bfloat16, seed=1)
+    w = rand(hidden, k, dtype=torch.bfloat16, seed=2, scale=0.2)
+    x = rand(m, hidden, seed=3, scale=2.0)
+    x[m // 2] *= 50.0                                            # rows of different size: each needs its own rms
+    gain = (rand(hidden, seed=4) + 1.0).to(torch.bfloat16)
+    v = rand(2 * n, hidden, dtype=torch.bfloat16, seed=5, scale=0.1)
+    eps = 1e-3
+    fresh = x.double().cpu() + a.double().cpu() @ w.double().cpu().t()
+    normed = P.rmsnorm(fresh, gain.double().cpu(), eps)
+
+    scaled = ops.linear(a, w, x, accumulate=True, then_norm=(gain, eps))
+    assert scaled is not None and scaled.shape == (m, hidden)
+    assert rel(x.cpu(), fresh) < 1e-5
+    tiles = (hidden + 15) // 16
+    padded = torch.zeros(m, tiles * 16, dtype=torch.float64)
+    padded[:, :hidden] = x.double().cpu() ** 2
+    assert rel(scaled.squares[:, :m].t().cpu(), padded.reshape(m, tiles, 16).sum(-1)) < 1e-6
+    assert rel(scaled.values.cpu(), x.double().cpu() * gain.double().cpu()) < ULP["bfloat16"]
+
+    want = normed @ v.double().cpu().t()
+    for out_dtype in (torch.float32, torch.bfloat16):
+        out = torch.empty(m, 2 * n, dtype=out_dtype, device=DEV)
+        ops.linear(scaled, v, out)
+        # the rows of y are rounded to bfloat16 before the product, by either way of doing the norm
+        unfused = torch.empty(m, hidden, dtype=torch.bfloat16, device=DEV)
+        ops.rmsnorm(x, gain, eps, unfused)
+        spread = rel(unfused.double().cpu() @ v.double().cpu().t(), want)
+        assert rel(out.cpu(), want) < 2 * spread + ULP["bfloat16" if out_dtype == torch.bfloat16 else "float32"] * 2
+    glu = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops.linear_glu(scaled, v, glu)
+    assert rel(glu.cpu(), P.swiglu(want[:, :n], want[:, n:])) < 2e-2
+    # and once more into the residual stream, with the norm after it handed on again
+    again = ops.linear(scaled, v[:hidden % 64 + 64], torch.zeros(m, hidden % 64 + 64, device=DEV), accumulate=True,
+                       then_norm=((rand(hidden % 64 + 64, seed=6) + 1.0), eps))
+    assert again is not None
+
+
+def test_rmsnorm_is_left_to_its_own_kernel_where_the_products_cannot_do_it(ops):
+    gain = rand(200, seed=4).to(torch.bfloat16)
+    for m, dtype in ((17, torch.bfloat16), (300, torch.bfloat16), (4, torch.float32)):
+        a, w = rand(m, 64, dtype=dtype), rand(200, 64, dtype=dtype)
+        x = rand(m, 200, seed=3)
+        want = x.double().cpu() + a.double().cpu() @ w.double().cpu().t()
+        assert ops.linear(a, w, x, accumulate=True, then_norm=(gain, 1e-5)) is None
+        assert rel(x.cpu(), want) < 1e-5
+    assert ops.linear(rand(4, 64, dtype=torch.bfloat16), rand(204, 64, dtype=torch.bfloat16), rand(4, 204),
+                      accumulate=True, then_norm=(rand(204).to(torch.bfloat16), 1e-5)) is None   # 204 columns: no product takes them
+
+
 def test_linear_refuses_what_it_cannot_do(ops):
     from xeno_rt_amd.ops.hip import KernelError
     a, w = rand(2, 8), rand(4, 8)

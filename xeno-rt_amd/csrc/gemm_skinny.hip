@@ -14,10 +14,18 @@
 // The eight partial sums are added in wavefront order through LDS, so the result does not
 // depend on timing. Epilogues: store (bfloat16 or float32), accumulate into float32, or the
 // gated pair silu(gate) * up with the two halves of w (rows n and n + N).
+//
+// Around an RMSNorm between two products (x += a w^T; y = rmsnorm(x) * gain; z = y v^T) a step of
+// up to 16 rows needs no kernel for the norm: the accumulating product also writes
+// bfloat16(x * gain) and, for every tile of 16 columns, each row's sum of squares; the product
+// after it takes those as its activations and multiplies its rows by 1 / sqrt(sum / width + eps).
+// The sums are added in a fixed order (tiles in eighths by wavefront, then wavefront by wavefront).
 #include "common.h"
 #include "xrt_hip.h"
 
 namespace {
+
+using LinearNorm = xrt_linear_norm;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -31,11 +39,22 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 // MT: tiles of 16 rows of x; RT: tiles of 16 rows of w per wavefront; GATED doubles the w tiles.
 // With one tile of x (the common decode case) the kernel is held to 128 registers, so that at
 // least two workgroups fit a compute unit: the stream from HBM needs the wavefronts in flight.
-template <int MT, int RT, int MODE, typename TO>
+// AROUND: the kernel also does its share of an RMSNorm before or after the product (one tile of x,
+// one tile of w per wavefront); kernels without it keep their registers for the stream.
+template <int MT, int RT, int MODE, typename TO, bool AROUND = false>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skinny_kernel(
-    const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K) {
+    const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
+    const LinearNorm norm) {
+    static_assert(!AROUND || (MT == 1 && RT == 1), "the norm around a product: one tile of x, one of w per wavefront");
     constexpr int WT = RT * (MODE == MODE_GATED ? 2 : 1);       // w tiles per wavefront
+    constexpr int SQUARES_AHEAD = 8;                            // sums of squares a lane asks for when the kernel starts
     __shared__ floatx4 partial[2][WAVES][XRT_WAVE];
+    __shared__ float squares[WAVES][16];
+    // what the epilogue needs from global memory is asked for when the kernel starts and goes
+    // straight into LDS, past the registers: it is there when the stream of w has run through
+    __shared__ __attribute__((aligned(16))) float early_squares[AROUND ? WAVES : 1][SQUARES_AHEAD][XRT_WAVE];
+    __shared__ floatx4 early_out[XRT_WAVE];
+    __shared__ float early_gain[XRT_WAVE];
 
     const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
     const int r = lane % 16, c = lane / 16;
@@ -47,7 +66,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     const int k_end = min(K, k_begin + steps_per_wave * KSTEP);
 
     // CHAINS accumulators per output tile, used in turn and added at the end
-    constexpr int CHAINS = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
+    constexpr int CHAINS = MT == 1 ? (AROUND && WT == 2 ? 2 : 4) : (MT == 2 ? 2 : 1);
     floatx4 chain[CHAINS][WT][MT];
 #pragma unroll
     for (int h = 0; h < CHAINS; ++h)
@@ -94,6 +113,63 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     // Whole steps of 128 along k run through a pipeline of two register sets: while the matrix
     // cores consume one step, the loads of the next are in flight. The steady-state loop body has
     // no branch; the last one or two steps are peeled off.
+    // The sums of squares of this wavefront's eighth of the tiles (lane (r, c): row r, every fourth tile from c).
+    const int square_tiles = AROUND && norm.squares_in ? norm.tiles_in : 0;
+    const bool out_ahead = AROUND && MODE == MODE_ACCUMULATE && N % 4 == 0;     // 16 bytes of out per lane, aligned
+    auto square_range = [&](int thread, int& first, int& end) {
+        const int per_wave = (square_tiles + WAVES - 1) / WAVES;
+        first = thread / XRT_WAVE * per_wave + thread % XRT_WAVE / 16;
+        end = min(square_tiles, (thread / XRT_WAVE + 1) * per_wave);
+    };
+    if constexpr (AROUND) {
+        if (square_tiles > 0) {
+            int first, end;
+            square_range(threadIdx.x, first, end);
+#pragma unroll
+            for (int i = 0; i < SQUARES_AHEAD; ++i) {
+                const int t = min(first + 4 * i, square_tiles - 1);
+                load_dword_to_lds(norm.squares_in, (unsigned)t * (XRT_SQUARES_STRIDE * 4u) + (unsigned)min(r, M - 1) * 4u,
+                                  __builtin_amdgcn_readfirstlane(lds_address(&early_squares[wave][i][0])));
+            }
+        }
+        if constexpr (MODE == MODE_ACCUMULATE) {
+            if (wave == 0) {                                    // the wavefront that writes the tile
+                if (out_ahead) {
+                    const long column = min(n0 + c * 4, (long)N - 4);
+                    load_to_lds(out, (unsigned)(((long)min(r, M - 1) * N + column) * 4), lds_address(&early_out[0]));
+                }
+                if (norm.squares_out) {                         // the tile's 16 gains: N is a multiple of 8 here
+                    const unsigned at = norm.gain_dtype == XRT_F32 ? (unsigned)min(n0 + lane, (long)N - 1) * 4u
+                                                                   : (unsigned)min(n0 + 2 * lane, (long)N - 2) * 2u;
+                    load_dword_to_lds(norm.gain, at, lds_address(&early_gain[0]));
+                }
+            }
+        }
+    }
+    // (the lane's place is worked out again from the thread index, behind a fence for the compiler's
+    // eyes, so that nothing of this is kept in registers while the stream of w runs)
+    auto add_squares = [&]() {
+        if constexpr (AROUND) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // what went to LDS has arrived
+            if (square_tiles > 0) {
+                int thread = threadIdx.x;
+                asm volatile("" : "+v"(thread));
+                int first, end;
+                square_range(thread, first, end);
+                const int row = min(thread % 16, M - 1);
+                float sum = 0.f;
+#pragma unroll
+                for (int i = 0; i < SQUARES_AHEAD; ++i)
+                    sum += first + 4 * i < end ? early_squares[thread / XRT_WAVE][i][thread % XRT_WAVE] : 0.f;
+                for (int t = first + 4 * SQUARES_AHEAD; t < end; t += 4)
+                    sum += norm.squares_in[(long)t * XRT_SQUARES_STRIDE + row];
+                sum += __shfl_xor(sum, 16);
+                sum += __shfl_xor(sum, 32);
+                if (thread % XRT_WAVE < 16) squares[thread / XRT_WAVE][thread % 16] = sum;   // read after the barrier of the first tile below
+            }
+        }
+    };
+
     const int full = max(0, (min(k_end, K / KSTEP * KSTEP) - k_begin) / KSTEP);     // whole steps of this wavefront
     if (full > 0) {
         bf16x8 w_a[WT][4], w_b[WT][4];
@@ -137,6 +213,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
             }
         }
     }
+    add_squares();
     floatx4 acc[WT][MT];
 #pragma unroll
     for (int t = 0; t < WT; ++t)
@@ -172,16 +249,51 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
         if (wave == tile % WAVES) {
             const int mm = m * 16 + r;                          // lane holds column m = lane % 16 ...
             const long nn = n0 + rt * 16 + c * 4;               // ... and rows n = (lane / 16) * 4 + i
+            float g[4] = {gate_sum.x, gate_sum.y, gate_sum.z, gate_sum.w};
+            float u[4] = {up_sum.x, up_sum.y, up_sum.z, up_sum.w};
+            if constexpr (AROUND) {
+                if (square_tiles > 0) {                         // the rows of a were not divided by their rms yet
+                    float total = squares[0][r];
+#pragma unroll
+                    for (int other = 1; other < WAVES; ++other) total += squares[other][r];
+                    const float inv_rms = 1.0f / sqrtf(total / (float)norm.width_in + norm.eps);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { g[i] *= inv_rms; u[i] *= inv_rms; }
+                }
+            }
+            float fresh[4] = {0.f, 0.f, 0.f, 0.f};              // what out holds now, 0 outside of it
             if (mm < M) {
-                const float g[4] = {gate_sum.x, gate_sum.y, gate_sum.z, gate_sum.w};
-                const float u[4] = {up_sum.x, up_sum.y, up_sum.z, up_sum.w};
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     if (nn + i >= N) continue;
                     TO* dst = out + (long)mm * N + nn + i;
                     if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(g[i]);
-                    if constexpr (MODE == MODE_ACCUMULATE) *dst = from_float<TO>(to_float(*dst) + g[i]);
+                    if constexpr (MODE == MODE_ACCUMULATE) {
+                        float before;
+                        if constexpr (AROUND) before = out_ahead ? early_out[lane][i] : to_float(*dst);
+                        else before = to_float(*dst);
+                        fresh[i] = before + g[i];
+                        *dst = from_float<TO>(fresh[i]);
+                    }
                     if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(silu(g[i]) * u[i]);
+                }
+            }
+            if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
+                if (norm.squares_out) {
+                    float sum = fmaf(fresh[3], fresh[3], fmaf(fresh[2], fresh[2], fmaf(fresh[1], fresh[1], fresh[0] * fresh[0])));
+                    sum += __shfl_xor(sum, 16);
+                    sum += __shfl_xor(sum, 32);
+                    if (mm < M) {
+                        if (c == 0) norm.squares_out[(long)blockIdx.x * XRT_SQUARES_STRIDE + mm] = sum;
+                        bf16* scaled = (bf16*)norm.scaled_out + (long)mm * N + nn;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            if (nn + i >= N) continue;
+                            const float gain = norm.gain_dtype == XRT_F32 ? early_gain[c * 4 + i]
+                                                                          : to_float(((const bf16*)early_gain)[c * 4 + i]);
+                            scaled[i] = from_float<bf16>(fresh[i] * gain);
+                        }
+                    }
                 }
             }
         }
@@ -190,15 +302,28 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 }
 
 template <int MT, int RT, typename TO>
-int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, hipStream_t s) {
+int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
+                hipStream_t s) {
     const unsigned grid = (unsigned)((N + 16 * RT - 1) / (16 * RT));
     const dim3 block(WAVES * XRT_WAVE);
+    if constexpr (MT == 1 && RT == 1) {
+        if (norm.squares_in || norm.squares_out) {
+            if (mode == MODE_STORE)
+                gemm_skinny_kernel<1, 1, MODE_STORE, TO, true><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+            else if (mode == MODE_ACCUMULATE)
+                gemm_skinny_kernel<1, 1, MODE_ACCUMULATE, TO, true><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+            else
+                gemm_skinny_kernel<1, 1, MODE_GATED, TO, true><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+            XRT_LAUNCH_CHECK("linear (skinny, with norm)");
+            return 0;
+        }
+    }
     if (mode == MODE_STORE)
-        gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K);
+        gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
     else if (mode == MODE_ACCUMULATE)
-        gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K);
+        gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
     else if constexpr (RT == 1)
-        gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K);
+        gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
     else {
         xrt_set_error("linear (skinny): a gated product takes one row tile per wavefront");
         return 1;
@@ -208,14 +333,16 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
 }
 
 template <typename TO>
-int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, hipStream_t s) {
+int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
+                 hipStream_t s) {
     const int mt = (M + 15) / 16;
     // two row tiles per wavefront keep more loads in flight and halve the reads of x, if enough
     // workgroups remain to fill the chip
     // (with three or four tiles of x the reads of x from L2 outweigh those of w from HBM: then
     // the wider tile pays as soon as it leaves most compute units a workgroup)
-    const bool wide = mode != MODE_GATED && (N / 32) >= (mt >= 3 ? 160 : 1024);
-#define XRT_SKINNY(MT_) (wide ? launch_mode<MT_, 2, TO>(x, w, out, M, N, K, mode, s) : launch_mode<MT_, 1, TO>(x, w, out, M, N, K, mode, s))
+    const bool around = norm.squares_in || norm.squares_out;
+    const bool wide = !around && mode != MODE_GATED && (N / 32) >= (mt >= 3 ? 160 : 1024);
+#define XRT_SKINNY(MT_) (wide ? launch_mode<MT_, 2, TO>(x, w, out, M, N, K, mode, norm, s) : launch_mode<MT_, 1, TO>(x, w, out, M, N, K, mode, norm, s))
     switch (mt) {
         case 1: return XRT_SKINNY(1);
         case 2: return XRT_SKINNY(2);
@@ -232,8 +359,17 @@ bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K) {
     return M >= 1 && M <= 64 && K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
 }
 
+// The norm around a product needs one tile of x.
+bool xrt_linear_skinny_takes_norm(int M) { return M <= 16; }
+
 int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
-                      hipStream_t s) {
-    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, s);
-    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, s);
+                      const LinearNorm* norm, hipStream_t s) {
+    const LinearNorm none = {};
+    if (norm && !xrt_linear_skinny_takes_norm(M)) {
+        xrt_set_error("linear (skinny): the norm around a product takes at most 16 rows, found %d", M);
+        return 1;
+    }
+    const LinearNorm& around = norm ? *norm : none;
+    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, around, s);
+    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, around, s);
 }

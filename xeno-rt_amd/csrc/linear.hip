@@ -5,8 +5,9 @@
 int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
                      int mode, hipStream_t s);
 bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K);
+bool xrt_linear_skinny_takes_norm(int M);
 int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
-                      hipStream_t s);
+                      const xrt_linear_norm* norm, hipStream_t s);
 bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, int mode);
 int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                     hipStream_t s);
@@ -37,8 +38,32 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
             return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, workspace, (hipStream_t)stream);
     }
     if (dtype == XRT_BF16 && xrt_linear_skinny_accepts(a, w, M, K))
-        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
+        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, nullptr, (hipStream_t)stream);
     if (dtype == XRT_BF16 && xrt_linear_mfma_accepts(a, w, M, N, K, mode))
         return xrt_linear_mfma(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
     return xrt_linear_plain(a, w, dtype, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
+}
+
+extern "C" int xrt_linear_takes_norm(const void* a, const void* w, int dtype, int M, int N, int K, int mode) {
+    return dtype == XRT_BF16 && M >= 1 && N > 0 && K > 0 && mode >= 0 && mode <= 2 &&
+           xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_norm(M);
+}
+
+extern "C" int xrt_linear_normed(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N,
+                                 int K, int mode, const xrt_linear_norm* norm, void* stream) {
+    XRT_REQUIRE(a && w && out && norm, "linear with norm: null operand");
+    XRT_REQUIRE(xrt_linear_takes_norm(a, w, dtype, M, N, K, mode),
+                "linear with norm: M=%d N=%d K=%d of dtype %d is not a product that takes it", M, N, K, dtype);
+    XRT_REQUIRE(out_dtype == XRT_F32 || out_dtype == XRT_BF16, "linear with norm: unknown output dtype %d", out_dtype);
+    XRT_REQUIRE(mode != 1 || out_dtype == XRT_F32, "linear with norm: accumulation needs a float32 output");
+    if (norm->squares_in)
+        XRT_REQUIRE(norm->width_in == K && norm->tiles_in == (K + 15) / 16,
+                    "linear with norm: sums of squares of %d tiles over %d columns for a of %d columns",
+                    norm->tiles_in, norm->width_in, K);
+    if (norm->squares_out || norm->scaled_out || norm->gain) {
+        XRT_REQUIRE(mode == 1, "linear with norm: only an accumulating product writes what the norm after it needs");
+        XRT_REQUIRE(norm->squares_out && norm->scaled_out && norm->gain, "linear with norm: scaled_out, gain and squares_out come together");
+        XRT_REQUIRE(norm->gain_dtype == XRT_F32 || norm->gain_dtype == XRT_BF16, "linear with norm: unknown gain dtype %d", norm->gain_dtype);
+    }
+    return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, norm, (hipStream_t)stream);
 }

@@ -29,6 +29,22 @@ int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype
                int mode, float* workspace, long workspace_floats, void* stream);
 long xrt_linear_workspace(const void* a, const void* w, int dtype, int M, int N, int K, int mode);
 
+// An RMSNorm between two products, x += a w^T; y = rmsnorm(x) * gain; z = y v^T, without a kernel of
+// its own. The first product (mode 1) also writes scaled_out[m, n] = bfloat16(x[m, n] * gain[n]) and
+// squares_out[t * XRT_SQUARES_STRIDE + m], the sum of x[m, n]^2 over the 16 columns n of tile t. The
+// second takes scaled_out as its a, squares_in (tiles_in = ceil(width_in / 16) tiles) and multiplies its
+// rows by 1 / sqrt(sum of squares / width_in + eps) before its epilogue. A half left all zero is not done.
+// xrt_linear_takes_norm says whether a product can do this (bfloat16 operands, few rows); if not,
+// xrt_linear_normed refuses it.
+#define XRT_SQUARES_STRIDE 64
+typedef struct xrt_linear_norm {
+    const float* squares_in; int tiles_in; int width_in; float eps;
+    void* scaled_out; const void* gain; int gain_dtype; float* squares_out;
+} xrt_linear_norm;
+int xrt_linear_takes_norm(const void* a, const void* w, int dtype, int M, int N, int K, int mode);
+int xrt_linear_normed(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
+                      int mode, const xrt_linear_norm* norm, void* stream);
+
 // per-head RMSNorm of q and k (optional), rotation of q and k (optional), write of k and v
 // into the cache (optional); qkv rows are [q heads | k heads | v heads]. longest_run: the most
 // consecutive tokens that one sequence brings (0 if unknown); it only picks the faster way to

@@ -91,8 +91,16 @@ class DecoderModel:
         """Logits [len(batch.logit_rows), vocab] in float32 for the tokens of `batch`."""
         spec = self.spec
         x = spec.embedding.forward(batch.token_ids)
+        h = None            # the next block's first norm of x, where the block before it has made it already
         for index, call in enumerate(spec.schedule):
-            spec.layers[call.layer].forward(x, batch, cache.layer_cache(index))
+            block = spec.layers[call.layer]
+            if not getattr(block, "passes_norms", False):
+                block.forward(x, batch, cache.layer_cache(index))
+                h = None
+                continue
+            after = spec.layers[spec.schedule[index + 1].layer] if index + 1 < len(spec.schedule) else None
+            then = after.first_norm() if after is not None and getattr(after, "passes_norms", False) else None
+            h = block.forward(x, batch, cache.layer_cache(index), h=h, then=then)
         if batch.n_logit_rows == 0:
             return self.runtime.empty((0, spec.head.vocab), torch.float32)
         y = spec.final_norm.forward(x, rows=batch.logit_rows)

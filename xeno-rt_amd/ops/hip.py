@@ -8,7 +8,8 @@ from __future__ import annotations
 
 import ctypes
 import os
-from typing import Optional
+from dataclasses import dataclass
+from typing import Optional, Tuple
 
 import torch
 
@@ -29,6 +30,30 @@ def _code(tensor: torch.Tensor) -> int:
 
 def _ptr(tensor: Optional[torch.Tensor]):
     return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
+
+
+SQUARES_STRIDE = 64         # rows of a table of sums of squares (XRT_SQUARES_STRIDE of the library)
+
+
+@dataclass
+class Prescaled:
+    """Rows of the residual stream on their way through an RMSNorm whose division is still to do:
+    values[m, k] = bfloat16(x[m, k] * gain[k]) and squares[t, m] = the sum of x[m, k]^2 over the 16
+    columns k of tile t. `linear` and `linear_glu` take it in place of the normed rows and divide
+    the rows of their result by the rms; nothing else can read it."""
+    values: torch.Tensor
+    squares: torch.Tensor
+    eps: float
+
+    @property
+    def shape(self):
+        return self.values.shape
+
+
+class _LinearNorm(ctypes.Structure):
+    _fields_ = [("squares_in", ctypes.c_void_p), ("tiles_in", ctypes.c_int), ("width_in", ctypes.c_int),
+                ("eps", ctypes.c_float), ("scaled_out", ctypes.c_void_p), ("gain", ctypes.c_void_p),
+                ("gain_dtype", ctypes.c_int), ("squares_out", ctypes.c_void_p)]
 
 
 class HipOps:
@@ -57,7 +82,7 @@ class HipOps:
         self.path = path
         self.lib.xrt_last_error.restype = ctypes.c_char_p
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
-                     "xrt_attention", "xrt_sample"):
+                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_normed"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
 
@@ -112,7 +137,10 @@ class HipOps:
         self._check(self.lib.xrt_rmsnorm(_ptr(x), _ptr(weight), _code(weight), ctypes.c_float(eps), _ptr(out),
                                          _code(out), _ptr(rows), n_rows, hidden, self._stream(x)))
 
-    def _linear(self, a, w, out, mode, n):
+    def _linear(self, a, w, out, mode, n, then_norm=None):
+        scaled = a if isinstance(a, Prescaled) else None
+        if scaled is not None:
+            a = scaled.values
         if a.dim() != 2 or w.dim() != 2:
             raise KernelError("linear: operands must be [rows, k]")
         m, k = a.shape
@@ -121,13 +149,39 @@ class HipOps:
         if w.shape[1] != k:
             raise KernelError(f"linear: a has {k} columns, w has {w.shape[1]}")
         self._require(out, "linear out", None, (m, n), a)
-        need = int(self.lib.xrt_linear_workspace(_ptr(a), _ptr(w), _code(a), m, n, k, mode))
+        sizes = (_ptr(a), _ptr(w), _code(a))
+        # the norm after an accumulating product: only if that product, and one of the same rows
+        # over the n columns it writes, can take it
+        emit = None
+        if then_norm is not None and mode == 1 and n % 8 == 0 and self.lib.xrt_linear_takes_norm(*sizes, m, n, k, mode):
+            gain, eps = then_norm
+            self._require(gain, "norm gain", None, (n,), a)
+            emit = Prescaled(torch.empty((m, n), dtype=torch.bfloat16, device=a.device),
+                             torch.empty(((n + 15) // 16, SQUARES_STRIDE), dtype=torch.float32, device=a.device),
+                             float(eps))
+        if scaled is not None or emit is not None:
+            norm = _LinearNorm()
+            if scaled is not None:
+                tiles = (k + 15) // 16
+                self._require(scaled.squares, "sums of squares", torch.float32, (tiles, SQUARES_STRIDE), a)
+                norm.squares_in, norm.tiles_in, norm.width_in, norm.eps = scaled.squares.data_ptr(), tiles, k, scaled.eps
+            if emit is not None:
+                norm.scaled_out, norm.squares_out = emit.values.data_ptr(), emit.squares.data_ptr()
+                norm.gain, norm.gain_dtype = then_norm[0].data_ptr(), _code(then_norm[0])
+            self._check(self.lib.xrt_linear_normed(*sizes, _ptr(out), _code(out), m, n, k, mode, ctypes.byref(norm),
+                                                   self._stream(a)))
+            return emit
+        need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
-        self._check(self.lib.xrt_linear(_ptr(a), _ptr(w), _code(a), _ptr(out), _code(out), m, n, k, mode,
+        self._check(self.lib.xrt_linear(*sizes, _ptr(out), _code(out), m, n, k, mode,
                                         _ptr(workspace), ctypes.c_long(need), self._stream(a)))
+        return None
 
-    def linear(self, a, w, out, accumulate=False):
-        self._linear(a, w, out, 1 if accumulate else 0, w.shape[0])
+    def linear(self, a, w, out, accumulate=False, then_norm: Optional[Tuple[torch.Tensor, float]] = None):
+        """out (+)= a w^T. `a` may be a Prescaled. then_norm = (gain, eps) of an RMSNorm that follows an
+        accumulating product: if this product can, it returns a Prescaled of the updated `out` for the
+        product after the norm; None means that the caller runs the norm."""
+        return self._linear(a, w, out, 1 if accumulate else 0, w.shape[0], then_norm)
 
     def linear_glu(self, a, w_gate_up, out):
         if w_gate_up.shape[0] % 2 != 0:

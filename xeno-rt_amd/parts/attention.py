@@ -24,6 +24,8 @@ from .position import Rotary
 
 
 class Attention(Mixer):
+    passes_norms = True
+
     @property
     def capturable(self) -> bool:
         return self.position is None or self.position.capturable
@@ -82,7 +84,7 @@ class Attention(Mixer):
         if self.position is not None:
             self.position.bind(tensors, runtime)
 
-    def forward(self, h: torch.Tensor, batch, cache, residual: torch.Tensor) -> None:
+    def forward(self, h, batch, cache, residual: torch.Tensor, then=None):
         rt = self.runtime
         ops = rt.ops
         tokens = h.shape[0]
@@ -113,7 +115,8 @@ class Attention(Mixer):
 
         out = rt.empty((tokens, self.q_width))
         ops.attention(qkv, *dims, kv, batch, out, scale=self.scale, window=self.window)
-        ops.linear(out, self.w_o, residual, accumulate=True)
+        return ops.linear(out, self.w_o, residual, accumulate=True,
+                          then_norm=None if then is None else then.row_scale())
 
 
 register_part("mixer", "attention", Attention)

@@ -110,6 +110,14 @@ class Norm(Part):
         """Normalise the float32 rows of x (only `rows`, if given); result in the compute dtype."""
         raise NotImplementedError
 
+    def row_scale(self) -> Optional[Tuple[torch.Tensor, float]]:
+        """(gain, eps) if the norm is y = x / sqrt(mean(x^2) + eps) * gain over whole rows, None otherwise.
+
+        Such a norm between two matrix products can be done by the two of them (`then` below), which
+        saves a kernel where a step is short of work.
+        """
+        return None
+
 
 class PositionEncoding(Part):
     def apply(self, qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, batch) -> None:
@@ -118,6 +126,15 @@ class PositionEncoding(Part):
         qkv is [tokens, (n_heads + 2*n_kv_heads) * head_dim]: queries, then keys, then values.
         """
         raise NotImplementedError
+
+
+# A mixer, a feed-forward or a block may set `passes_norms = True`. It then promises two things.
+# Its `forward` takes a keyword `then`: the norm that follows it on the residual stream, or None. If
+# it can have its last product do that norm's work (`ops.linear(..., then_norm=then.row_scale())`),
+# it returns what that product returns, else None, and the caller runs the norm. And what it is
+# given as `h` may be such a returned object instead of a tensor: it hands `h` to `ops.linear` or
+# `ops.linear_glu` and reads nothing of it but `h.shape`. Parts without the attribute are called
+# as their interface below says and always get tensors.
 
 
 class Mixer(Part):
@@ -149,8 +166,17 @@ class Block(Part):
         return CacheNeeds()
 
     def forward(self, x: torch.Tensor, batch, cache) -> None:
-        """Update the float32 residual stream x [tokens, hidden] in place."""
+        """Update the float32 residual stream x [tokens, hidden] in place.
+
+        A block with `passes_norms` also takes `h`, the result of its first norm if the block before it
+        has already made it, and `then`, the first norm of the block after it, and returns that norm's
+        result or None.
+        """
         raise NotImplementedError
+
+    def first_norm(self) -> Optional[Norm]:
+        """The norm this block applies to the residual stream before anything else, if it starts with one."""
+        return None
 
 
 # ----------------------------------------------------------------------------

@@ -39,11 +39,27 @@ class PreNormBlock(Block):
         for part in self.parts():
             part.bind(tensors, runtime)
 
-    def forward(self, x, batch, cache) -> None:
-        h = self.mixer_norm.forward(x)
-        self.mixer.forward(h, batch, cache, x)
-        h = self.feed_forward_norm.forward(x)
+    @property
+    def passes_norms(self) -> bool:
+        return bool(getattr(self.mixer, "passes_norms", False))
+
+    def first_norm(self):
+        return self.mixer_norm
+
+    def forward(self, x, batch, cache, h=None, then=None):
+        if h is None:
+            h = self.mixer_norm.forward(x)
+        # a norm is left to the products around it only if the part after it reads nothing but products of it
+        if self.passes_norms and getattr(self.feed_forward, "passes_norms", False):
+            h = self.mixer.forward(h, batch, cache, x, then=self.feed_forward_norm)
+        else:
+            h = self.mixer.forward(h, batch, cache, x)
+        if h is None:
+            h = self.feed_forward_norm.forward(x)
+        if then is not None and getattr(self.feed_forward, "passes_norms", False):
+            return self.feed_forward.forward(h, batch, x, then=then)
         self.feed_forward.forward(h, batch, x)
+        return None
 
 
 register_part("block", "pre_norm", PreNormBlock)

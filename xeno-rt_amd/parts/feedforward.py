@@ -17,6 +17,7 @@ from .base import FeedForward, Runtime, WeightSpec, register_part
 
 class GatedMLP(FeedForward):
     capturable = True
+    passes_norms = True
 
     ACTIVATIONS = ("silu",)
 
@@ -45,12 +46,13 @@ class GatedMLP(FeedForward):
                                     runtime.matrix(tensors[p + "up_proj.weight"])], dim=0).contiguous()
         self.w_down = runtime.matrix(tensors[p + "down_proj.weight"])
 
-    def forward(self, h: torch.Tensor, batch, residual: torch.Tensor) -> None:
+    def forward(self, h, batch, residual: torch.Tensor, then=None):
         rt = self.runtime
         tokens = h.shape[0]
         act = rt.empty((tokens, self.intermediate))
         rt.ops.linear_glu(h, self.w_gate_up, act)
-        rt.ops.linear(act, self.w_down, residual, accumulate=True)
+        return rt.ops.linear(act, self.w_down, residual, accumulate=True,
+                             then_norm=None if then is None else then.row_scale())
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

@@ -28,6 +28,9 @@ class RMSNorm(Norm):
         super().bind(tensors, runtime)
         self.weight = runtime.vector(tensors[self.prefix + "weight"])
 
+    def row_scale(self):
+        return self.weight, self.eps
+
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         count = x.shape[0] if rows is None else rows.shape[0]
         out = self.runtime.empty((count, self.dim))
