@@ -48,11 +48,10 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     static_assert(!AROUND || (MT == 1 && RT == 1), "the norm around a product: one tile of x, one of w per wavefront");
     constexpr int WT = RT * (MODE == MODE_GATED ? 2 : 1);       // w tiles per wavefront
     constexpr int SQUARES_AHEAD = 8;                            // sums of squares a lane asks for when the kernel starts
-    __shared__ floatx4 partial[2][WAVES][XRT_WAVE];
+    __shared__ floatx4 partial[RT * MT > 1 ? 2 : 1][WAVES][XRT_WAVE];
     __shared__ float squares[WAVES][16];
-    // what the epilogue needs from global memory is asked for when the kernel starts and goes
-    // straight into LDS, past the registers: it is there when the stream of w has run through
-    __shared__ __attribute__((aligned(16))) float early_squares[AROUND ? WAVES : 1][SQUARES_AHEAD][XRT_WAVE];
+    // what the accumulating epilogue needs from global memory is asked for when the kernel starts and
+    // goes straight into LDS, past the registers: it is there when the stream of w has run through
     __shared__ floatx4 early_out[XRT_WAVE];
     __shared__ float early_gain[XRT_WAVE];
 
@@ -66,7 +65,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     const int k_end = min(K, k_begin + steps_per_wave * KSTEP);
 
     // CHAINS accumulators per output tile, used in turn and added at the end
-    constexpr int CHAINS = MT == 1 ? (AROUND && WT == 2 ? 2 : 4) : (MT == 2 ? 2 : 1);
+    constexpr int CHAINS = MT == 1 ? (AROUND && WT == 2 ? 3 : 4) : (MT == 2 ? 2 : 1);
     floatx4 chain[CHAINS][WT][MT];
 #pragma unroll
     for (int h = 0; h < CHAINS; ++h)
@@ -113,7 +112,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     // Whole steps of 128 along k run through a pipeline of two register sets: while the matrix
     // cores consume one step, the loads of the next are in flight. The steady-state loop body has
     // no branch; the last one or two steps are peeled off.
-    // The sums of squares of this wavefront's eighth of the tiles (lane (r, c): row r, every fourth tile from c).
+    // The sums of squares of this wavefront's eighth of the tiles (lane (r, c): row r, every fourth
+    // tile from c): the first ones are asked for now and added up when the stream of w has run through.
     const int square_tiles = AROUND && norm.squares_in ? norm.tiles_in : 0;
     const bool out_ahead = AROUND && MODE == MODE_ACCUMULATE && N % 4 == 0;     // 16 bytes of out per lane, aligned
     auto square_range = [&](int thread, int& first, int& end) {
@@ -121,18 +121,22 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
         first = thread / XRT_WAVE * per_wave + thread % XRT_WAVE / 16;
         end = min(square_tiles, (thread / XRT_WAVE + 1) * per_wave);
     };
+    float early_squares[AROUND ? SQUARES_AHEAD : 1] = {};
     if constexpr (AROUND) {
         if (square_tiles > 0) {
             int first, end;
             square_range(threadIdx.x, first, end);
+            const float* row = norm.squares_in + min(r, M - 1);
 #pragma unroll
             for (int i = 0; i < SQUARES_AHEAD; ++i) {
-                const int t = min(first + 4 * i, square_tiles - 1);
-                load_dword_to_lds(norm.squares_in, (unsigned)t * (XRT_SQUARES_STRIDE * 4u) + (unsigned)min(r, M - 1) * 4u,
-                                  __builtin_amdgcn_readfirstlane(lds_address(&early_squares[wave][i][0])));
+                const int t = first + 4 * i;
+                early_squares[i] = t < end ? row[(long)t * XRT_SQUARES_STRIDE] : 0.f;
             }
         }
-        if constexpr (MODE == MODE_ACCUMULATE) {
+    }
+    // (what the accumulating epilogue reads is asked for behind the first loads of w: those have the longer way)
+    auto ask_early = [&]() {
+        if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
             if (wave == 0) {                                    // the wavefront that writes the tile
                 if (out_ahead) {
                     const long column = min(n0 + c * 4, (long)N - 4);
@@ -145,12 +149,12 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                 }
             }
         }
-    }
+    };
     // (the lane's place is worked out again from the thread index, behind a fence for the compiler's
     // eyes, so that nothing of this is kept in registers while the stream of w runs)
     auto add_squares = [&]() {
         if constexpr (AROUND) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // what went to LDS has arrived
+            if constexpr (MODE == MODE_ACCUMULATE) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // what went to LDS has arrived
             if (square_tiles > 0) {
                 int thread = threadIdx.x;
                 asm volatile("" : "+v"(thread));
@@ -159,8 +163,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                 const int row = min(thread % 16, M - 1);
                 float sum = 0.f;
 #pragma unroll
-                for (int i = 0; i < SQUARES_AHEAD; ++i)
-                    sum += first + 4 * i < end ? early_squares[thread / XRT_WAVE][i][thread % XRT_WAVE] : 0.f;
+                for (int i = 0; i < SQUARES_AHEAD; ++i) sum += early_squares[i];
                 for (int t = first + 4 * SQUARES_AHEAD; t < end; t += 4)
                     sum += norm.squares_in[(long)t * XRT_SQUARES_STRIDE + row];
                 sum += __shfl_xor(sum, 16);
@@ -176,6 +179,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
         bf16x8 x_a[MT][4], x_b[MT][4];
         load_x(x_a, k_begin);
         load_w(w_a, k_begin);
+        ask_early();
         int i = 0;
         for (; i + 2 < full; i += 2) {
             load_x(x_b, k_begin + (i + 1) * KSTEP);
@@ -193,6 +197,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
         } else {
             multiply(w_a, x_a);
         }
+    } else {
+        ask_early();
     }
     // what is left of K when it is no multiple of 128: one guarded step, in the wavefront that owns it
     const int tail_begin = k_begin + full * KSTEP;
@@ -230,7 +236,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 #pragma unroll
     for (int tile = 0; tile < TILES; ++tile) {
         const int rt = tile / MT, m = tile % MT;
-        const int slot = tile & 1;
+        const int slot = RT * MT > 1 ? tile & 1 : 0;
         float4 gate_sum = {0.f, 0.f, 0.f, 0.f}, up_sum = {0.f, 0.f, 0.f, 0.f};
         constexpr int PASSES = MODE == MODE_GATED ? 2 : 1;
 #pragma unroll
@@ -262,17 +268,24 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                 }
             }
             float fresh[4] = {0.f, 0.f, 0.f, 0.f};              // what out holds now, 0 outside of it
-            if (mm < M) {
+            bool written = false;
+            if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
+                if (out_ahead && mm < M && nn < N) {            // the four values in one piece, as they came
+                    const floatx4 before = early_out[lane];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) fresh[i] = before[i] + g[i];
+                    *reinterpret_cast<floatx4*>(out + (long)mm * N + nn) = floatx4{fresh[0], fresh[1], fresh[2], fresh[3]};
+                    written = true;
+                }
+            }
+            if (mm < M && !written) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     if (nn + i >= N) continue;
                     TO* dst = out + (long)mm * N + nn + i;
                     if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(g[i]);
                     if constexpr (MODE == MODE_ACCUMULATE) {
-                        float before;
-                        if constexpr (AROUND) before = out_ahead ? early_out[lane][i] : to_float(*dst);
-                        else before = to_float(*dst);
-                        fresh[i] = before + g[i];
+                        fresh[i] = to_float(*dst) + g[i];
                         *dst = from_float<TO>(fresh[i]);
                     }
                     if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(silu(g[i]) * u[i]);
@@ -285,13 +298,15 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                     sum += __shfl_xor(sum, 32);
                     if (mm < M) {
                         if (c == 0) norm.squares_out[(long)blockIdx.x * XRT_SQUARES_STRIDE + mm] = sum;
-                        bf16* scaled = (bf16*)norm.scaled_out + (long)mm * N + nn;
+                        if (nn < N) {                           // N is a multiple of 8: all four or none
+                            struct alignas(8) Four { bf16 e[4]; } scaled;
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            if (nn + i >= N) continue;
-                            const float gain = norm.gain_dtype == XRT_F32 ? early_gain[c * 4 + i]
-                                                                          : to_float(((const bf16*)early_gain)[c * 4 + i]);
-                            scaled[i] = from_float<bf16>(fresh[i] * gain);
+                            for (int i = 0; i < 4; ++i) {
+                                const float gain = norm.gain_dtype == XRT_F32 ? early_gain[c * 4 + i]
+                                                                              : to_float(((const bf16*)early_gain)[c * 4 + i]);
+                                scaled.e[i] = from_float<bf16>(fresh[i] * gain);
+                            }
+                            *reinterpret_cast<Four*>((bf16*)norm.scaled_out + (long)mm * N + nn) = scaled;
                         }
                     }
                 }
