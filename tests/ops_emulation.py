@@ -74,6 +74,10 @@ class EmulatedOps:
         out.copy_(((gate / (1.0 + torch.exp(-gate))) * up).to(out.dtype))
 
     # -- attention --------------------------------------------------------------
+    def linear_qkv(self, a, w, qkv, *args, **kwargs):
+        self.linear(a, w, qkv)
+        self.qkv_prepare(qkv, *args, **kwargs)
+
     def qkv_prepare(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots,
                     q_norm=None, k_norm=None, norm_eps=0.0, rope_theta=None, rope_dim=0,
                     rope_scale=1.0, kv=None, longest_run=0):

@@ -270,6 +270,56 @@ def test_qkv_prepare_of_many_tokens(ops, dtype, nh, nkv, hd, rope_dim):
     assert int((kv_got.k != 0).any(-1).sum()) == (tokens - 1) * nkv
 
 
+@pytest.mark.parametrize("nh,nkv,hd,rope_dim,k,tokens", [(32, 8, 128, 128, 4096, 8), (4, 2, 64, 64, 200, 9), (3, 3, 48, 32, 96, 16),
+                                                          (2, 1, 256, 256, 72, 1), (5, 1, 16, 16, 64, 3), (4, 2, 64, 0, 128, 9),
+                                                          (4, 4, 80, 48, 264, 7)])
+def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens):
+    """The projection of a short step with the rotation and the cache write in its epilogue, against the two
+    kernels one after the other; without a norm before it and with one."""
+    positions = i32([0, 1, 63, 64, 65, 127, 128, 500, 1000, 2, 3, 4, 5, 6, 7, 8][:tokens])
+    slots = i32([0, 0, 0, 0, 1, 1, -1, 1, 0, 1, 1, 1, 1, 1, 1, 1][:tokens])                # one token is padding
+    width = (nh + 2 * nkv) * hd
+    a = rand(tokens, k, dtype=torch.bfloat16, seed=hd)
+    w = rand(width, k, dtype=torch.bfloat16, seed=k, scale=1.0 / math.sqrt(k))
+    kv = make_cache(40, nkv, hd, torch.bfloat16, 2, 16)
+    kv.block_table[0, :16] = torch.arange(3, 19, dtype=torch.int32)
+    kv.block_table[1, :16] = torch.arange(39, 23, -1, dtype=torch.int32)
+    theta = (torch.tensor(10000.0) ** (torch.arange(rope_dim // 2) * 2.0 / max(rope_dim, 1))).to(DEV) if rope_dim else None
+    args = dict(rope_theta=theta, rope_dim=rope_dim, rope_scale=0.5)
+    # the norm before the projection, handed over by the product before it
+    x = rand(tokens, k, seed=3, scale=2.0)
+    gain = (rand(k, seed=4) + 1.0).to(torch.bfloat16)
+    scaled = ops.linear(rand(tokens, 64, dtype=torch.bfloat16, seed=5), rand(k, 64, dtype=torch.bfloat16, seed=6), x,
+                        accumulate=True, then_norm=(gain, 1e-4))
+    assert scaled is not None
+    for rows in (a, scaled):
+        got = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
+        want = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
+        kv_got, kv_want = clone_cache(kv), clone_cache(kv)
+        ops.linear_qkv(rows, w, got, nh, nkv, hd, positions, slots, kv=kv_got, **args)
+        ops.linear(rows, w, want)
+        ops.qkv_prepare(want, nh, nkv, hd, positions, slots, kv=kv_want, **args)
+        # the same sums, roundings and formulas in both: at most the contraction of a multiply-add may differ
+        assert rel(got.float(), want.float()) < ULP["bfloat16"]
+        assert float((got.float() - want.float()).abs().gt(0).float().mean()) < 0.01
+        assert rel(kv_got.k.float(), kv_want.k.float()) < ULP["bfloat16"]
+        assert torch.equal(kv_got.v, kv_want.v)
+        assert int((kv_got.k != 0).any(-1).sum()) == int((slots >= 0).sum()) * nkv
+    # without a cache to write (a layer that reads another layer's), and with head norms (two kernels then)
+    got = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
+    want = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
+    ops.linear_qkv(a, w, got, nh, nkv, hd, positions, slots, **args)
+    ops.linear(a, w, want)
+    ops.qkv_prepare(want, nh, nkv, hd, positions, slots, **args)
+    assert rel(got.float(), want.float()) < ULP["bfloat16"]
+    qn, kn = rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0
+    kv_got, kv_want = clone_cache(kv), clone_cache(kv)
+    ops.linear_qkv(a, w, got, nh, nkv, hd, positions, slots, q_norm=qn, k_norm=kn, norm_eps=1e-4, kv=kv_got, **args)
+    ops.linear(a, w, want)
+    ops.qkv_prepare(want, nh, nkv, hd, positions, slots, q_norm=qn, k_norm=kn, norm_eps=1e-4, kv=kv_want, **args)
+    assert torch.equal(got, want) and torch.equal(kv_got.k, kv_want.k) and torch.equal(kv_got.v, kv_want.v)
+
+
 def test_rope_reference_vector_and_pairing(ops):
     # tests/kernels_test.rs:94-108: one head of 4, position 2, base 1e4 -> pairs (0,2), (1,3)
     qkv = torch.zeros(1, 3 * 16, device=DEV)

@@ -77,6 +77,17 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     for (int w = 0; w < waves; ++w) total += scratch[w];
     return total;
 }
+// ---- the cache ---------------------------------------------------------------------------
+// Element offset of the cache block that holds `pos` of sequence `slot`, for one key/value head;
+// -1 if there is none (padding, or a table entry that names no block).
+__device__ __forceinline__ long cache_block_base(const int* block_table, int table_stride, int n_blocks, int slot,
+                                                 int pos, int n_kv_heads, int kv_head, int head_dim) {
+    if (slot < 0) return -1;
+    const int block = block_table[(long)slot * table_stride + pos / XRT_BLOCK_TOKENS];
+    if (block < 0 || block >= n_blocks) return -1;
+    return ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * head_dim;
+}
+
 // ---- global memory -> LDS without passing registers (gfx950) ----------------------------------
 // 16 bytes per lane from global memory into LDS without passing registers: lane l of the
 // wavefront writes LDS byte address lds_base + 16 * l (lds_base is the same for the whole

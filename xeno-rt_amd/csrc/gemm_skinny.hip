@@ -20,8 +20,13 @@
 // bfloat16(x * gain) and, for every tile of 16 columns, each row's sum of squares; the product
 // after it takes those as its activations and multiplies its rows by 1 / sqrt(sum / width + eps).
 // The sums are added in a fixed order (tiles in eighths by wavefront, then wavefront by wavefront).
+//
+// The q/k/v projection of such a step can also rotate q and k and write k and v into the cache: a
+// tile of 16 rows of w is then the 8 + 8 rows of a head whose outputs the rotation pairs (dims d and
+// d + rope_dim / 2), so that a lane finds its partner 32 lanes away.
 #include "common.h"
 #include "xrt_hip.h"
+#include "gemm_skinny.h"
 
 namespace {
 
@@ -39,13 +44,16 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 // MT: tiles of 16 rows of x; RT: tiles of 16 rows of w per wavefront; GATED doubles the w tiles.
 // With one tile of x (the common decode case) the kernel is held to 128 registers, so that at
 // least two workgroups fit a compute unit: the stream from HBM needs the wavefronts in flight.
-// AROUND: the kernel also does its share of an RMSNorm before or after the product (one tile of x,
-// one tile of w per wavefront); kernels without it keep their registers for the stream.
-template <int MT, int RT, int MODE, typename TO, bool AROUND = false>
+// EXTRA 1: the kernel also does its share of an RMSNorm before or after the product (one tile of x,
+// one tile of w per wavefront); 2: and what follows a q/k/v projection. Kernels without keep their
+// registers for the stream.
+template <int MT, int RT, int MODE, typename TO, int EXTRA = 0>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skinny_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    const LinearNorm norm) {
+    const LinearNorm norm, const QkvAfter after) {
+    constexpr bool AROUND = EXTRA != 0, QKV = EXTRA == 2;
     static_assert(!AROUND || (MT == 1 && RT == 1), "the norm around a product: one tile of x, one of w per wavefront");
+    static_assert(!QKV || (MODE == MODE_STORE && sizeof(TO) == 2), "after a q/k/v projection: a bfloat16 store");
     constexpr int WT = RT * (MODE == MODE_GATED ? 2 : 1);       // w tiles per wavefront
     constexpr int SQUARES_AHEAD = 8;                            // sums of squares a lane asks for when the kernel starts
     __shared__ floatx4 partial[RT * MT > 1 ? 2 : 1][WAVES][XRT_WAVE];
@@ -54,10 +62,28 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     // goes straight into LDS, past the registers: it is there when the stream of w has run through
     __shared__ floatx4 early_out[XRT_WAVE];
     __shared__ float early_gain[XRT_WAVE];
+    // for the q/k/v epilogue, worked out while the first loads are on their way: cosine and sine of
+    // the lane's four angles, and where the lane's token lies in the cache
+    __shared__ float early_cos[QKV ? XRT_WAVE : 1][4], early_sin[QKV ? XRT_WAVE : 1][4];
+    __shared__ long early_base[QKV ? 16 : 1];
+    __shared__ int early_within[QKV ? 16 : 1];
 
     const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
     const int r = lane % 16, c = lane / 16;
     const long n0 = (long)blockIdx.x * (16 * RT);
+    // after a q/k/v projection: the tile's head, and the dims of the head its rows 0..7 and 8..15 make
+    int head = 0, lower_dim = 0, upper_dim = 8;
+    bool rotates = false;
+    if constexpr (QKV) {
+        const int tiles_per_head = after.head_dim / 16;
+        head = blockIdx.x / tiles_per_head;
+        const int s = blockIdx.x % tiles_per_head;
+        const bool is_value = head >= after.n_heads + after.n_kv_heads;
+        const int rotated_tiles = (after.rope_theta && !is_value) ? after.rope_dim / 16 : 0;
+        rotates = s < rotated_tiles;
+        lower_dim = rotates ? 8 * s : 16 * s;
+        upper_dim = rotates ? after.rope_dim / 2 + 8 * s : 16 * s + 8;
+    }
 
     const int steps = (K + KSTEP - 1) / KSTEP;
     const int steps_per_wave = (steps + WAVES - 1) / WAVES;
@@ -80,7 +106,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 #pragma unroll
     for (int t = 0; t < WT; ++t) {
         const int rt = t % RT, half = t / RT;                   // half 1: the "up" rows of a gated product
-        const long n = min(n0 + rt * 16 + r, (long)N - 1);
+        long n = min(n0 + rt * 16 + r, (long)N - 1);
+        if constexpr (QKV) n = (long)head * after.head_dim + (r < 8 ? lower_dim + r : upper_dim + r - 8);
         w_ptr[t] = w + (n + (long)half * N) * K + c * 8;
     }
     const bf16* x_ptr[MT];
@@ -136,6 +163,24 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     }
     // (what the accumulating epilogue reads is asked for behind the first loads of w: those have the longer way)
     auto ask_early = [&]() {
+        if constexpr (QKV) {
+            const int token = min(r, M - 1);
+            if (rotates && wave < 4) {                          // the lane's four angles, one per wavefront; read by wavefront 0
+                const float angle = (float)after.positions[token] * after.rope_scale / after.rope_theta[lower_dim + (c % 2) * 4 + wave];
+                sincosf(angle, &early_sin[lane][wave], &early_cos[lane][wave]);     // lanes c and c ^ 2 hold the two halves of a pair
+            }
+            if (wave == 4 && c == 0) {
+                const int pos = after.positions[token];
+                long base = -1;
+                if (after.k_cache && head >= after.n_heads) {
+                    const int kv_head = (head - after.n_heads) % after.n_kv_heads;
+                    base = cache_block_base(after.block_table, after.table_stride, after.n_blocks, after.slots[token],
+                                            pos, after.n_kv_heads, kv_head, after.head_dim);
+                }
+                early_base[r] = base;
+                early_within[r] = pos % XRT_BLOCK_TOKENS;
+            }
+        }
         if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
             if (wave == 0) {                                    // the wavefront that writes the tile
                 if (out_ahead) {
@@ -267,6 +312,41 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                     for (int i = 0; i < 4; ++i) { g[i] *= inv_rms; u[i] *= inv_rms; }
                 }
             }
+            if constexpr (QKV) {
+                // as the two-kernel way does it: the projection rounded to bfloat16, then rotated in float32
+                float mine[4], other[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    mine[i] = to_float(from_float<bf16>(g[i]));
+                    other[i] = __shfl_xor(mine[i], 32);
+                }
+                struct alignas(8) Four { bf16 e[4]; } packed;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float value = mine[i];
+                    if (rotates) {
+                        const float cosine = early_cos[lane][i], sine = early_sin[lane][i];
+                        value = c < 2 ? mine[i] * cosine - other[i] * sine : other[i] * sine + mine[i] * cosine;
+                    }
+                    packed.e[i] = from_float<bf16>(value);
+                }
+                if (mm < M) {
+                    const int dim = (c < 2 ? lower_dim : upper_dim) + (c % 2) * 4;
+                    *reinterpret_cast<Four*>((bf16*)out + (long)mm * N + (long)head * after.head_dim + dim) = packed;
+                    const long base = early_base[r];
+                    if (base >= 0) {
+                        const int within = early_within[r];
+                        if (head < after.n_heads + after.n_kv_heads) {
+                            *reinterpret_cast<Four*>(after.k_cache + base + (long)within * after.head_dim + dim) = packed;
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                after.v_cache[base + (long)(dim + i) * XRT_BLOCK_TOKENS + within] = packed.e[i];
+                        }
+                    }
+                }
+                continue;
+            }
             float fresh[4] = {0.f, 0.f, 0.f, 0.f};              // what out holds now, 0 outside of it
             bool written = false;
             if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
@@ -318,27 +398,38 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 
 template <int MT, int RT, typename TO>
 int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
-                hipStream_t s) {
+                const QkvAfter* after, hipStream_t s) {
     const unsigned grid = (unsigned)((N + 16 * RT - 1) / (16 * RT));
     const dim3 block(WAVES * XRT_WAVE);
+    const QkvAfter none = {};
     if constexpr (MT == 1 && RT == 1) {
-        if (norm.squares_in || norm.squares_out) {
+        if (after) {
+            if constexpr (sizeof(TO) == 2) {
+                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, *after);
+                XRT_LAUNCH_CHECK("linear (skinny, q/k/v)");
+                return 0;
+            }
+        } else if (norm.squares_in || norm.squares_out) {
             if (mode == MODE_STORE)
-                gemm_skinny_kernel<1, 1, MODE_STORE, TO, true><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
             else if (mode == MODE_ACCUMULATE)
-                gemm_skinny_kernel<1, 1, MODE_ACCUMULATE, TO, true><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+                gemm_skinny_kernel<1, 1, MODE_ACCUMULATE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
             else
-                gemm_skinny_kernel<1, 1, MODE_GATED, TO, true><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+                gemm_skinny_kernel<1, 1, MODE_GATED, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
             XRT_LAUNCH_CHECK("linear (skinny, with norm)");
             return 0;
         }
     }
+    if (after) {
+        xrt_set_error("linear (skinny): what follows a q/k/v projection takes one tile of bfloat16 rows");
+        return 1;
+    }
     if (mode == MODE_STORE)
-        gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+        gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
     else if (mode == MODE_ACCUMULATE)
-        gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+        gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
     else if constexpr (RT == 1)
-        gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm);
+        gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
     else {
         xrt_set_error("linear (skinny): a gated product takes one row tile per wavefront");
         return 1;
@@ -349,15 +440,15 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
 
 template <typename TO>
 int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
-                 hipStream_t s) {
+                 const QkvAfter* after, hipStream_t s) {
     const int mt = (M + 15) / 16;
     // two row tiles per wavefront keep more loads in flight and halve the reads of x, if enough
     // workgroups remain to fill the chip
     // (with three or four tiles of x the reads of x from L2 outweigh those of w from HBM: then
     // the wider tile pays as soon as it leaves most compute units a workgroup)
-    const bool around = norm.squares_in || norm.squares_out;
+    const bool around = norm.squares_in || norm.squares_out || after;
     const bool wide = !around && mode != MODE_GATED && (N / 32) >= (mt >= 3 ? 160 : 1024);
-#define XRT_SKINNY(MT_) (wide ? launch_mode<MT_, 2, TO>(x, w, out, M, N, K, mode, norm, s) : launch_mode<MT_, 1, TO>(x, w, out, M, N, K, mode, norm, s))
+#define XRT_SKINNY(MT_) (wide ? launch_mode<MT_, 2, TO>(x, w, out, M, N, K, mode, norm, after, s) : launch_mode<MT_, 1, TO>(x, w, out, M, N, K, mode, norm, after, s))
     switch (mt) {
         case 1: return XRT_SKINNY(1);
         case 2: return XRT_SKINNY(2);
@@ -377,14 +468,24 @@ bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K) {
 // The norm around a product needs one tile of x.
 bool xrt_linear_skinny_takes_norm(int M) { return M <= 16; }
 
+// So does what follows a q/k/v projection; and the rotation must pair whole groups of 8 dims.
+bool xrt_linear_skinny_takes_qkv(int M, int N, const QkvAfter& after) {
+    return M <= 16 && after.head_dim % 16 == 0 && N == (after.n_heads + 2 * after.n_kv_heads) * after.head_dim &&
+           (after.rope_theta == nullptr || (after.rope_dim % 16 == 0 && after.rope_dim <= after.head_dim));
+}
+
 int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
-                      const LinearNorm* norm, hipStream_t s) {
+                      const LinearNorm* norm, const QkvAfter* after, hipStream_t s) {
     const LinearNorm none = {};
     if (norm && !xrt_linear_skinny_takes_norm(M)) {
         xrt_set_error("linear (skinny): the norm around a product takes at most 16 rows, found %d", M);
         return 1;
     }
+    if (after && !(xrt_linear_skinny_takes_qkv(M, N, *after) && mode == MODE_STORE && out_dtype == XRT_BF16)) {
+        xrt_set_error("linear (skinny): M=%d N=%d mode %d is no q/k/v projection whose epilogue this kernel does", M, N, mode);
+        return 1;
+    }
     const LinearNorm& around = norm ? *norm : none;
-    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, around, s);
-    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, around, s);
+    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, around, after, s);
+    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, around, after, s);
 }

@@ -1,13 +1,10 @@
 // Entry point of all matrix products: checks the operands and picks the kernel.
 #include "common.h"
 #include "xrt_hip.h"
+#include "gemm_skinny.h"
 
 int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
                      int mode, hipStream_t s);
-bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K);
-bool xrt_linear_skinny_takes_norm(int M);
-int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
-                      const xrt_linear_norm* norm, hipStream_t s);
 bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, int mode);
 int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                     hipStream_t s);
@@ -38,7 +35,7 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
             return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, workspace, (hipStream_t)stream);
     }
     if (dtype == XRT_BF16 && xrt_linear_skinny_accepts(a, w, M, K))
-        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, nullptr, (hipStream_t)stream);
+        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, nullptr, nullptr, (hipStream_t)stream);
     if (dtype == XRT_BF16 && xrt_linear_mfma_accepts(a, w, M, N, K, mode))
         return xrt_linear_mfma(a, w, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
     return xrt_linear_plain(a, w, dtype, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
@@ -65,5 +62,32 @@ extern "C" int xrt_linear_normed(const void* a, const void* w, int dtype, void* 
         XRT_REQUIRE(norm->squares_out && norm->scaled_out && norm->gain, "linear with norm: scaled_out, gain and squares_out come together");
         XRT_REQUIRE(norm->gain_dtype == XRT_F32 || norm->gain_dtype == XRT_BF16, "linear with norm: unknown gain dtype %d", norm->gain_dtype);
     }
-    return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, norm, (hipStream_t)stream);
+    return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, norm, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int xrt_linear_qkv(const void* a, const void* w, int dtype, void* qkv, int M, int K,
+                              const xrt_linear_norm* norm, int n_heads, int n_kv_heads, int head_dim,
+                              const int* positions, const int* slots, const void* q_norm, const void* k_norm,
+                              int norm_dtype, float norm_eps, const float* rope_theta, int rope_dim,
+                              float rope_scale, void* k_cache, void* v_cache, const int* block_table,
+                              int table_stride, int n_blocks, int longest_run, float* workspace,
+                              long workspace_floats, void* stream) {
+    XRT_REQUIRE(n_heads > 0 && n_kv_heads > 0 && head_dim > 0, "linear_qkv: bad head sizes %d/%d x %d", n_heads, n_kv_heads, head_dim);
+    const int N = (n_heads + 2 * n_kv_heads) * head_dim;
+    if (M == 0) return 0;
+    // a decode step without head norms: one kernel does the product, the rotation and the cache write
+    QkvAfter after = {positions, slots, rope_theta, rope_dim, rope_scale, n_heads, n_kv_heads, head_dim,
+                      (bf16*)k_cache, (bf16*)v_cache, block_table, table_stride, n_blocks};
+    if (dtype == XRT_BF16 && a && w && qkv && M > 0 && K > 0 && !q_norm && !k_norm && positions &&
+        xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_qkv(M, N, after) &&
+        (uintptr_t)qkv % 8 == 0 && (uintptr_t)k_cache % 8 == 0 && (k_cache == nullptr) == (v_cache == nullptr) &&
+        (k_cache == nullptr || (block_table && slots && table_stride > 0 && n_blocks > 0)) &&
+        (rope_theta == nullptr || rope_dim > 0))
+        return xrt_linear_skinny(a, w, qkv, XRT_BF16, M, N, K, 0, norm, &after, (hipStream_t)stream);
+    const int status = norm ? xrt_linear_normed(a, w, dtype, qkv, dtype, M, N, K, 0, norm, stream)
+                            : xrt_linear(a, w, dtype, qkv, dtype, M, N, K, 0, workspace, workspace_floats, stream);
+    if (status != 0) return status;
+    return xrt_qkv_prepare(qkv, dtype, M, n_heads, n_kv_heads, head_dim, positions, slots, q_norm, k_norm, norm_dtype,
+                           norm_eps, rope_theta, rope_dim, rope_scale, k_cache, v_cache, block_table, table_stride,
+                           n_blocks, longest_run, stream);
 }

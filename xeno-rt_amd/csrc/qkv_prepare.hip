@@ -97,16 +97,6 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) qkv_prepare_kernel(
 }
 
 
-// Element offset of the cache block that holds `pos` of sequence `slot`, for one key/value head;
-// -1 if there is none (padding, or a table entry that names no block).
-__device__ __forceinline__ long cache_block_base(const int* block_table, int table_stride, int n_blocks, int slot,
-                                                 int pos, int n_kv_heads, int kv_head, int head_dim) {
-    if (slot < 0) return -1;
-    const int block = block_table[(long)slot * table_stride + pos / XRT_BLOCK_TOKENS];
-    if (block < 0 || block >= n_blocks) return -1;
-    return ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * head_dim;
-}
-
 template <typename T, int N> struct alignas(sizeof(T) * N) Pack { T e[N]; };
 
 // One workgroup per token. LANES lanes per head; head_dim = 2 * LANES * VEC with VEC elements in

@@ -56,6 +56,17 @@ int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, int n_kv_head
                     void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks,
                     int longest_run, void* stream);
 
+// The q/k/v projection qkv = a w^T followed by xrt_qkv_prepare (same arguments), in one kernel where a
+// decode step allows it (bfloat16, at most 16 rows, no head norms), else in two. norm: null, or the
+// squares_in half of an RMSNorm before the projection (then a is what xrt_linear_normed would take).
+// workspace as for xrt_linear.
+int xrt_linear_qkv(const void* a, const void* w, int dtype, void* qkv, int M, int K, const xrt_linear_norm* norm,
+                   int n_heads, int n_kv_heads, int head_dim, const int* positions, const int* slots,
+                   const void* q_norm, const void* k_norm, int norm_dtype, float norm_eps,
+                   const float* rope_theta, int rope_dim, float rope_scale,
+                   void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                   int longest_run, float* workspace, long workspace_floats, void* stream);
+
 // causal attention of every token of a step over its sequence's cache. The sequences of the
 // step may be described (seq_* arrays, n_seqs, the largest token count of a sequence and the
 // longest sequence after the step): then the matrix-core kernels can be used; decode needs a

@@ -82,7 +82,7 @@ class HipOps:
         self.path = path
         self.lib.xrt_last_error.restype = ctypes.c_char_p
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
-                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_normed"):
+                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_normed", "xrt_linear_qkv"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
 
@@ -188,8 +188,9 @@ class HipOps:
             raise KernelError("linear_glu: the weight needs gate rows followed by as many up rows")
         self._linear(a, w_gate_up, out, 2, w_gate_up.shape[0] // 2)
 
-    def qkv_prepare(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm=None, k_norm=None,
-                    norm_eps=0.0, rope_theta=None, rope_dim=0, rope_scale=1.0, kv=None, longest_run=0):
+    def _prepare_arguments(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm, k_norm, norm_eps,
+                           rope_theta, rope_dim, rope_scale, kv, longest_run):
+        """Checks the operands of qkv_prepare; returns the C arguments from n_heads to longest_run."""
         tokens = qkv.shape[0]
         width = (n_heads + 2 * n_kv_heads) * head_dim
         self._require(qkv, "qkv", None, (tokens, width))
@@ -208,11 +209,42 @@ class HipOps:
         stride = n_blocks = 0
         if kv is not None:
             k_cache, v_cache, table, stride, n_blocks = self._kv(kv, qkv, n_kv_heads, head_dim)
-        self._check(self.lib.xrt_qkv_prepare(
-            _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(positions), _ptr(slots),
-            _ptr(q_norm), _ptr(k_norm), norm_code, ctypes.c_float(norm_eps), _ptr(rope_theta), int(rope_dim),
-            ctypes.c_float(rope_scale), _ptr(k_cache), _ptr(v_cache), _ptr(table), stride, n_blocks,
-            int(longest_run), self._stream(qkv)))
+        return (n_heads, n_kv_heads, head_dim, _ptr(positions), _ptr(slots),
+                _ptr(q_norm), _ptr(k_norm), norm_code, ctypes.c_float(norm_eps), _ptr(rope_theta), int(rope_dim),
+                ctypes.c_float(rope_scale), _ptr(k_cache), _ptr(v_cache), _ptr(table), stride, n_blocks,
+                int(longest_run))
+
+    def qkv_prepare(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm=None, k_norm=None,
+                    norm_eps=0.0, rope_theta=None, rope_dim=0, rope_scale=1.0, kv=None, longest_run=0):
+        prepare = self._prepare_arguments(qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm, k_norm,
+                                          norm_eps, rope_theta, rope_dim, rope_scale, kv, longest_run)
+        self._check(self.lib.xrt_qkv_prepare(_ptr(qkv), _code(qkv), qkv.shape[0], *prepare, self._stream(qkv)))
+
+    def linear_qkv(self, a, w, qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm=None, k_norm=None,
+                   norm_eps=0.0, rope_theta=None, rope_dim=0, rope_scale=1.0, kv=None, longest_run=0):
+        """qkv = a w^T, then qkv_prepare of it: one kernel where a step is short enough. `a` may be a Prescaled."""
+        scaled = a if isinstance(a, Prescaled) else None
+        if scaled is not None:
+            a = scaled.values
+        if a.dim() != 2 or w.dim() != 2:
+            raise KernelError("linear_qkv: operands must be [rows, k]")
+        m, k = a.shape
+        self._require(a, "linear_qkv a")
+        self._require(w, "linear_qkv w", a.dtype, ((n_heads + 2 * n_kv_heads) * head_dim, k), a)
+        self._require(qkv, "qkv", a.dtype, (m, w.shape[0]), a)
+        prepare = self._prepare_arguments(qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm, k_norm,
+                                          norm_eps, rope_theta, rope_dim, rope_scale, kv, longest_run)
+        norm = None
+        if scaled is not None:
+            tiles = (k + 15) // 16
+            self._require(scaled.squares, "sums of squares", torch.float32, (tiles, SQUARES_STRIDE), a)
+            norm = _LinearNorm()
+            norm.squares_in, norm.tiles_in, norm.width_in, norm.eps = scaled.squares.data_ptr(), tiles, k, scaled.eps
+        need = int(self.lib.xrt_linear_workspace(_ptr(a), _ptr(w), _code(a), m, w.shape[0], k, 0))
+        workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
+        self._check(self.lib.xrt_linear_qkv(_ptr(a), _ptr(w), _code(a), _ptr(qkv), m, k,
+                                            None if norm is None else ctypes.byref(norm), *prepare,
+                                            _ptr(workspace), ctypes.c_long(need), self._stream(a)))
 
     def _kv(self, kv, like, n_kv_heads, head_dim):
         from ..cache import BLOCK_TOKENS

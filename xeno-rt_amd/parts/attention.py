@@ -90,15 +90,14 @@ class Attention(Mixer):
         tokens = h.shape[0]
         kv = cache.kv
         qkv = rt.empty((tokens, self.q_width + 2 * self.kv_width))
-        ops.linear(h, self.w_qkv, qkv)
 
         dims = (self.n_heads, self.n_kv_heads, self.head_dim)
         write_to = kv if cache.writable else None
         longest_run = int(getattr(batch, "max_count", 0) or 0)      # picks how the values are written; 0: unknown
         rotary = self.position if isinstance(self.position, Rotary) else None
         if rotary is not None or self.position is None:
-            # one pass: head norms, rotation, cache write
-            ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots,
+            # the projection, then in one pass (in the same kernel, where a step is short): head norms, rotation, cache write
+            ops.linear_qkv(h, self.w_qkv, qkv, *dims, batch.positions, batch.slots,
                             q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.qk_norm_eps,
                             rope_theta=None if rotary is None else rotary.theta,
                             rope_dim=0 if rotary is None else rotary.rope_dim,
@@ -106,6 +105,7 @@ class Attention(Mixer):
                             kv=write_to, longest_run=longest_run)
         else:
             # any other position encoding: norms, then the encoding, then the cache write
+            ops.linear(h, self.w_qkv, qkv)
             if self.qk_norm:
                 ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots,
                                 q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.qk_norm_eps)
