@@ -469,9 +469,11 @@ int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
 
 // ---- 17 to 64 rows of x: too many for the kernel that streams w through registers (it would read
 // x from L2 up to four times as often as w from HBM), too few for the tiles above to fill the chip.
-// Tiles of 64 x 128 take their x through LDS; k is split among workgroups until there are enough
-// of them to pull w at the rate of HBM; each writes float32 sums of its part of k to a workspace,
-// and a second kernel adds the parts in order and applies the epilogue.
+// Tiles of 64 x 128 take their x through LDS; k is split among workgroups as far as every compute
+// unit still gets at most one of them (one long stream per unit pulls w faster than several short
+// ones, measured); each writes float32 sums of its part of k to a workspace, and a second kernel
+// adds the parts in order and applies the epilogue. Where w has tiles enough without a split, the
+// tiles apply the epilogue themselves and there is no second kernel.
 // With more rows of x (up to a few hundred) the tiles of 128 x 128 do the same when they are too
 // few to fill the chip: such products are still bound by reading w.
 constexpr int SPLIT_BM = 64, SPLIT_BN = 128;
@@ -484,7 +486,7 @@ SplitPlan split_plan(int M, int N, int K, int mode) {
     const int units = K / 64;                                  // k is dealt out in pieces of 64
     int splits, least;                                         // least: pieces of k that a part should have
     if (M <= SPLIT_BM) {
-        splits = (int)((384 + tiles_n - 1) / tiles_n);         // about one and a half workgroups per compute unit
+        splits = (int)(256 / tiles_n);                         // one workgroup per compute unit, or fewer
         least = 1;
     } else {
         const long tiles = (long)((M + 127) / 128) * tiles_n;  // two of these workgroups share a compute unit
@@ -519,9 +521,17 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restri
 template <typename TO>
 int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, float* workspace, hipStream_t s) {
     const SplitPlan plan = split_plan(M, N, K, mode);
+    if (M <= SPLIT_BM && plan.splits == 1) {                   // tiles enough: each applies the epilogue itself
+        if (mode == MODE_STORE) return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s);
+        if (mode == MODE_GATED) return launch_kernel<SPLIT_BM, SPLIT_BN, 2, 2, MODE_GATED, 64, 3, TO>(a, w, out, M, N, K, 0, N, s);
+        if constexpr (sizeof(TO) == 4)
+            return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_ACCUMULATE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s);
+        XRT_REQUIRE(false, "linear (mfma): accumulation needs a float32 output");
+    }
+    XRT_REQUIRE(workspace != nullptr, "linear (mfma): a product split along k needs its workspace");
     // the product of all rows of w, ungated, into the workspace: [splits][M][rows_w]
     const int status = M <= SPLIT_BM
-        ? launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 32, 4, float>(
+        ? launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, float>(
               a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split)
         : launch_kernel<128, 128, 2, 2, MODE_STORE, 64, 2, float>(
               a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split);
@@ -547,14 +557,16 @@ int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int 
     return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, s);
 }
 
-// Floats of workspace with which a product runs split along k (17 to 64 rows of x, or more rows
-// and few tiles); 0 if this product does not take that path.
-long xrt_linear_split_workspace(const void* a, const void* w, int M, int N, int K, int mode) {
-    if (M <= 16 || K % 64 != 0 || K < 128 || !xrt_linear_mfma_accepts(a, w, M, N, K, mode)) return 0;
+// Whether a product runs through the tiles of this section (17 to 64 rows of x, or more rows and few
+// tiles), and the floats of workspace it then needs (0 where k is not split).
+bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats) {
+    *workspace_floats = 0;
+    if (M <= 16 || K % 64 != 0 || K < 128 || !xrt_linear_mfma_accepts(a, w, M, N, K, mode)) return false;
     const SplitPlan plan = split_plan(M, N, K, mode);
-    if (M > SPLIT_BM && plan.splits == 1) return 0;            // enough tiles without a split: the kernels above
-    if (plan.rows_w * (long)M >= (1L << 31)) return 0;
-    return (long)plan.splits * M * plan.rows_w;
+    if (plan.splits == 1) return M <= SPLIT_BM;               // more rows and enough tiles without a split: the kernels above
+    if (plan.rows_w * (long)M >= (1L << 31)) return false;
+    *workspace_floats = (long)plan.splits * M * plan.rows_w;
+    return true;
 }
 
 int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,

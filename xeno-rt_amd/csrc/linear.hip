@@ -9,13 +9,15 @@ bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, 
 int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                     hipStream_t s);
 
-long xrt_linear_split_workspace(const void* a, const void* w, int M, int N, int K, int mode);
+bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats);
 int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                      float* workspace, hipStream_t s);
 
 extern "C" long xrt_linear_workspace(const void* a, const void* w, int dtype, int M, int N, int K, int mode) {
+    long need = 0;
     if (dtype != XRT_BF16 || M <= 0 || N <= 0 || K <= 0 || mode < 0 || mode > 2) return 0;
-    return xrt_linear_split_workspace(a, w, M, N, K, mode);
+    xrt_linear_split_takes(a, w, M, N, K, mode, &need);
+    return need;
 }
 
 extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N,
@@ -29,9 +31,9 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
     XRT_REQUIRE(a && w && out, "linear: null operand");
     if (M == 0) return 0;
     // bfloat16: the matrix-core kernels; float32, and shapes they refuse: the plain kernel
-    if (dtype == XRT_BF16 && workspace != nullptr) {
-        const long need = xrt_linear_split_workspace(a, w, M, N, K, mode);
-        if (need > 0 && workspace_floats >= need)
+    if (dtype == XRT_BF16) {
+        long need = 0;
+        if (xrt_linear_split_takes(a, w, M, N, K, mode, &need) && (need == 0 || (workspace != nullptr && workspace_floats >= need)))
             return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, workspace, (hipStream_t)stream);
     }
     if (dtype == XRT_BF16 && xrt_linear_skinny_accepts(a, w, M, K))
