@@ -221,3 +221,61 @@ def test_engine_conveniences(pair):
     assert table.device.type == "cpu" and tuple(table.shape) == (engine.config.vocab_size, engine.config.hidden_size)
     with pytest.raises(KeyError):
         engine.get_tensor("model.no_such.weight")
+
+
+def test_norms_are_handed_to_the_products_only_where_every_part_agrees(pair, tmp_path):
+    """A norm between two products may be done by them (parts with `passes_norms`); the result is the same
+    with and without, and a part that does not say so is never given anything but tensors."""
+    from xeno_rt_amd.parts.base import FeedForward
+
+    engine, plain = pair
+    ids = [5, 9, 2, 7, 11, 3]
+    want = engine.step([(engine.alloc_slot(), ids, list(range(len(ids))))])
+    engine.free_slot(0)
+
+    handed = []
+    ops = EmulatedOps()
+    plain_linear = ops.linear
+
+    def watching_linear(a, w, out, accumulate=False, then_norm=None):
+        handed.append((isinstance(a, EmulatedOps.Prescaled), then_norm is not None))
+        return plain_linear(a, w, out, accumulate=accumulate, then_norm=then_norm)
+
+    ops.linear = watching_linear
+    folder = make_folder(TINY["llama"], tmp_path, seed=4, std=0.2)
+    watched = Engine.load(folder, dtype="float32", device="cpu", ops=ops, max_tokens=64 * 6, max_slots=3)
+    got = watched.step([(watched.alloc_slot(), ids, list(range(len(ids))))])
+    assert torch.allclose(got, want, rtol=0, atol=1e-5 * float(want.abs().max()))
+    layers = len(watched.model.spec.layers)
+    # per layer: o is followed by the feed-forward's norm, down by the next layer's first norm (the last by none)
+    assert sum(1 for _, then in handed if then) == 2 * layers - 1
+    # every layer but the first takes its q/k/v projection's rows from the layer before (gate/up, which takes them
+    # from o, goes through linear_glu); the output head takes a tensor
+    assert sum(1 for scaled, _ in handed if scaled) == layers - 1
+
+    # a feed-forward that does not promise: it is called without `then`, gets a tensor, and the block runs both norms
+    class Opaque(FeedForward):
+        capturable = True
+
+        def __init__(self, inner):
+            self.inner = inner
+
+        def weight_specs(self):
+            return self.inner.weight_specs()
+
+        def bind(self, tensors, runtime):
+            self.inner.bind(tensors, runtime)
+
+        def forward(self, h, batch, residual):
+            assert isinstance(h, torch.Tensor)
+            self.inner.forward(h, batch, residual)
+
+    watched.free_slot(0)
+    block = watched.model.spec.layers[0]
+    block.feed_forward = Opaque(block.feed_forward)
+    handed.clear()
+    again = watched.step([(watched.alloc_slot(), ids, list(range(len(ids))))])
+    assert torch.allclose(again, want, rtol=0, atol=1e-5 * float(want.abs().max()))
+    # layer 0's o is no longer followed by a handed norm, and nothing is handed on behind its down
+    assert sum(1 for _, then in handed if then) == 2 * layers - 1 - 2
+    assert sum(1 for scaled, _ in handed if scaled) == layers - 2
