@@ -138,7 +138,8 @@ class EmulatedOps:
                 out[t, head * head_dim:(head + 1) * head_dim] = (probs @ values[:, kvh, :]).to(out.dtype)
 
     # -- sampling ---------------------------------------------------------------
-    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms):
+    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms,
+               small_top_k=False):
         rows, vocab = logits.shape
         for r in range(rows):
             row = logits[r].to(torch.float32).clone()

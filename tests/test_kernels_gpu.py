@@ -507,9 +507,15 @@ def sample(ops, logits, temperature=0.0, top_k=0, top_p=1.0, penalty=1.0, histor
     offsets = i32([len(history) * r for r in range(rows + 1)])
     out = torch.empty(rows, dtype=torch.int32, device=DEV)
     uniforms = torch.tensor(draws if draws is not None else [0.5] * rows, dtype=torch.float32, device=DEV)
-    ops.sample(logits, out, f(temperature), torch.full((rows,), top_k, dtype=torch.int32, device=DEV), f(top_p),
-               f(penalty), i32(list(history) * rows), offsets, uniforms)
-    return out.tolist()
+    operands = (logits, out, f(temperature), torch.full((rows,), top_k, dtype=torch.int32, device=DEV), f(top_p),
+                f(penalty), i32(list(history) * rows), offsets, uniforms)
+    ops.sample(*operands)
+    picked = out.tolist()
+    # the way through slices (taken by rows with a small top-k, where the vocabulary is large enough) picks the same
+    out.fill_(-1)
+    ops.sample(*operands, small_top_k=True)
+    assert out.tolist() == picked
+    return picked
 
 
 def test_sample_reference_cases(ops):

@@ -14,6 +14,12 @@
 // is gathered into LDS (if it fits) and top-p and the CDF work on that short list; only without
 // a top-k do they pass over the whole row. A workgroup is one compute unit, so a pass is bound by
 // how many loads it keeps in flight: sixteen per thread.
+//
+// A small top-k (up to 64, the usual case) does not pass over the row eight times: the row is cut
+// into slices of 4096 tokens, a workgroup per slice holds its slice in registers and finds the
+// slice's own k largest (ties included), and the row's workgroup then works on those few
+// candidates only: the row's k largest are among them. Slices whose ties overflow their list send the
+// row back to the path above.
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -65,8 +71,9 @@ constexpr int SUMS = 17;               // most values that block_sums adds at on
 // Sums over the block of N values per thread; every thread gets the sums. The order of the
 // additions is fixed: lanes in a tree, then wavefronts in order. `scratch` holds
 // (BLOCK_WAVES + 1) * SUMS values.
-template <typename T, int N>
+template <typename T, int N, int WAVES_ = BLOCK_WAVES>
 __device__ __forceinline__ void block_sums(T (&v)[N], T* scratch) {
+    constexpr int BLOCK_WAVES = WAVES_;
     static_assert(N <= SUMS, "scratch too small");
     const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
 #pragma unroll
@@ -88,11 +95,12 @@ __device__ __forceinline__ void block_sums(T (&v)[N], T* scratch) {
     for (int j = 0; j < N; ++j) v[j] = scratch[BLOCK_WAVES * N + j];
 }
 
-__global__ void __launch_bounds__(THREADS) sample_kernel(
+// The whole of it for row r, by one workgroup of THREADS threads; `seen` holds vocab bits of LDS.
+__device__ void sample_row(
+    const int r, unsigned* seen,
     const float* __restrict__ logits, int vocab, int* __restrict__ out, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ penalty,
     const int* __restrict__ history, const int* __restrict__ history_offsets, const float* __restrict__ uniforms) {
-    extern __shared__ unsigned seen[];                 // vocab bits
     __shared__ float scratch_f[(BLOCK_WAVES + 1) * SUMS];
     __shared__ unsigned scratch_u[(BLOCK_WAVES + 1) * SUMS];
     __shared__ int survivor_id[BLOCK_WAVES * SEGMENT];      // what top-k leaves, by wavefront run, in the order of ids
@@ -103,7 +111,7 @@ __global__ void __launch_bounds__(THREADS) sample_kernel(
     __shared__ float target_in_wave;
     __shared__ int chosen_wave, chosen;
 
-    const int r = blockIdx.x, tid = threadIdx.x;
+    const int tid = threadIdx.x;
     const int lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
     Row row;
     row.logits = logits + (long)r * vocab;
@@ -393,11 +401,342 @@ __global__ void __launch_bounds__(THREADS) sample_kernel(
     if (tid == 0) out[r] = chosen >= 0 ? chosen : best_index;   // sampler.rs:195: fall back to the top candidate
 }
 
+__global__ void __launch_bounds__(THREADS) sample_kernel(
+    const float* __restrict__ logits, int vocab, int* __restrict__ out, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ penalty,
+    const int* __restrict__ history, const int* __restrict__ history_offsets, const float* __restrict__ uniforms) {
+    extern __shared__ unsigned seen[];                 // vocab bits
+    sample_row(blockIdx.x, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms);
+}
+
+// ---- a small top-k: candidates by slice, then the row ---------------------------------------------
+constexpr int SLICE = 4096;            // tokens of a slice
+constexpr int SLICE_THREADS = 256;
+constexpr int SLICE_WAVES = SLICE_THREADS / XRT_WAVE;
+constexpr int SLICE_EACH = SLICE / SLICE_THREADS;
+constexpr int SLICE_HOLDS = 128;       // candidates that a slice can hand on
+constexpr int FAST_TOP_K = 64;         // the largest top-k that goes this way
+constexpr int MOST_SLICES = (MAX_VOCAB + SLICE - 1) / SLICE;
+constexpr int ROW_HOLDS = THREADS;     // survivors of the row's top-k that the row's workgroup can hold: one per thread
+
+constexpr int SLICE_TOPS = 8;          // of a slice's largest values, one per thread that holds them, what it hands on apart
+constexpr int LEAST_SLICES = 8;        // with fewer slices their tops are too few to bound a top-k of FAST_TOP_K
+
+struct SliceCandidates {
+    int count;                         // -1: this row does not go this way; more than SLICE_HOLDS: they did not fit
+    int unused[3];
+    unsigned top[SLICE_TOPS];          // keys of SLICE_TOPS different tokens of the slice, the largest first (0: none)
+    int id[SLICE_HOLDS];
+    float value[SLICE_HOLDS];          // after the penalty
+};
+
+__device__ __forceinline__ bool goes_by_slices(float temperature, int k, int vocab) {
+    return temperature > 1e-5f && k > 0 && k <= FAST_TOP_K && k < vocab;
+}
+
+// How many of the block's threads hold a larger maximum than this one (ties: lower thread first): the
+// place of the thread's maximum among all. The thread in place k - 1 holds a lower bound of the k-th
+// largest of all keys of the block (there are k keys at or above it, one in each of k threads); what
+// lies at or above the bound is a short list, in which the exact place can then be looked for.
+// `mine` is the thread's largest key (0: it holds none).
+template <int THREADS_>
+__device__ __forceinline__ int place_of_maximum(unsigned mine, unsigned* maxima) {
+    maxima[threadIdx.x] = mine;
+    __syncthreads();
+    int larger = 0;
+    for (int j = 0; j < THREADS_; j += 4) {
+        const uint4 other = *reinterpret_cast<const uint4*>(&maxima[j]);
+        larger += other.x > mine || (other.x == mine && j + 0 < (int)threadIdx.x) ? 1 : 0;
+        larger += other.y > mine || (other.y == mine && j + 1 < (int)threadIdx.x) ? 1 : 0;
+        larger += other.z > mine || (other.z == mine && j + 2 < (int)threadIdx.x) ? 1 : 0;
+        larger += other.w > mine || (other.w == mine && j + 3 < (int)threadIdx.x) ? 1 : 0;
+    }
+    return larger;
+}
+
+__global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
+    const float* __restrict__ logits, int vocab, const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ penalty, const int* __restrict__ history, const int* __restrict__ history_offsets,
+    SliceCandidates* __restrict__ candidates, int slices) {
+    __shared__ unsigned seen[SLICE / 32];
+    __shared__ __attribute__((aligned(16))) unsigned maxima[SLICE_THREADS];
+    __shared__ unsigned bound;
+    __shared__ int held;
+    const int r = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
+    SliceCandidates& mine = candidates[(long)r * slices + slice];
+    const int k = top_k[r];
+    if (!goes_by_slices(temperature[r], k, vocab)) {
+        if (tid == 0) mine.count = -1;
+        return;
+    }
+    const int first = slice * SLICE;
+    const float factor = penalty[r];
+    const int h_begin = history_offsets[r], h_end = history_offsets[r + 1];
+    const bool penalised = factor > 1.0f && h_end > h_begin;
+    if (tid < SLICE / 32) seen[tid] = 0u;
+    if (tid == 0) held = 0;
+    __syncthreads();
+    if (penalised) {
+        for (int i = h_begin + tid; i < h_end; i += SLICE_THREADS) {
+            const int token = history[i] - first;
+            if (token >= 0 && token < SLICE && token + first < vocab) atomicOr(&seen[token >> 5], 1u << (token & 31));
+        }
+        __syncthreads();
+    }
+    // thread t holds tokens first + e * 256 + t
+    float value[SLICE_EACH];
+    unsigned key[SLICE_EACH];
+    const float* row = logits + (long)r * vocab;
+#pragma unroll
+    for (int e = 0; e < SLICE_EACH; ++e) value[e] = row[min(first + e * SLICE_THREADS + tid, vocab - 1)];
+#pragma unroll
+    for (int e = 0; e < SLICE_EACH; ++e) {
+        const int local = e * SLICE_THREADS + tid;
+        const float v = value[e];
+        const float changed = v > 0.f ? v / factor : v * factor;
+        value[e] = (seen[local >> 5] >> (local & 31)) & 1u ? changed : v;
+        // key 0 stands for "no token"; no float maps to it but a NaN with all bits set, which can go without loss
+        key[e] = first + local < vocab ? order_key(value[e]) : 0u;
+    }
+    unsigned largest = 0u;
+#pragma unroll
+    for (int e = 0; e < SLICE_EACH; ++e) largest = max(largest, key[e]);
+    const int place = place_of_maximum<SLICE_THREADS>(largest, maxima);
+    if (place == k - 1) bound = largest;                // 0 if fewer than k threads hold a token
+    if (place < SLICE_TOPS) mine.top[place] = largest;
+    __syncthreads();
+    const unsigned threshold = bound;
+#pragma unroll
+    for (int e = 0; e < SLICE_EACH; ++e) {
+        if (key[e] != 0u && key[e] >= threshold) {
+            const int at = atomicAdd(&held, 1);
+            if (at < SLICE_HOLDS) {
+                mine.id[at] = first + e * SLICE_THREADS + tid;
+                mine.value[at] = value[e];
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) mine.count = held;
+}
+
+__global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
+    const float* __restrict__ logits, int vocab, int* __restrict__ out, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ penalty,
+    const int* __restrict__ history, const int* __restrict__ history_offsets, const float* __restrict__ uniforms,
+    const SliceCandidates* __restrict__ candidates, int slices) {
+    extern __shared__ unsigned seen[];                 // vocab bits, for the rows that take the whole-row path
+    __shared__ float scratch_f[(BLOCK_WAVES + 1) * SUMS];
+    __shared__ int first_place[MOST_SLICES + 1];
+    __shared__ unsigned bound, exact;
+    __shared__ int kept_id[ROW_HOLDS];
+    __shared__ float kept_value[ROW_HOLDS];
+    __shared__ int sorted_id[ROW_HOLDS];
+    __shared__ float sorted_weight[ROW_HOLDS];
+    __shared__ int kept, survivors;
+    static_assert(MOST_SLICES <= XRT_WAVE, "one lane per slice");
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const SliceCandidates* mine = candidates + (long)r * slices;
+    // where every slice's candidates start in the row's list (one lane per slice; an inclusive sum over the
+    // lanes); a slice that says "not this way" or "they did not fit" sends the row to the whole-row path
+    const int k = top_k[r];
+    if (tid < XRT_WAVE) {
+        const int count = tid < slices ? mine[tid].count : 0;
+        const bool bad = count < 0 || count > SLICE_HOLDS;
+        int through = max(count, 0);
+#pragma unroll
+        for (int offset = 1; offset < XRT_WAVE; offset <<= 1) {
+            const int below = __shfl_up(through, offset, XRT_WAVE);
+            if (tid >= offset) through += below;
+        }
+        if (tid < slices) first_place[tid + 1] = through;
+        if (tid == 0) { first_place[0] = 0; kept = 0; survivors = 0; bound = 0u; }
+        if (__ballot(bad) != 0ull) {
+            if (tid == 0) first_place[0] = -1;
+        } else {
+            // A lower bound of the row's k-th largest key: the k-th largest of the slices' tops, which are all
+            // different tokens. A lane holds two of them; `depth` per slice make at least FAST_TOP_K in all.
+            const int depth = min(SLICE_TOPS, 2 * XRT_WAVE / slices);
+            unsigned held[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int slot = tid + h * XRT_WAVE;
+                held[h] = slot < slices * depth ? mine[slot / depth].top[slot % depth] : 0u;
+            }
+            int before[2] = {0, 0};                             // tops that come before this one (ties: lower slot first)
+            for (int j = 0; j < XRT_WAVE; ++j) {
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    const unsigned other = __shfl(held[g], j, XRT_WAVE);
+                    const int other_slot = j + g * XRT_WAVE;
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        before[h] += other > held[h] || (other == held[h] && other_slot < tid + h * XRT_WAVE) ? 1 : 0;
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                if (before[h] == k - 1) bound = held[h];        // 0 if fewer than k tops exist
+        }
+    }
+    __syncthreads();
+    if (first_place[0] < 0) {                                   // the same for all threads
+        __syncthreads();
+        sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms);
+        return;
+    }
+    const int total = first_place[slices];
+    // thread t holds candidates t, t + THREADS, ...: at most MOST_SLICES * SLICE_HOLDS / THREADS of them
+    constexpr int EACH = (MOST_SLICES * SLICE_HOLDS + THREADS - 1) / THREADS;
+    float value[EACH];
+    int id[EACH];
+    unsigned key[EACH];
+#pragma unroll
+    for (int e = 0; e < EACH; ++e) {
+        const int place = e * THREADS + tid;
+        key[e] = 0u; value[e] = 0.f; id[e] = 0;
+        if (place < total) {
+            int s = 0;
+            while (first_place[s + 1] <= place) ++s;            // few slices; places of a wavefront share most of the walk
+            const int within = place - first_place[s];
+            value[e] = mine[s].value[within];
+            id[e] = mine[s].id[within];
+            key[e] = order_key(value[e]);
+        }
+    }
+    // what lies at or above the lower bound of the k-th largest goes to a list ...
+    const unsigned at_least = bound;
+#pragma unroll
+    for (int e = 0; e < EACH; ++e) {
+        if (key[e] != 0u && key[e] >= at_least) {
+            const int place = atomicAdd(&kept, 1);
+            if (place < ROW_HOLDS) { kept_id[place] = id[e]; kept_value[place] = value[e]; }
+        }
+    }
+    __syncthreads();
+    const int listed = kept;
+    if (listed > ROW_HOLDS) {                                   // ties by the thousand
+        __syncthreads();
+        sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms);
+        return;
+    }
+    // ... in which the k-th largest is the one that k - 1 others come before (ties: lower id first); it and
+    // all that tie with it stay, as on the whole row
+    const unsigned my_key = tid < listed ? order_key(kept_value[tid]) : 0u;
+    const int my_id = tid < listed ? kept_id[tid] : 0;
+    if (tid < listed) {
+        int before = 0;
+        for (int j = 0; j < listed; ++j) {
+            const unsigned other = order_key(kept_value[j]);
+            before += other > my_key || (other == my_key && kept_id[j] < my_id) ? 1 : 0;
+        }
+        if (before == min(k, listed) - 1) exact = my_key;
+    }
+    __syncthreads();
+    const bool survives = tid < listed && my_key >= exact;
+    if (survives) atomicAdd(&survivors, 1);
+    __syncthreads();
+    const int n = survivors;
+    // the survivors in the order of their ids: a survivor's place is the number of survivors with smaller ids
+    float best = -INFINITY;
+    for (int j = 0; j < listed; ++j) best = fmaxf(best, kept_value[j]);
+    const float inv_temp = 1.0f / temperature[r];
+    float weight = 0.f;
+    if (survives) {
+        int place = 0;
+        for (int j = 0; j < listed; ++j) place += order_key(kept_value[j]) >= exact && kept_id[j] < my_id ? 1 : 0;
+        weight = expf((kept_value[tid] - best) * inv_temp);
+        sorted_id[place] = my_id;
+        sorted_weight[place] = weight;
+    }
+    __syncthreads();
+    const float p = top_p[r];
+    if (n <= XRT_WAVE) {
+        // the usual case: one wavefront holds them all, lane j the j-th in the order of ids
+        if (tid >= XRT_WAVE) return;
+        const float w = tid < n ? sorted_weight[tid] : 0.f;
+        float w_threshold = 0.f;
+        if (p < 1.0f) {
+            // the largest weight whose own and all larger weights together reach p of the total, sums in lane order
+            float all = 0.f, with_larger = 0.f;
+            for (int j = 0; j < n; ++j) {
+                const float other = __shfl(w, j, XRT_WAVE);
+                all += other;
+                with_larger += other >= w ? other : 0.f;
+            }
+            float reaches = tid < n && with_larger >= p * all ? w : 0.f;
+#pragma unroll
+            for (int offset = XRT_WAVE / 2; offset > 0; offset >>= 1) reaches = fmaxf(reaches, __shfl_xor(reaches, offset, XRT_WAVE));
+            w_threshold = fminf(reaches, 1.0f);
+        }
+        const float mine_kept = w >= w_threshold ? w : 0.f;
+        float sum = 0.f;
+        for (int j = 0; j < n; ++j) sum += __shfl(mine_kept, j, XRT_WAVE);
+        const float target = uniforms[r] * sum;
+        float running = 0.f;
+        int pick = -1, last_kept = -1;
+        for (int j = 0; j < n; ++j) {                           // every lane walks the same list: lane order is id order
+            const float x = __shfl(mine_kept, j, XRT_WAVE);
+            if (x > 0.f && pick < 0) {
+                last_kept = j;
+                running += x;
+                if (running > target) pick = j;
+            }
+        }
+        if (pick < 0) pick = last_kept;                         // rounding at the end: the last kept token
+        if (tid == 0) out[r] = sorted_id[pick];                 // n >= 1: the largest candidate has weight 1
+        return;
+    }
+    // top-p: the largest weight threshold whose kept mass reaches p * total, as on the whole row
+    float w_threshold = 0.f;
+    if (p < 1.0f) {
+        float all[1] = {weight};
+        block_sums(all, scratch_f);
+        const float need = p * all[0];
+        unsigned low = 0u;
+        for (int shift = 28; shift >= 0; shift -= 4) {
+            float mass[CANDIDATES];
+#pragma unroll
+            for (int j = 0; j < CANDIDATES; ++j) mass[j] = __float_as_uint(weight) >= (low | ((unsigned)(j + 1) << shift)) ? weight : 0.f;
+            block_sums(mass, scratch_f);
+            unsigned digit = 0u;
+#pragma unroll
+            for (int j = 0; j < CANDIDATES; ++j) if (mass[j] >= need) digit = (unsigned)(j + 1);
+            low |= digit << shift;
+        }
+        w_threshold = __uint_as_float(min(low, __float_as_uint(1.0f)));
+    }
+    if (tid == 0) {
+        float sum = 0.f;
+        for (int j = 0; j < n; ++j) sum += sorted_weight[j] >= w_threshold ? sorted_weight[j] : 0.f;
+        const float target = uniforms[r] * sum;
+        float running = 0.f;
+        int pick = -1, last_kept = -1;
+        for (int j = 0; j < n && pick < 0; ++j) {
+            const float x = sorted_weight[j];
+            if (x >= w_threshold && x > 0.f) {
+                last_kept = sorted_id[j];
+                running += x;
+                if (running > target) pick = last_kept;
+            }
+        }
+        if (pick < 0) pick = last_kept;                         // rounding at the end: the last kept token
+        out[r] = pick;                                          // n >= 1: the largest candidate has weight 1
+    }
+}
+
 }  // namespace
+
+// Bytes of workspace with which small top-ks take the way through slices (0: the vocabulary is too small to gain).
+extern "C" long xrt_sample_workspace(int rows, int vocab) {
+    if (rows <= 0 || (vocab + SLICE - 1) / SLICE < LEAST_SLICES || vocab > MAX_VOCAB) return 0;
+    return (long)rows * ((vocab + SLICE - 1) / SLICE) * (long)sizeof(SliceCandidates);
+}
 
 extern "C" int xrt_sample(const float* logits, int rows, int vocab, int* out, const float* temperature,
                           const int* top_k, const float* top_p, const float* penalty, const int* history,
-                          const int* history_offsets, const float* uniforms, void* stream) {
+                          const int* history_offsets, const float* uniforms, void* workspace, long workspace_bytes,
+                          void* stream) {
     XRT_REQUIRE(rows >= 0, "sample: negative row count");
     XRT_REQUIRE(vocab > 0, "sample: cannot sample from an empty logits vector");          // sampler.rs:56-60
     XRT_REQUIRE(vocab <= MAX_VOCAB, "sample: vocabulary %d exceeds %d", vocab, MAX_VOCAB);
@@ -405,6 +744,18 @@ extern "C" int xrt_sample(const float* logits, int rows, int vocab, int* out, co
                 "sample: null operand");
     if (rows == 0) return 0;
     const size_t lds = (size_t)((vocab + 31) / 32) * sizeof(unsigned);
+    const long need = xrt_sample_workspace(rows, vocab);
+    if (workspace != nullptr && need > 0 && workspace_bytes >= need) {
+        const int slices = (vocab + SLICE - 1) / SLICE;
+        sample_slices_kernel<<<dim3(slices, rows), SLICE_THREADS, 0, (hipStream_t)stream>>>(
+            logits, vocab, temperature, top_k, penalty, history, history_offsets, (SliceCandidates*)workspace, slices);
+        XRT_LAUNCH_CHECK("sample (slices)");
+        sample_candidates_kernel<<<rows, THREADS, lds, (hipStream_t)stream>>>(
+            logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms,
+            (const SliceCandidates*)workspace, slices);
+        XRT_LAUNCH_CHECK("sample (candidates)");
+        return 0;
+    }
     sample_kernel<<<rows, THREADS, lds, (hipStream_t)stream>>>(logits, vocab, out, temperature, top_k, top_p,
                                                               penalty, history, history_offsets, uniforms);
     XRT_LAUNCH_CHECK("sample");

@@ -77,10 +77,14 @@ int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_
                   const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs,
                   int max_count, int max_context, float* workspace, long workspace_floats, void* stream);
 
-// one token per row of float32 logits
+// one token per row of float32 logits. With a workspace of xrt_sample_workspace(rows, vocab) bytes (0: this
+// vocabulary gains nothing from it) rows with a top-k of 1 to 64 are sampled from candidates that
+// workgroups find slice by slice, instead of in eight passes over the row; without, all rows take the passes.
 int xrt_sample(const float* logits, int rows, int vocab, int* out, const float* temperature,
                const int* top_k, const float* top_p, const float* penalty, const int* history,
-               const int* history_offsets, const float* uniforms, void* stream);
+               const int* history_offsets, const float* uniforms, void* workspace, long workspace_bytes,
+               void* stream);
+long xrt_sample_workspace(int rows, int vocab);
 
 #ifdef __cplusplus
 }

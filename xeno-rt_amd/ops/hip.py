@@ -85,6 +85,7 @@ class HipOps:
                      "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_normed", "xrt_linear_qkv"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
+        self.lib.xrt_sample_workspace.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
     def _check(self, status: int) -> None:
@@ -289,7 +290,9 @@ class HipOps:
             ctypes.c_float(scale), int(window or 0), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
 
-    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms):
+    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms,
+               small_top_k=False):
+        """small_top_k: some row has a top-k of 1 to 64 and a temperature: worth the kernels that look for candidates."""
         if logits.dim() != 2:
             raise KernelError("sample: logits must be [rows, vocab]")
         rows, vocab = logits.shape
@@ -301,6 +304,8 @@ class HipOps:
                 ("history_offsets", history_offsets, torch.int32, (rows + 1,)),
                 ("uniforms", uniforms, torch.float32, (rows,)), ("history", history, torch.int32, None)):
             self._require(tensor, f"sample {what}", dtype, shape, logits)
+        need = int(self.lib.xrt_sample_workspace(rows, vocab)) if small_top_k else 0
+        workspace = torch.empty(need, dtype=torch.uint8, device=logits.device) if need > 0 else None
         self._check(self.lib.xrt_sample(_ptr(logits), rows, vocab, _ptr(out), _ptr(temperature), _ptr(top_k),
                                         _ptr(top_p), _ptr(penalty), _ptr(history), _ptr(history_offsets),
-                                        _ptr(uniforms), self._stream(logits)))
+                                        _ptr(uniforms), _ptr(workspace), ctypes.c_long(need), self._stream(logits)))
