@@ -4,9 +4,11 @@
 // Such a product is bound by reading w once from HBM, so the kernel is built around that
 // stream. A workgroup of 8 wavefronts owns 16 (or 32) rows of w. Each wavefront takes one
 // eighth of K and streams its part of those rows straight from global memory into the A
-// operand of v_mfma_f32_16x16x32_bf16: a 128-wide K step is four load instructions, and in each
-// the four lanes (r, 0..3) of a row read 64 contiguous bytes of it, so that one instruction
-// asks for 16 half cache lines and a row is read in 256-byte runs. The B operand holds the
+// operand of v_mfma_f32_16x16x32_bf16: a 64-wide K step is two load instructions, and in each
+// the four lanes (r, 0..3) of a row read 64 contiguous bytes of it, so that a step takes one
+// whole cache line of each of 16 rows. (Steps of 128 cost 20 registers more and with them
+// wavefronts in flight: 2 us more on the largest product; steps of 32, half a line at a time,
+// are a quarter slower.) The B operand holds the
 // activations x (16 rows of m per tile), read with the same K permutation. Loads carry no
 // branches (addresses are clamped into the operands instead), run one step ahead of the
 // matrix cores, and the products of a step go to accumulators that do not wait on each other:
@@ -36,7 +38,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int WAVES = 8;
-constexpr int KSTEP = 128;       // K covered by one step of a wavefront: 4 lane groups x 32
+constexpr int KSTEP = 64;         // K covered by one step of a wavefront
+constexpr int JL = KSTEP / 32;   // load instructions per operand tile and step: 4 lane groups x 8 elements each
 enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
 
 __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
@@ -91,7 +94,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     const int k_end = min(K, k_begin + steps_per_wave * KSTEP);
 
     // CHAINS accumulators per output tile, used in turn and added at the end
-    constexpr int CHAINS = MT == 1 ? (AROUND && WT == 2 ? 3 : 4) : (MT == 2 ? 2 : 1);
+    constexpr int CHAINS = MT == 1 ? 2 : (MT == 2 ? 2 : 1);
     floatx4 chain[CHAINS][WT][MT];
 #pragma unroll
     for (int h = 0; h < CHAINS; ++h)
@@ -114,21 +117,21 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 #pragma unroll
     for (int m = 0; m < MT; ++m) x_ptr[m] = x + (long)min(m * 16 + r, M - 1) * K + c * 8;
 
-    auto load_w = [&](bf16x8 (&regs)[WT][4], int kb) {
+    auto load_w = [&](bf16x8 (&regs)[WT][JL], int kb) {
 #pragma unroll
         for (int t = 0; t < WT; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) regs[t][j] = *reinterpret_cast<const bf16x8*>(w_ptr[t] + kb + j * 32);
+            for (int j = 0; j < JL; ++j) regs[t][j] = *reinterpret_cast<const bf16x8*>(w_ptr[t] + kb + j * 32);
     };
-    auto load_x = [&](bf16x8 (&regs)[MT][4], int kb) {
+    auto load_x = [&](bf16x8 (&regs)[MT][JL], int kb) {
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) regs[m][j] = *reinterpret_cast<const bf16x8*>(x_ptr[m] + kb + j * 32);
+            for (int j = 0; j < JL; ++j) regs[m][j] = *reinterpret_cast<const bf16x8*>(x_ptr[m] + kb + j * 32);
     };
-    auto multiply = [&](const bf16x8 (&wregs)[WT][4], const bf16x8 (&xregs)[MT][4]) {
+    auto multiply = [&](const bf16x8 (&wregs)[WT][JL], const bf16x8 (&xregs)[MT][JL]) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < JL; ++j)
 #pragma unroll
             for (int t = 0; t < WT; ++t)
 #pragma unroll
@@ -136,7 +139,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                     chain[j % CHAINS][t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wregs[t][j], xregs[m][j], chain[j % CHAINS][t][m], 0, 0, 0);
     };
 
-    // Whole steps of 128 along k run through a pipeline of two register sets: while the matrix
+    // Whole steps along k run through a pipeline of two register sets: while the matrix
     // cores consume one step, the loads of the next are in flight. The steady-state loop body has
     // no branch; the last one or two steps are peeled off.
     // The sums of squares of this wavefront's eighth of the tiles (lane (r, c): row r, every fourth
@@ -220,8 +223,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 
     const int full = max(0, (min(k_end, K / KSTEP * KSTEP) - k_begin) / KSTEP);     // whole steps of this wavefront
     if (full > 0) {
-        bf16x8 w_a[WT][4], w_b[WT][4];
-        bf16x8 x_a[MT][4], x_b[MT][4];
+        bf16x8 w_a[WT][JL], w_b[WT][JL];
+        bf16x8 x_a[MT][JL], x_b[MT][JL];
         load_x(x_a, k_begin);
         load_w(w_a, k_begin);
         ask_early();
@@ -245,11 +248,11 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     } else {
         ask_early();
     }
-    // what is left of K when it is no multiple of 128: one guarded step, in the wavefront that owns it
+    // what is left of K when it is no multiple of the step: one guarded step, in the wavefront that owns it
     const int tail_begin = k_begin + full * KSTEP;
     if (tail_begin < k_end) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < JL; ++j) {
             const bool inside = tail_begin + j * 32 + c * 8 + 8 <= K;       // K is a multiple of 8
             bf16x8 b[MT];
 #pragma unroll
