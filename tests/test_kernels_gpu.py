@@ -594,20 +594,23 @@ def test_sample_small_top_k_through_slices(ops, vocab):
     """Rows of every kind in one call (greedy, no top-k, top-k of 1, 40 and 64, a penalty, ties that overflow a
     slice's list, ties across slices): the way through slices picks what the passes over the row pick."""
     g = torch.Generator().manual_seed(vocab)
-    rows = 9
+    rows = 12
     logits = torch.randn(rows, vocab, generator=g) * 3.0
+    logits[9, torch.randperm(vocab, generator=g)[:12]] += 25.0     # a dozen tokens hold nearly all the mass, as a model's do
+    logits[10, torch.randperm(vocab, generator=g)[:70]] += 25.0    # seventy: more than the candidates of a top-p alone
+    logits[11, 1000:1100] = 30.0                                   # a hundred that tie at the top
     logits[5, 5000:5300] = 40.0                                    # 300 tokens tie at the top of one slice
     logits[6, ::4096] = 35.0                                       # one token at the top of every slice: they tie across slices
     logits[7] = logits[7].abs() * -1.0                             # all negative
     logits[8, vocab - 3:] = 50.0                                   # the last, partly filled slice holds the largest
     logits = logits.to(DEV)
-    temperature = torch.tensor([0.0, 1.0, 0.8, 0.8, 1.3, 1.0, 1.0, 0.7, 1.0], device=DEV)
-    top_k = i32([40, 0, 1, 40, 64, 20, 5, 40, 2])
-    top_p = torch.tensor([1.0, 0.9, 1.0, 0.95, 0.5, 1.0, 1.0, 0.9, 1.0], device=DEV)
-    penalty = torch.tensor([1.0, 1.0, 1.0, 1.1, 2.0, 1.0, 1.0, 1.5, 1.0], device=DEV)
+    temperature = torch.tensor([0.0, 1.0, 0.8, 0.8, 1.3, 1.0, 1.0, 0.7, 1.0, 1.0, 0.9, 1.0], device=DEV)
+    top_k = i32([40, 0, 1, 40, 64, 20, 5, 40, 2, 0, 0, 0])         # rows 1 and 9 to 11: a top-p alone
+    top_p = torch.tensor([1.0, 0.9, 1.0, 0.95, 0.5, 1.0, 1.0, 0.9, 1.0, 0.9, 0.95, 0.8], device=DEV)
+    penalty = torch.tensor([1.0, 1.0, 1.0, 1.1, 2.0, 1.0, 1.0, 1.5, 1.0, 1.0, 1.0, 1.0], device=DEV)
     history = i32(list(range(0, vocab, 997)))
-    offsets = i32([0, 0, 0, 0] + [len(history)] * 6)               # the history is row 3's alone
-    for draw in (0.03, 0.37, 0.71, 0.999):
+    offsets = i32([0, 0, 0, 0] + [len(history)] * 9)               # the history is row 3's alone
+    for draw in (0.03, 0.37, 0.71, 0.93, 0.999):
         uniforms = torch.full((rows,), draw, device=DEV)
         whole, sliced = torch.empty(rows, dtype=torch.int32, device=DEV), torch.full((rows,), -1, dtype=torch.int32, device=DEV)
         ops.sample(logits, whole, temperature, top_k, top_p, penalty, history, offsets, uniforms)
@@ -616,6 +619,7 @@ def test_sample_small_top_k_through_slices(ops, vocab):
     picks = whole.tolist()
     assert picks[2] == int(logits[2].argmax())                     # top-k 1
     assert 5000 <= picks[5] < 5300 and picks[6] % 4096 == 0 and picks[8] >= vocab - 3
+    assert float(logits[9, picks[9]]) > 15.0 and float(logits[10, picks[10]]) > 15.0 and 1000 <= picks[11] < 1100
 
 
 def test_sample_rows_are_independent(ops):

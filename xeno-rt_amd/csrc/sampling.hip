@@ -424,14 +424,21 @@ constexpr int LEAST_SLICES = 8;        // with fewer slices their tops are too f
 
 struct SliceCandidates {
     int count;                         // -1: this row does not go this way; more than SLICE_HOLDS: they did not fit
-    int unused[3];
+    float largest, mass;               // for a row without top-k: the slice's largest value, and the sum of exp((value - largest) / temperature)
+    int unused;
     unsigned top[SLICE_TOPS];          // keys of SLICE_TOPS different tokens of the slice, the largest first (0: none)
     int id[SLICE_HOLDS];
     float value[SLICE_HOLDS];          // after the penalty
 };
 
-__device__ __forceinline__ bool goes_by_slices(float temperature, int k, int vocab) {
-    return temperature > 1e-5f && k > 0 && k <= FAST_TOP_K && k < vocab;
+// The top-k that a row takes through the slices; 0: it does not go this way. A row with a top-p but
+// no top-k goes as if it had the largest top-k: when those candidates hold top-p's share of the whole
+// row's mass (usual with a model's logits), top-p's threshold lies among them and the answer is exact;
+// when they do not, the row's workgroup turns to the passes over the row.
+__device__ __forceinline__ int top_k_by_slices(float temperature, int k, float p, int vocab) {
+    if (!(temperature > 1e-5f) || vocab <= FAST_TOP_K) return 0;
+    if (k > 0) return k <= FAST_TOP_K ? k : 0;
+    return p < 1.0f ? FAST_TOP_K : 0;
 }
 
 // How many of the block's threads hold a larger maximum than this one (ties: lower thread first): the
@@ -456,16 +463,17 @@ __device__ __forceinline__ int place_of_maximum(unsigned mine, unsigned* maxima)
 
 __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
     const float* __restrict__ logits, int vocab, const float* __restrict__ temperature, const int* __restrict__ top_k,
-    const float* __restrict__ penalty, const int* __restrict__ history, const int* __restrict__ history_offsets,
-    SliceCandidates* __restrict__ candidates, int slices) {
+    const float* __restrict__ top_p, const float* __restrict__ penalty, const int* __restrict__ history,
+    const int* __restrict__ history_offsets, SliceCandidates* __restrict__ candidates, int slices) {
     __shared__ unsigned seen[SLICE / 32];
     __shared__ __attribute__((aligned(16))) unsigned maxima[SLICE_THREADS];
     __shared__ unsigned bound;
+    __shared__ float slice_largest, wave_mass[SLICE_WAVES];
     __shared__ int held;
     const int r = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
     SliceCandidates& mine = candidates[(long)r * slices + slice];
-    const int k = top_k[r];
-    if (!goes_by_slices(temperature[r], k, vocab)) {
+    const int k = top_k_by_slices(temperature[r], top_k[r], top_p[r], vocab);
+    if (k == 0) {
         if (tid == 0) mine.count = -1;
         return;
     }
@@ -499,13 +507,34 @@ __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
         key[e] = first + local < vocab ? order_key(value[e]) : 0u;
     }
     unsigned largest = 0u;
+    float largest_value = -INFINITY;
 #pragma unroll
-    for (int e = 0; e < SLICE_EACH; ++e) largest = max(largest, key[e]);
+    for (int e = 0; e < SLICE_EACH; ++e) {
+        if (key[e] > largest) { largest = key[e]; largest_value = value[e]; }
+    }
     const int place = place_of_maximum<SLICE_THREADS>(largest, maxima);
     if (place == k - 1) bound = largest;                // 0 if fewer than k threads hold a token
     if (place < SLICE_TOPS) mine.top[place] = largest;
+    if (place == 0) slice_largest = largest_value;
     __syncthreads();
     const unsigned threshold = bound;
+    if (top_k[r] == 0) {
+        // the slice's share of the row's mass, relative to its own largest value: threads add their tokens in
+        // order, lanes in a tree, wavefronts in order
+        const float inv_temp = 1.0f / temperature[r], top = slice_largest;
+        float sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < SLICE_EACH; ++e) sum += key[e] != 0u ? expf((value[e] - top) * inv_temp) : 0.f;
+        sum = wave_sum(sum);
+        if (tid % XRT_WAVE == 0) wave_mass[tid / XRT_WAVE] = sum;
+        __syncthreads();
+        if (tid == 0) {
+            float total = 0.f;
+            for (int w = 0; w < SLICE_WAVES; ++w) total += wave_mass[w];
+            mine.mass = total;
+            mine.largest = top;
+        }
+    }
 #pragma unroll
     for (int e = 0; e < SLICE_EACH; ++e) {
         if (key[e] != 0u && key[e] >= threshold) {
@@ -534,12 +563,14 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
     __shared__ int sorted_id[ROW_HOLDS];
     __shared__ float sorted_weight[ROW_HOLDS];
     __shared__ int kept, survivors;
+    __shared__ float row_mass;
     static_assert(MOST_SLICES <= XRT_WAVE, "one lane per slice");
     const int r = blockIdx.x, tid = threadIdx.x;
     const SliceCandidates* mine = candidates + (long)r * slices;
     // where every slice's candidates start in the row's list (one lane per slice; an inclusive sum over the
     // lanes); a slice that says "not this way" or "they did not fit" sends the row to the whole-row path
-    const int k = top_k[r];
+    const bool no_top_k = top_k[r] == 0;                        // a top-p alone: see top_k_by_slices
+    const int k = no_top_k ? FAST_TOP_K : top_k[r];
     if (tid < XRT_WAVE) {
         const int count = tid < slices ? mine[tid].count : 0;
         const bool bad = count < 0 || count > SLICE_HOLDS;
@@ -651,6 +682,24 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
     }
     __syncthreads();
     const float p = top_p[r];
+    if (no_top_k) {
+        // The whole row's mass, from the slices (in their order), relative to the row's largest value. If the
+        // candidates that stayed hold less than top-p's share of it, the threshold lies below them: the passes
+        // over the row find it.
+        if (tid < XRT_WAVE) {
+            const float share = tid < slices ? mine[tid].mass * expf((mine[tid].largest - best) * inv_temp) : 0.f;
+            float total = 0.f;
+            for (int j = 0; j < slices; ++j) total += __shfl(share, j, XRT_WAVE);
+            if (tid == 0) row_mass = total;
+        }
+        float stayed[1] = {weight};
+        block_sums(stayed, scratch_f);                          // has a barrier before row_mass is read
+        if (!(stayed[0] >= p * row_mass)) {
+            __syncthreads();
+            sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms);
+            return;
+        }
+    }
     if (n <= XRT_WAVE) {
         // the usual case: one wavefront holds them all, lane j the j-th in the order of ids
         if (tid >= XRT_WAVE) return;
@@ -664,7 +713,8 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
                 all += other;
                 with_larger += other >= w ? other : 0.f;
             }
-            float reaches = tid < n && with_larger >= p * all ? w : 0.f;
+            const float need = p * (no_top_k ? row_mass : all);
+            float reaches = tid < n && with_larger >= need ? w : 0.f;
 #pragma unroll
             for (int offset = XRT_WAVE / 2; offset > 0; offset >>= 1) reaches = fmaxf(reaches, __shfl_xor(reaches, offset, XRT_WAVE));
             w_threshold = fminf(reaches, 1.0f);
@@ -692,7 +742,7 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
     if (p < 1.0f) {
         float all[1] = {weight};
         block_sums(all, scratch_f);
-        const float need = p * all[0];
+        const float need = p * (no_top_k ? row_mass : all[0]);
         unsigned low = 0u;
         for (int shift = 28; shift >= 0; shift -= 4) {
             float mass[CANDIDATES];
@@ -748,7 +798,7 @@ extern "C" int xrt_sample(const float* logits, int rows, int vocab, int* out, co
     if (workspace != nullptr && need > 0 && workspace_bytes >= need) {
         const int slices = (vocab + SLICE - 1) / SLICE;
         sample_slices_kernel<<<dim3(slices, rows), SLICE_THREADS, 0, (hipStream_t)stream>>>(
-            logits, vocab, temperature, top_k, penalty, history, history_offsets, (SliceCandidates*)workspace, slices);
+            logits, vocab, temperature, top_k, top_p, penalty, history, history_offsets, (SliceCandidates*)workspace, slices);
         XRT_LAUNCH_CHECK("sample (slices)");
         sample_candidates_kernel<<<rows, THREADS, lds, (hipStream_t)stream>>>(
             logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms,

@@ -292,7 +292,8 @@ class HipOps:
 
     def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms,
                small_top_k=False):
-        """small_top_k: some row has a top-k of 1 to 64 and a temperature: worth the kernels that look for candidates."""
+        """small_top_k: some row has a temperature and a top-k of 1 to 64, or a top-p without top-k: worth the
+        kernels that look for candidates slice by slice."""
         if logits.dim() != 2:
             raise KernelError("sample: logits must be [rows, vocab]")
         rows, vocab = logits.shape

@@ -93,7 +93,8 @@ class Sampler:
             ints = staging_for(self.device).upload([c.top_k for c in configs] + offsets + history)
             self._last = (made_from, (floats, ints))
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
-        small_top_k = any(not c.is_greedy() and 0 < c.top_k <= 64 for c in configs)      # a faster way for these rows
+        # rows that the kernels can sample from a few candidates instead of passes over the whole row
+        small_top_k = any(not c.is_greedy() and (0 < c.top_k <= 64 or (c.top_k == 0 and c.top_p < 1.0)) for c in configs)
         self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2],
                         ints[2 * rows + 1:], ints[rows:2 * rows + 1], floats[3], small_top_k=small_top_k)
         return out.tolist()
