@@ -45,8 +45,9 @@ enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
 __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 
 // MT: tiles of 16 rows of x; RT: tiles of 16 rows of w per wavefront; GATED doubles the w tiles.
-// With one tile of x (the common decode case) the kernel is held to 128 registers, so that at
-// least two workgroups fit a compute unit: the stream from HBM needs the wavefronts in flight.
+// With one tile of x (the common decode case) the kernel is held to 128 registers at most (it takes
+// 62 to 92), so that two to four workgroups fit a compute unit: the stream from HBM needs the
+// wavefronts in flight.
 // EXTRA 1: the kernel also does its share of an RMSNorm before or after the product (one tile of x,
 // one tile of w per wavefront); 2: and what follows a q/k/v projection. Kernels without keep their
 // registers for the stream.
@@ -94,7 +95,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     const int k_end = min(K, k_begin + steps_per_wave * KSTEP);
 
     // CHAINS accumulators per output tile, used in turn and added at the end
-    constexpr int CHAINS = MT == 1 ? 2 : (MT == 2 ? 2 : 1);
+    constexpr int CHAINS = MT <= 2 ? 2 : 1;
     floatx4 chain[CHAINS][WT][MT];
 #pragma unroll
     for (int h = 0; h < CHAINS; ++h)
