@@ -465,6 +465,25 @@ def test_attention_decode_on_matrix_cores(ops, nh, nkv, hd):
     assert torch.equal(out2[:-1], out) and float(out2[-1].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (24, 8, 64)])
+def test_attention_decode_of_many_sequences(ops, nh, nkv, hd):
+    """Seventy sequences: with so many (sequence, key/value head) pairs a workgroup takes all keys of its pair
+    and writes the result itself, without partial results and a merge; padding still gets zeros."""
+    lengths = [1 + (37 * i) % 300 for i in range(69)] + [900]
+    kv, keys, values = filled_cache(nkv, hd, torch.bfloat16, lengths, seed=hd)
+    slots = list(range(len(lengths)))
+    positions = [n - 1 for n in lengths]
+    batch = described(slots + [-1], [1] * (len(lengths) + 1), positions + [0])
+    batch.slots, batch.positions = i32(slots + [-1]), i32(positions + [0])
+    qkv = rand(len(lengths) + 1, (nh + 2 * nkv) * hd, dtype=torch.bfloat16, seed=3)
+    out = torch.full((len(lengths) + 1, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=1.0 / math.sqrt(hd))
+    want = expected_attention(qkv[:-1], slots, positions, keys, values, nh, nkv, hd)
+    assert torch.isfinite(out).all()
+    assert rel(out[:-1].cpu(), want) < 1e-2
+    assert float(out[-1].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("nh,nkv,hd", [(4, 4, 64), (8, 2, 128), (32, 8, 128), (6, 3, 64)])
 def test_attention_prefill_on_matrix_cores(ops, nh, nkv, hd):
     """Whole prompts of unequal lengths in one step, and a prompt that continues a cache."""

@@ -37,7 +37,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
     float scale, int chunk_blocks, int n_parts, int q_tiles,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, bf16* __restrict__ out) {
     constexpr int KS = HD / 32;                    // K steps of the score product
     constexpr int DT = HD / 16;                    // 16-row tiles of the value product
     __shared__ floatx4 merge_o[WAVES][DT][XRT_WAVE];
@@ -50,13 +50,20 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
     const int kv_head = blockIdx.y / q_tiles, q_tile = blockIdx.y % q_tiles;
     const int token = blockIdx.z;
     const int slot = slots[token];
-    if (slot < 0) return;                          // padding: the whole workgroup leaves
+    const int group = n_heads / n_kv_heads;
+    if (slot < 0) {                                // padding: the whole workgroup leaves
+        // (with one partial result per head there is no merge kernel after this one to write the zeros)
+        if (n_parts == 1 && wave == 0 && q_tile * 16 + r < group) {
+            bf16* dst = out + ((long)token * n_heads + kv_head * group + q_tile * 16 + r) * HD;
+            for (int d = c; d < HD; d += 4) dst[d] = (bf16)0.f;
+        }
+        return;
+    }
     const int n_keys = positions[token] + 1;
     if (part * WAVES * chunk_blocks * XRT_BLOCK_TOKENS >= n_keys) return;      // nothing here for any wavefront
     const int first_block = chunk * chunk_blocks;
     const bool active = first_block * XRT_BLOCK_TOKENS < n_keys;
     const int last_block = min((n_keys - 1) / XRT_BLOCK_TOKENS, first_block + chunk_blocks - 1);
-    const int group = n_heads / n_kv_heads;
     const int head_in_group = q_tile * 16 + r;             // this lane's query head (column of the products)
     const bool head_valid = head_in_group < group;
     const int head = kv_head * group + min(head_in_group, group - 1);
@@ -180,6 +187,19 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) total[dt] += merge_o[w][dt][lane] * weight;
         }
+        if (n_parts == 1) {
+            // the workgroup has seen all keys of the sequence: this is the result, and no merge kernel follows
+            const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+            bf16* final_row = out + ((long)token * n_heads + head) * HD;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                struct alignas(8) Four { bf16 e[4]; } four;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) four.e[i] = (bf16)(total[dt][i] * inv);
+                *reinterpret_cast<Four*>(final_row + dt * 16 + c * 4) = four;
+            }
+            return;
+        }
         const long index = ((long)token * n_heads + head) * n_parts + part;
         float* dst = part_o + index * HD;
         // accumulator register i of tile dt is dimension dt*16 + c*4 + i, for query head r
@@ -263,7 +283,10 @@ struct Cut { int chunk_blocks, n_parts; };
 
 Cut cut_for(int tokens, int n_kv_heads, int q_tiles, int max_context) {
     const int max_blocks = (max_context + XRT_BLOCK_TOKENS - 1) / XRT_BLOCK_TOKENS;
-    // enough wavefronts to fill the chip, but chunks as long as that allows
+    // Two workgroups of four wavefronts fit a compute unit. With that many (token, key/value head) pairs a
+    // workgroup takes all keys of its pair: nothing is left to merge, and the merge kernel is not launched.
+    if ((long)tokens * n_kv_heads * q_tiles >= 512) return Cut{(max_blocks + WAVES - 1) / WAVES, 1};
+    // else: enough wavefronts to fill the chip, but chunks as long as that allows
     long chunk_blocks = ((long)tokens * n_kv_heads * q_tiles * max_blocks) / 4096;
     chunk_blocks = chunk_blocks < 1 ? 1 : (chunk_blocks > 16 ? 16 : chunk_blocks);
     const int n_chunks = (int)((max_blocks + chunk_blocks - 1) / chunk_blocks);
@@ -287,8 +310,9 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
     const dim3 grid(cut.n_parts, n_kv_heads * q_tiles, tokens);
     attention_decode_kernel<HD><<<grid, WAVES * XRT_WAVE, 0, s>>>(
         qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, positions, slots,
-        scale, cut.chunk_blocks, cut.n_parts, q_tiles, part_o, part_ml);
+        scale, cut.chunk_blocks, cut.n_parts, q_tiles, part_o, part_ml, out);
     XRT_LAUNCH_CHECK("attention (decode)");
+    if (cut.n_parts == 1) return 0;
     const int part_keys = cut.chunk_blocks * WAVES * XRT_BLOCK_TOKENS;
     attention_decode_merge_kernel<HD><<<dim3(n_heads, tokens), HD, cut.n_parts * sizeof(float), s>>>(
         part_o, part_ml, positions, slots, n_heads, part_keys, cut.n_parts, out);
