@@ -229,9 +229,9 @@ def test_decoding_across_a_thousand_tokens(dtype, tmp_path):
         assert_logits(rows[0][-1][i:i + 1], want, dtype, f"sequence {i}, last decoded token")
 
 
-@pytest.mark.parametrize("arch", ["qwen3", "llama"])
+@pytest.mark.parametrize("arch,head_dim", [("qwen3", 64), ("llama", 64), ("llama", 128)])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_a_batch_of_forty_sequences(dtype, arch, tmp_path):
+def test_a_batch_of_forty_sequences(dtype, arch, head_dim, tmp_path):
     """Forty sequences of unequal lengths start together and end one after the other: the step's
     token count runs through 300-odd (prompts), 40 and down to 1, and with a width of 128 the
     bfloat16 products take every kernel there is on the way: the tiled one and the one split along
@@ -239,7 +239,7 @@ def test_a_batch_of_forty_sequences(dtype, arch, tmp_path):
     also does the norms' work and, without head norms (llama), the rotation and the cache write)."""
     from xeno_rt_amd.engine import Engine
     raw = dict(TINY[arch], hidden_size=128, intermediate_size=320, num_attention_heads=4, num_key_value_heads=2,
-               head_dim=64, num_hidden_layers=2, max_position_embeddings=128)
+               head_dim=head_dim, num_hidden_layers=2, max_position_embeddings=128)
     folder = make_folder(raw, tmp_path / "wide", seed=13, std=0.15)
     plain = P.PlainModel(folder)
     vocab = plain.config.vocab_size
