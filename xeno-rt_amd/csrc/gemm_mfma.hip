@@ -34,10 +34,15 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 
 // One tile of the product, by one workgroup: `id` is the workgroup's number among those that work
 // on the output columns from n_first on, tiles_m x tiles_n of them.
+// The rows of a that come without their RMSNorm's division (see xrt_linear_norm in xrt_hip.h): the sums of
+// squares per tile of 16 columns, from which a tile of up to 64 rows works out 1 / rms of its rows and
+// multiplies its sums by it before the epilogue. squares null: nothing of the kind.
+struct RowScale { const float* squares; int tiles; int width; float eps; };
+
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __device__ __forceinline__ void gemm_tile(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int id, int tiles_m, int tiles_n, int n_first, int k_per_split) {
+    int id, int tiles_m, int tiles_n, int n_first, int k_per_split, const RowScale scale = RowScale{}) {
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr int WAVE_M = BM / WM, WAVE_N = BN / WN;        // part of the tile owned by one wavefront
     constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;        // 32x32 accumulator tiles of a wavefront
@@ -85,6 +90,25 @@ __device__ __forceinline__ void gemm_tile(
             return min(n0 + r, (long)N - 1);
         }
     };
+    // 1 / rms of the tile's rows, if the rows of a come without it. The sums of squares are asked for now,
+    // all at once (a thread takes four neighbouring rows of every sixteenth tile, 16 bytes a load), and added
+    // up after the main loop, when they have long arrived.
+    constexpr int SQUARE_LOADS = 16;                           // tiles of 16 columns per thread: rows of up to 16 * 16 * 16 columns
+    __shared__ float row_scale[BM <= 64 ? 64 : 1];
+    __shared__ float row_parts[BM <= 64 ? 16 : 1][64];
+    float4 early_squares[BM <= 64 ? SQUARE_LOADS : 1];
+    const bool scaled = BM <= 64 && scale.squares != nullptr;
+    if constexpr (BM <= 64) {
+        if (scaled && tid < 256) {
+#pragma unroll
+            for (int u = 0; u < SQUARE_LOADS; ++u) {
+                const int t = tid / 16 + 16 * u;
+                early_squares[u] = t < scale.tiles
+                    ? *reinterpret_cast<const float4*>(scale.squares + (long)t * XRT_SQUARES_STRIDE + (tid % 16) * 4)
+                    : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    }
     floatx16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -303,6 +327,39 @@ __device__ __forceinline__ void gemm_tile(
     }
 
     // ---- epilogue: accumulator element e of tile (i, j) is row (e/4)*8 + (lane/32)*4 + e%4, column lane%32
+    if constexpr (BM <= 64) {
+        if (scaled) {                                          // the same for all threads of the workgroup
+            if (tid < 256) {
+                float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int u = 0; u < SQUARE_LOADS; ++u) {
+                    sum.x += early_squares[u].x; sum.y += early_squares[u].y; sum.z += early_squares[u].z; sum.w += early_squares[u].w;
+                }
+                // rows of more than 4096 columns: the tiles beyond, one after the other
+                for (int t = tid / 16 + 16 * SQUARE_LOADS; t < scale.tiles; t += 16) {
+                    const float4 more = *reinterpret_cast<const float4*>(scale.squares + (long)t * XRT_SQUARES_STRIDE + (tid % 16) * 4);
+                    sum.x += more.x; sum.y += more.y; sum.z += more.z; sum.w += more.w;
+                }
+                *reinterpret_cast<float4*>(&row_parts[tid / 16][(tid % 16) * 4]) = sum;
+            }
+            __syncthreads();
+            if (tid < 64) {
+                float total = 0.f;
+#pragma unroll
+                for (int part = 0; part < 16; ++part) total += row_parts[part][tid];
+                row_scale[tid] = 1.0f / sqrtf(total / (float)scale.width + scale.eps);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float by = row_scale[wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j][e] *= by;
+                }
+        }
+    }
     if constexpr (MODE == MODE_GATED) {
         static_assert(TN % 2 == 0, "a wavefront holds as many gate blocks as up blocks");
 #pragma unroll
@@ -350,8 +407,8 @@ __device__ __forceinline__ void gemm_tile(
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int tiles_m, int tiles_n, int n_first, int k_per_split) {
-    gemm_tile<BM, BN, WM, WN, MODE, DK, STAGES, TO>(a, w, out, M, N, K, blockIdx.x, tiles_m, tiles_n, n_first, k_per_split);
+    int tiles_m, int tiles_n, int n_first, int k_per_split, const RowScale scale) {
+    gemm_tile<BM, BN, WM, WN, MODE, DK, STAGES, TO>(a, w, out, M, N, K, blockIdx.x, tiles_m, tiles_n, n_first, k_per_split, scale);
 }
 
 // Two tile shapes in one launch: the first `large_blocks` workgroups take 256 x 256 tiles of the
@@ -373,7 +430,7 @@ __global__ void __launch_bounds__(8 * XRT_WAVE) gemm_mfma_mixed_kernel(
 // Launches the tiles of output columns [n_first, n_first + n_count).
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, hipStream_t s,
-                  int splits = 1, int k_per_split = 0) {
+                  int splits = 1, int k_per_split = 0, const RowScale scale = RowScale{}) {
     constexpr int BN_OUT = MODE == MODE_GATED ? BN / 2 : BN;
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr size_t staging = DK != 0 ? (size_t)STAGES * (BM + BN) * DK * sizeof(bf16) : (size_t)2 * (BM + BN) * PITCH * sizeof(bf16);
@@ -390,8 +447,9 @@ int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, in
     const int total = tiles_m * tiles_n;
     const unsigned grid = (unsigned)(((total + 7) / 8) * 8);           // a whole number of rounds over the XCDs
     XRT_REQUIRE(splits == 1 || DK != 0, "linear (mfma): only whole tiles along k can be split");
+    XRT_REQUIRE(scale.squares == nullptr || (BM <= 64 && splits == 1), "linear (mfma): rows are scaled by tiles of up to 64 rows that see all of k");
     kernel<<<dim3(grid, splits), THREADS, lds, s>>>(a, w, out, M, N, K, tiles_m, tiles_n, n_first,
-                                                    splits == 1 ? K : k_per_split);
+                                                    splits == 1 ? K : k_per_split, scale);
     XRT_LAUNCH_CHECK("linear (mfma)");
     return 0;
 }
@@ -500,32 +558,82 @@ SplitPlan split_plan(int M, int N, int K, int mode) {
     return SplitPlan{splits, per * 64, rows_w};
 }
 
-template <int MODE, typename TO>
+// NORM 1: the rows of a came without their RMSNorm's division (norm.squares_in): the sums are multiplied by
+// 1 / rms of their row first. NORM 2 (accumulating): bfloat16(out * gain) and the sums of squares of out per
+// tile of 16 columns are written as well (N a multiple of 16: the 16 lanes of a tile then share a row).
+template <int MODE, typename TO, int NORM = 0>
 __global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restrict__ parts, int splits, int M, int N,
-                                                            TO* __restrict__ out) {
+                                                            TO* __restrict__ out, const xrt_linear_norm norm) {
+    __shared__ float wave_sums[256 / XRT_WAVE];
     const long rows_w = MODE == MODE_GATED ? 2L * N : N;
     const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (index >= (long)M * N) return;
-    const long m = index / N, n = index % N;
-    float sum = 0.f, up = 0.f;
-    for (int p = 0; p < splits; ++p) {
-        const float* part = parts + ((long)p * M + m) * rows_w;
-        sum += part[n];
-        if constexpr (MODE == MODE_GATED) up += part[N + n];
+    const bool inside = index < (long)M * N;
+    const long m = inside ? index / N : M - 1, n = inside ? index % N : 0;
+    // the row's sums of squares are asked for before the partial sums and used after them. A block lies
+    // within one row if N is a multiple of 256: then its threads share the work; else every thread adds
+    // up its row's sums itself, in the order of the tiles.
+    float mine = 0.f;
+    if constexpr (NORM == 1) {
+        if (N % 256 == 0)
+            for (int t = threadIdx.x; t < norm.tiles_in; t += 256) mine += norm.squares_in[(long)t * XRT_SQUARES_STRIDE + m];
+        else
+            for (int t = 0; t < norm.tiles_in; ++t) mine += norm.squares_in[(long)t * XRT_SQUARES_STRIDE + m];
     }
-    if constexpr (MODE == MODE_STORE) out[index] = from_float<TO>(sum);
-    else if constexpr (MODE == MODE_ACCUMULATE) out[index] = from_float<TO>(to_float(out[index]) + sum);
-    else out[index] = from_float<TO>(silu(sum) * up);
+    float sum = 0.f, up = 0.f;
+    if (inside) {
+        for (int p = 0; p < splits; ++p) {
+            const float* part = parts + ((long)p * M + m) * rows_w;
+            sum += part[n];
+            if constexpr (MODE == MODE_GATED) up += part[N + n];
+        }
+    }
+    float by = 1.0f;
+    if constexpr (NORM == 1) {
+        float total = mine;
+        if (N % 256 == 0) {
+            mine = wave_sum(mine);
+            if (threadIdx.x % XRT_WAVE == 0) wave_sums[threadIdx.x / XRT_WAVE] = mine;
+            __syncthreads();
+            total = 0.f;
+            for (int w = 0; w < 256 / XRT_WAVE; ++w) total += wave_sums[w];
+        }
+        by = 1.0f / sqrtf(total / (float)norm.width_in + norm.eps);
+    }
+    sum *= by;
+    up *= by;
+    float fresh = 0.f;
+    if (inside) {
+        if constexpr (MODE == MODE_STORE) out[index] = from_float<TO>(sum);
+        else if constexpr (MODE == MODE_ACCUMULATE) { fresh = to_float(out[index]) + sum; out[index] = from_float<TO>(fresh); }
+        else out[index] = from_float<TO>(silu(sum) * up);
+    }
+    if constexpr (NORM == 2) {
+        float squares = fresh * fresh;
+        squares += __shfl_xor(squares, 1, XRT_WAVE);
+        squares += __shfl_xor(squares, 2, XRT_WAVE);
+        squares += __shfl_xor(squares, 4, XRT_WAVE);
+        squares += __shfl_xor(squares, 8, XRT_WAVE);
+        if (inside) {
+            if (n % 16 == 0) norm.squares_out[(n / 16) * XRT_SQUARES_STRIDE + m] = squares;
+            const float gain = norm.gain_dtype == XRT_F32 ? ((const float*)norm.gain)[n] : to_float(((const bf16*)norm.gain)[n]);
+            ((bf16*)norm.scaled_out)[index] = from_float<bf16>(fresh * gain);
+        }
+    }
 }
 
 template <typename TO>
-int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, float* workspace, hipStream_t s) {
+int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, float* workspace,
+                 const xrt_linear_norm* norm, hipStream_t s) {
     const SplitPlan plan = split_plan(M, N, K, mode);
+    const bool scaled = norm && norm->squares_in, emits = norm && norm->squares_out;
+    XRT_REQUIRE(!norm || M <= SPLIT_BM, "linear (mfma): the norm around a product takes at most %d rows here", SPLIT_BM);
+    const RowScale scale = scaled ? RowScale{norm->squares_in, norm->tiles_in, norm->width_in, norm->eps} : RowScale{};
     if (M <= SPLIT_BM && plan.splits == 1) {                   // tiles enough: each applies the epilogue itself
-        if (mode == MODE_STORE) return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s);
-        if (mode == MODE_GATED) return launch_kernel<SPLIT_BM, SPLIT_BN, 2, 2, MODE_GATED, 64, 3, TO>(a, w, out, M, N, K, 0, N, s);
+        XRT_REQUIRE(!emits, "linear (mfma): only a product split along k writes what the norm after it needs");
+        if (mode == MODE_STORE) return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s, 1, 0, scale);
+        if (mode == MODE_GATED) return launch_kernel<SPLIT_BM, SPLIT_BN, 2, 2, MODE_GATED, 64, 3, TO>(a, w, out, M, N, K, 0, N, s, 1, 0, scale);
         if constexpr (sizeof(TO) == 4)
-            return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_ACCUMULATE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s);
+            return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_ACCUMULATE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s, 1, 0, scale);
         XRT_REQUIRE(false, "linear (mfma): accumulation needs a float32 output");
     }
     XRT_REQUIRE(workspace != nullptr, "linear (mfma): a product split along k needs its workspace");
@@ -537,9 +645,18 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
               a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split);
     if (status != 0) return status;
     const unsigned blocks = (unsigned)(((long)M * N + 255) / 256);
-    if (mode == MODE_STORE) split_reduce_kernel<MODE_STORE, TO><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out);
-    else if (mode == MODE_ACCUMULATE) split_reduce_kernel<MODE_ACCUMULATE, TO><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out);
-    else split_reduce_kernel<MODE_GATED, TO><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out);
+    const xrt_linear_norm none = {};
+    const xrt_linear_norm& around = norm ? *norm : none;
+    XRT_REQUIRE(!(scaled && emits), "linear (mfma): one product does one half of a norm");
+#define XRT_REDUCE(MODE_, NORM_) split_reduce_kernel<MODE_, TO, NORM_><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around)
+    if (mode == MODE_STORE) { if (scaled) XRT_REDUCE(MODE_STORE, 1); else XRT_REDUCE(MODE_STORE, 0); }
+    else if (mode == MODE_GATED) { if (scaled) XRT_REDUCE(MODE_GATED, 1); else XRT_REDUCE(MODE_GATED, 0); }
+    else if (scaled) XRT_REDUCE(MODE_ACCUMULATE, 1);
+    else if (emits) {
+        XRT_REQUIRE(N % 16 == 0, "linear (mfma): sums of squares per 16 columns need N = %d to be a multiple of 16", N);
+        XRT_REDUCE(MODE_ACCUMULATE, 2);
+    } else XRT_REDUCE(MODE_ACCUMULATE, 0);
+#undef XRT_REDUCE
     XRT_LAUNCH_CHECK("linear (split reduce)");
     return 0;
 }
@@ -569,8 +686,18 @@ bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, i
     return true;
 }
 
+// Whether a product of 17 to 64 rows can do its half of an RMSNorm: take rows that come without the
+// division (any mode), or, accumulating and split along k, write what the norm after it needs, provided
+// the product after the norm (same rows, N columns of a) will run through these tiles too.
+bool xrt_linear_split_takes_norm(const void* a, const void* w, int M, int N, int K, int mode) {
+    long unused = 0;
+    if (M <= 16 || M > SPLIT_BM || !xrt_linear_split_takes(a, w, M, N, K, mode, &unused)) return false;
+    if (mode != MODE_ACCUMULATE) return true;
+    return split_plan(M, N, K, mode).splits > 1 && N % 64 == 0 && N >= 128;
+}
+
 int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
-                     float* workspace, hipStream_t s) {
-    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, workspace, s);
-    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, workspace, s);
+                     float* workspace, const xrt_linear_norm* norm, hipStream_t s) {
+    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, workspace, norm, s);
+    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, workspace, norm, s);
 }

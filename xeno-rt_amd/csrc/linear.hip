@@ -10,8 +10,9 @@ int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int 
                     hipStream_t s);
 
 bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats);
+bool xrt_linear_split_takes_norm(const void* a, const void* w, int M, int N, int K, int mode);
 int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
-                     float* workspace, hipStream_t s);
+                     float* workspace, const xrt_linear_norm* norm, hipStream_t s);
 
 extern "C" long xrt_linear_workspace(const void* a, const void* w, int dtype, int M, int N, int K, int mode) {
     long need = 0;
@@ -34,7 +35,7 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
     if (dtype == XRT_BF16) {
         long need = 0;
         if (xrt_linear_split_takes(a, w, M, N, K, mode, &need) && (need == 0 || (workspace != nullptr && workspace_floats >= need)))
-            return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, workspace, (hipStream_t)stream);
+            return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, workspace, nullptr, (hipStream_t)stream);
     }
     if (dtype == XRT_BF16 && xrt_linear_skinny_accepts(a, w, M, K))
         return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, nullptr, nullptr, (hipStream_t)stream);
@@ -44,27 +45,37 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
 }
 
 extern "C" int xrt_linear_takes_norm(const void* a, const void* w, int dtype, int M, int N, int K, int mode) {
-    return dtype == XRT_BF16 && M >= 1 && N > 0 && K > 0 && mode >= 0 && mode <= 2 &&
-           xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_norm(M);
+    if (dtype != XRT_BF16 || M < 1 || N <= 0 || K <= 0 || mode < 0 || mode > 2) return 0;
+    if (xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_norm(M)) return 1;
+    return xrt_linear_split_takes_norm(a, w, M, N, K, mode) ? 1 : 0;
 }
 
 extern "C" int xrt_linear_normed(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N,
-                                 int K, int mode, const xrt_linear_norm* norm, void* stream) {
+                                 int K, int mode, const xrt_linear_norm* norm, float* workspace,
+                                 long workspace_floats, void* stream) {
     XRT_REQUIRE(a && w && out && norm, "linear with norm: null operand");
-    XRT_REQUIRE(xrt_linear_takes_norm(a, w, dtype, M, N, K, mode),
-                "linear with norm: M=%d N=%d K=%d of dtype %d is not a product that takes it", M, N, K, dtype);
+    XRT_REQUIRE(dtype == XRT_BF16 && M >= 1 && N > 0 && K > 0 && mode >= 0 && mode <= 2,
+                "linear with norm: M=%d N=%d K=%d mode %d of dtype %d is not a product that takes it", M, N, K, mode, dtype);
     XRT_REQUIRE(out_dtype == XRT_F32 || out_dtype == XRT_BF16, "linear with norm: unknown output dtype %d", out_dtype);
     XRT_REQUIRE(mode != 1 || out_dtype == XRT_F32, "linear with norm: accumulation needs a float32 output");
     if (norm->squares_in)
         XRT_REQUIRE(norm->width_in == K && norm->tiles_in == (K + 15) / 16,
                     "linear with norm: sums of squares of %d tiles over %d columns for a of %d columns",
                     norm->tiles_in, norm->width_in, K);
-    if (norm->squares_out || norm->scaled_out || norm->gain) {
+    const bool emits = norm->squares_out || norm->scaled_out || norm->gain;
+    if (emits) {
         XRT_REQUIRE(mode == 1, "linear with norm: only an accumulating product writes what the norm after it needs");
         XRT_REQUIRE(norm->squares_out && norm->scaled_out && norm->gain, "linear with norm: scaled_out, gain and squares_out come together");
         XRT_REQUIRE(norm->gain_dtype == XRT_F32 || norm->gain_dtype == XRT_BF16, "linear with norm: unknown gain dtype %d", norm->gain_dtype);
+        XRT_REQUIRE(xrt_linear_takes_norm(a, w, dtype, M, N, K, mode), "linear with norm: M=%d N=%d K=%d cannot write what the norm after it needs", M, N, K);
     }
-    return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, norm, nullptr, (hipStream_t)stream);
+    if (xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_norm(M))
+        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, norm, nullptr, (hipStream_t)stream);
+    long need = 0;
+    XRT_REQUIRE(M <= 64 && xrt_linear_split_takes(a, w, M, N, K, mode, &need),
+                "linear with norm: M=%d N=%d K=%d is not a product that takes it", M, N, K);
+    XRT_REQUIRE(need == 0 || (workspace != nullptr && workspace_floats >= need), "linear with norm: the workspace needs %ld floats", need);
+    return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, workspace, norm, (hipStream_t)stream);
 }
 
 extern "C" int xrt_linear_qkv(const void* a, const void* w, int dtype, void* qkv, int M, int K,
@@ -86,7 +97,7 @@ extern "C" int xrt_linear_qkv(const void* a, const void* w, int dtype, void* qkv
         (k_cache == nullptr || (block_table && slots && table_stride > 0 && n_blocks > 0)) &&
         (rope_theta == nullptr || rope_dim > 0))
         return xrt_linear_skinny(a, w, qkv, XRT_BF16, M, N, K, 0, norm, &after, (hipStream_t)stream);
-    const int status = norm ? xrt_linear_normed(a, w, dtype, qkv, dtype, M, N, K, 0, norm, stream)
+    const int status = norm ? xrt_linear_normed(a, w, dtype, qkv, dtype, M, N, K, 0, norm, workspace, workspace_floats, stream)
                             : xrt_linear(a, w, dtype, qkv, dtype, M, N, K, 0, workspace, workspace_floats, stream);
     if (status != 0) return status;
     return xrt_qkv_prepare(qkv, dtype, M, n_heads, n_kv_heads, head_dim, positions, slots, q_norm, k_norm, norm_dtype,

@@ -34,8 +34,9 @@ long xrt_linear_workspace(const void* a, const void* w, int dtype, int M, int N,
 // squares_out[t * XRT_SQUARES_STRIDE + m], the sum of x[m, n]^2 over the 16 columns n of tile t. The
 // second takes scaled_out as its a, squares_in (tiles_in = ceil(width_in / 16) tiles) and multiplies its
 // rows by 1 / sqrt(sum of squares / width_in + eps) before its epilogue. A half left all zero is not done.
-// xrt_linear_takes_norm says whether a product can do this (bfloat16 operands, few rows); if not,
-// xrt_linear_normed refuses it.
+// xrt_linear_takes_norm says whether an accumulating product can write these (bfloat16 operands, up to 64 rows,
+// and with more than 16 rows: split along k, N a multiple of 64); then the product after it (same rows) can
+// take them, and xrt_linear_normed refuses what cannot. workspace: as for xrt_linear.
 #define XRT_SQUARES_STRIDE 64
 typedef struct xrt_linear_norm {
     const float* squares_in; int tiles_in; int width_in; float eps;
@@ -43,7 +44,7 @@ typedef struct xrt_linear_norm {
 } xrt_linear_norm;
 int xrt_linear_takes_norm(const void* a, const void* w, int dtype, int M, int N, int K, int mode);
 int xrt_linear_normed(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
-                      int mode, const xrt_linear_norm* norm, void* stream);
+                      int mode, const xrt_linear_norm* norm, float* workspace, long workspace_floats, void* stream);
 
 // per-head RMSNorm of q and k (optional), rotation of q and k (optional), write of k and v
 // into the cache (optional); qkv rows are [q heads | k heads | v heads]. longest_run: the most

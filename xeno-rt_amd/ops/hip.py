@@ -169,8 +169,10 @@ class HipOps:
             if emit is not None:
                 norm.scaled_out, norm.squares_out = emit.values.data_ptr(), emit.squares.data_ptr()
                 norm.gain, norm.gain_dtype = then_norm[0].data_ptr(), _code(then_norm[0])
+            need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
+            workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
             self._check(self.lib.xrt_linear_normed(*sizes, _ptr(out), _code(out), m, n, k, mode, ctypes.byref(norm),
-                                                   self._stream(a)))
+                                                   _ptr(workspace), ctypes.c_long(need), self._stream(a)))
             return emit
         need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
