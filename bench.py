@@ -57,6 +57,8 @@ def sync():
 class Bench:
     def __init__(self, engine, seed):
         from xeno_rt_amd.sampling import Sampler, SamplerConfig
+        from xeno_rt_amd.staging import staging_for
+        self.staging = staging_for(engine.device)
         self.engine = engine
         self.sampler = Sampler(engine.ops, engine.device)
         self.greedy = SamplerConfig(temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
@@ -79,23 +81,31 @@ class Bench:
     def decode(self, batch, steps, warmup, context):
         """Tokens per second and ms per step of `steps` decode steps that end at `context` tokens."""
         engine = self.engine
+        warmup = max(warmup, 1)            # the step that makes the first logits is not timed
         start_length = context - steps - warmup
         slots = [engine.alloc_slot() for _ in range(batch)]
         try:
             self.fill(slots, start_length)
-            tokens = self.ids(batch)
             configs, histories, draws = [self.greedy] * batch, [[]] * batch, [0.0] * batch
+            staging = self.staging
+            entries = [(slot, row) for row, slot in enumerate(slots)]
+            logits = engine.step([(slot, [token], [0]) for slot, token in zip(slots, self.ids(batch))])
 
-            def one_step(tokens):
-                logits = engine.step([(slot, [token], [0]) for slot, token in zip(slots, tokens)])
-                return self.sampler.sample(logits, configs, histories, draws)
+            def one_step(logits):
+                """As the generation loop does it: the next step starts from the sampled tokens on the
+                device, and the host reads them while it runs."""
+                drawn = self.sampler.launch(logits, configs, histories, draws)
+                fetched = staging.fetch(drawn)
+                logits = engine.step_from(drawn, entries)
+                fetched.values()
+                return logits
 
-            for _ in range(warmup):
-                tokens = one_step(tokens)
+            for _ in range(warmup - 1):      # one warm-up step has been done above
+                logits = one_step(logits)
             sync()
             begin = time.perf_counter()
             for _ in range(steps):
-                tokens = one_step(tokens)
+                logits = one_step(logits)
             sync()
             elapsed = time.perf_counter() - begin
             mean_length = start_length + warmup + (steps - 1) / 2.0 + 1     # keys each timed step reads, on average

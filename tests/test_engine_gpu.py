@@ -252,3 +252,54 @@ def test_a_batch_of_forty_sequences(dtype, arch, head_dim, tmp_path):
         assert_logits(rows, plain.logits(ids), dtype, f"request {i} of 40")
     engine.cache.check()
     assert engine.cache.slots.n_held == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_generation_a_step_ahead_equals_generation_through_the_host(dtype, models, engines):
+    """The loop starts a step from the sampled tokens on the device before it has seen them. The same
+    requests, sampled with a temperature, through a loop written here that brings every token to the
+    host first, with the same uniform numbers: the same tokens, also where a request draws a stop token
+    (and has been stepped once for nothing) while the others go on."""
+    from xeno_rt_amd.engine import GenerateRequest, generate
+    from xeno_rt_amd.sampling import Sampler, uniform
+    engine = engines("llama", dtype)
+    vocab = engine.config.vocab_size
+    prompts = [token_ids(vocab, n, seed=300 + n) for n in (9, 3, 14)]
+    options = dict(temperature=0.9, top_k=12, top_p=0.9, repetition_penalty=1.0)
+
+    def through_the_host(stops):
+        sampler = Sampler(engine.ops, engine.device)
+        config = GenerateRequest([], **options).sampler_config()
+        slots = [engine.alloc_slot() for _ in prompts]
+        produced = [[] for _ in prompts]
+        live = list(range(len(prompts)))
+        logits = engine.step([(slots[i], prompts[i], [len(prompts[i]) - 1]) for i in live])
+        while live:
+            tokens = sampler.sample(logits, [config] * len(live), [[]] * len(live),
+                                    [uniform(70 + i, 0, len(produced[i])) for i in live])
+            still = []
+            for i, token in zip(live, tokens):
+                if token in stops:
+                    continue
+                produced[i].append(token)
+                if len(produced[i]) < 24:
+                    still.append(i)
+            live = still
+            if live:
+                logits = engine.step([(slots[i], [produced[i][-1]], [0]) for i in live])
+        for slot in slots:
+            engine.free_slot(slot)
+        return produced
+
+    free = through_the_host(())
+    # a stop token that the second request draws half-way, and that may end others too
+    stop = free[1][10]
+    want = through_the_host((stop,))
+    assert len(want[1]) <= 10 and max(len(tokens) for tokens in want) > len(want[1]) + 1
+    requests = [GenerateRequest(prompt, max_tokens=24, seed=70 + i, stop_ids=[stop], **options)
+                for i, prompt in enumerate(prompts)]
+    got = generate(engine, requests)
+    assert [result.tokens for result in got] == want
+    assert [result.finish_reason for result in got] == ["length" if len(t) == 24 else "stop" for t in want]
+    engine.cache.check()
+    assert engine.cache.slots.n_held == 0 and engine.cache.held_blocks() == 0

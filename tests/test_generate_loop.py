@@ -8,6 +8,7 @@ from ops_emulation import EmulatedOps
 import plain_llama as P
 from xeno_rt_amd.engine import (Engine, GenerateRequest, StepError, decide, generate, plan_batches,
                                 resolve_prompt)
+from xeno_rt_amd.engine.generate import goes_on_whatever_it_draws
 from xeno_rt_amd.sampling import SamplerConfig, uniform
 
 GREEDY = dict(temperature=0.0, repetition_penalty=1.0)
@@ -86,6 +87,77 @@ def test_stop_tokens_end_a_request_early_and_are_not_returned(pair):
     # the configuration's eos ids are the default stop set
     default = generate(engine, [GenerateRequest(prompt, max_tokens=8, **GREEDY)])[0]
     assert default.tokens == P.generate_greedy(plain, prompt, 8)
+
+
+def test_which_requests_may_be_stepped_before_their_token_is_seen():
+    """Exactly those that `decide` and the full context let go on with any token that is no stop token."""
+    for context in (4, 9):
+        for history in range(1, context + 1):
+            for max_tokens in (1, 2, 5):
+                for produced in range(max_tokens):
+                    keep, reason = decide(7, {1}, history, context, produced, max_tokens)
+                    goes_on = keep and reason is None and history + 1 < context
+                    assert goes_on_whatever_it_draws(history, context, produced, max_tokens) == goes_on
+
+
+def test_a_step_from_tokens_on_the_device_is_the_step_from_the_same_tokens(pair):
+    engine, _ = pair
+    prompts = [[4, 8, 15, 16], [42], [7] * 9]
+
+    def run(ahead):
+        slots = [engine.alloc_slot() for _ in prompts]
+        try:
+            engine.step([(slot, ids, []) for slot, ids in zip(slots, prompts)])
+            nexts = [11, 250, 3]
+            if ahead:       # rows in another order than the sequences, and one row that nobody reads
+                drawn = torch.tensor([nexts[2], 99, nexts[0], nexts[1]], dtype=torch.int32)
+                first = engine.step_from(drawn, [(slots[0], 2), (slots[1], 3), (slots[2], 0)])
+                second = engine.step_from(drawn, [(slots[2], 1)])
+            else:
+                first = engine.step([(slot, [token], [0]) for slot, token in zip(slots, nexts)])
+                second = engine.step([(slots[2], [99], [0])])
+            assert [engine.length(slot) for slot in slots] == [5, 2, 11]
+            return first.clone(), second.clone()
+        finally:
+            for slot in slots:
+                engine.free_slot(slot)
+
+    for got, want in zip(run(True), run(False)):
+        assert torch.equal(got, want)
+    slot = engine.alloc_slot()
+    try:
+        engine.step([(slot, [1, 2], [])])
+        with pytest.raises(StepError, match="outside the 2 tokens"):
+            engine.step_from(torch.tensor([1, 2], dtype=torch.int32), [(slot, 2)])
+        assert engine.length(slot) == 2
+    finally:
+        engine.free_slot(slot)
+    engine.cache.check()
+
+
+def test_the_loop_runs_a_step_ahead_unless_a_penalty_needs_the_history(pair, monkeypatch):
+    engine, plain = pair
+    calls = {"step": 0, "step_from": 0}
+    step, step_from = engine.step, engine.step_from
+    monkeypatch.setattr(engine, "step", lambda *a, **k: (calls.__setitem__("step", calls["step"] + 1), step(*a, **k))[1])
+    monkeypatch.setattr(engine, "step_from",
+                        lambda *a, **k: (calls.__setitem__("step_from", calls["step_from"] + 1), step_from(*a, **k))[1])
+    prompt = [4, 8, 15]
+    free = P.generate_greedy(plain, prompt, 8, stop_ids=[])
+    stop = free[3]
+    requests = [GenerateRequest(prompt, max_tokens=8, stop_ids=[stop], **GREEDY),
+                GenerateRequest([50, 60], max_tokens=6, stop_ids=[], **GREEDY)]
+    results = generate(engine, requests)
+    assert results[0].tokens == free[:3] and results[0].finish_reason == "stop"
+    assert results[1].tokens == P.generate_greedy(plain, [50, 60], 6, stop_ids=[])
+    # the prompts' step, then five steps for six tokens, none of them through the host
+    assert calls == {"step": 1, "step_from": 5}
+    calls.update(step=0, step_from=0)
+    penalised = [GenerateRequest(prompt, max_tokens=4, stop_ids=[], temperature=0.0, repetition_penalty=1.3)]
+    generate(engine, penalised)
+    assert calls == {"step": 4, "step_from": 0}
+    engine.cache.check()
+    assert engine.cache.slots.n_held == 0 and engine.cache.held_blocks() == 0
 
 
 def test_context_and_zero_length_limits(pair):

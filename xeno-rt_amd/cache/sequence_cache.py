@@ -22,6 +22,8 @@ from typing import Dict, List, Optional
 import numpy as np
 import torch
 
+from ..staging import staging_for
+
 from ..parts.base import CacheNeeds, KVSpec
 from .allocator import BLOCK_TOKENS, CacheError, CacheFull, Pool, blocks_for
 
@@ -56,7 +58,7 @@ class KVGroup:
         self._table = np.full((max_slots, max_blocks_per_sequence), -1, dtype=np.int32)
         self.table = torch.from_numpy(self._table)
         self.device_table = self.table.to(device)
-        self.dirty = False
+        self._changed = set()              # slots whose row of the table the device has not seen yet
         self._end: Dict[int, int] = {}     # slot -> logical blocks [floor, end) may be held
         self._floor: Dict[int, int] = {}   # slot -> lowest logical block it may still hold
         shape_k = (len(calls), n_blocks, spec.n_kv_heads, BLOCK_TOKENS, spec.head_dim)
@@ -90,7 +92,7 @@ class KVGroup:
             raise
         if added:
             self._end[slot] = need
-            self.dirty = True
+            self._changed.add(slot)
         return added
 
     def drop(self, slot: int, logicals: List[int]) -> None:
@@ -98,7 +100,7 @@ class KVGroup:
             self.pool.release(int(self._table[slot, logical]))
             self._table[slot, logical] = -1
         if logicals:
-            self.dirty = True
+            self._changed.add(slot)
             end = self._end.get(slot, 0)
             while end > 0 and self._table[slot, end - 1] < 0:
                 end -= 1
@@ -120,9 +122,12 @@ class KVGroup:
         self._end.pop(slot, None)
 
     def sync(self) -> None:
-        if self.dirty:
-            self.device_table.copy_(self.table, non_blocking=False)
-            self.dirty = False
+        """The rows that changed go to the device through pinned memory, in the order of the stream and
+        without waiting for it: a host that prepares the next step while this one runs is not held up."""
+        if self._changed:
+            low, high = min(self._changed), max(self._changed) + 1
+            staging_for(self.device_table.device).upload(self.table[low:high], out=self.device_table[low:high])
+            self._changed.clear()
 
 
 class SequenceCache:

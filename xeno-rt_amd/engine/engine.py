@@ -20,6 +20,7 @@ from ..config import architecture, load_config
 from ..models import DecoderModel, ModelSpec
 from ..parts.base import Runtime
 from ..weights import check_names, load_tensors, random_tensors
+from ..staging import staging_for
 from .batch import StepBatch, build_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
@@ -149,6 +150,30 @@ class Engine:
             raise
         for slot, start, ids in zip(slots, starts, tokens):
             self.cache.commit(slot, start + len(ids))
+        return logits
+
+    def step_from(self, tokens: torch.Tensor, entries: Sequence[Tuple[int, int]]) -> torch.Tensor:
+        """One more token for some sequences, taken from the device: entries are (slot, row), and the
+        sequence in `slot` goes on with tokens[row] (int32, ids below the vocabulary's size: what the
+        sampler wrote). Returns logits [len(entries), vocab] like `step`. Nothing here waits for the
+        device, so a caller can start the next step before it has seen the tokens of the last one."""
+        slots, _, _, starts = self.prepare([(slot, [0], [0]) for slot, _ in entries])
+        rows = [int(row) for _, row in entries]
+        try:
+            if min(rows) < 0 or max(rows) >= tokens.numel():
+                raise StepError(f"rows {rows} are outside the {tokens.numel()} tokens given")
+            if self.graphs is not None:
+                logits = self.graphs.step(slots, [0] * len(slots), starts, source=(tokens, rows))
+            else:
+                batch = build_batch(slots, [[0]] * len(slots), starts, [[0]] * len(slots), self.device)
+                batch.token_ids.copy_(tokens.index_select(0, staging_for(self.device).upload(rows)))
+                logits = self.model.forward(batch, self.cache)
+        except Exception:
+            for slot in slots:
+                self.cache.cancel(slot)
+            raise
+        for slot, start in zip(slots, starts):
+            self.cache.commit(slot, start + 1)
         return logits
 
     def prepare(self, entries):

@@ -86,6 +86,12 @@ def decide(token: int, stops, history_length: int, context: int, produced: int, 
     return True, None
 
 
+def goes_on_whatever_it_draws(history_length: int, context: int, produced: int, max_tokens: int) -> bool:
+    """Whether only a stop token can end the request at the token being sampled: then its next step may
+    start before the token has been looked at. The same conditions as in `decide` and in the loop below."""
+    return history_length + 1 < context and produced + 1 < max_tokens
+
+
 def plan_batches(prompt_lengths: Sequence[int], max_tokens: Sequence[int], batch_size: int,
                  block_tokens: int, cache_tokens: int, context: int) -> List[List[int]]:
     """Cut the requests, in order, into batches that fit the slots and the cache.
@@ -116,6 +122,7 @@ def generate(engine, requests: Sequence[GenerateRequest], batch_size: Optional[i
     on_token(request_index, token_id) is called for every token kept, as it is produced.
     """
     from ..cache import BLOCK_TOKENS
+    from ..staging import staging_for
 
     config = engine.config
     context = engine.max_context
@@ -146,13 +153,26 @@ def generate(engine, requests: Sequence[GenerateRequest], batch_size: Optional[i
             running = [seq for seq in live if seq.finish_reason is None]
             if running:
                 logits = engine.step([(seq.slot, seq.history, [len(seq.history) - 1]) for seq in running])
+            # One step ahead of the host: the next step starts from the sampled tokens on the device, for
+            # every request that only a stop token could end, and the host looks at the tokens while it
+            # runs. A request that did draw a stop token has then been stepped once for nothing; its row
+            # of logits is dropped. A repetition penalty needs the history on the host first.
+            ahead = all(seq.request.repetition_penalty <= 1.0 for seq in running)
             while running:
-                tokens = sampler.sample(
+                drawn = sampler.launch(
                     logits, [seq.request.sampler_config() for seq in running],
                     [seq.history for seq in running],
                     [uniform(seq.seed, 0, len(seq.produced)) for seq in running])
+                fetched = staging_for(engine.device).fetch(drawn)
+                stepped, logits = [], None
+                if ahead:
+                    stepped = [(row, seq) for row, seq in enumerate(running)
+                               if goes_on_whatever_it_draws(len(seq.history), context, len(seq.produced),
+                                                            seq.request.max_tokens)]
+                    if stepped:
+                        logits = engine.step_from(drawn, [(seq.slot, row) for row, seq in stepped])
                 still = []
-                for seq, token in zip(running, tokens):
+                for seq, token in zip(running, fetched.values()):
                     keep, reason = decide(token, seq.stops, len(seq.history), context,
                                           len(seq.produced), seq.request.max_tokens)
                     if keep:
@@ -165,9 +185,15 @@ def generate(engine, requests: Sequence[GenerateRequest], batch_size: Optional[i
                     seq.finish_reason = reason
                     if reason is None:
                         still.append(seq)
+                if ahead:
+                    kept = [i for i, (_, seq) in enumerate(stepped) if seq.finish_reason is None]
+                    if [stepped[i][1] for i in kept] != still:
+                        raise RuntimeError("a request went on that was not stepped ahead")
+                    if still and len(kept) < len(stepped):
+                        logits = logits.index_select(0, staging_for(engine.device).upload(kept))
+                elif still:
+                    logits = engine.step([(seq.slot, [seq.history[-1]], [0]) for seq in still])
                 running = still
-                if running:
-                    logits = engine.step([(seq.slot, [seq.history[-1]], [0]) for seq in running])
         finally:
             for seq in live:
                 engine.free_slot(seq.slot)

@@ -39,8 +39,8 @@ class DecodeGraph:
         self.size = size
         self.context = context
         self.device = device
-        # [token ids | positions | slots | sequence slots | offsets | starts | logit rows]
-        self.layout = [size, size, size, size, size + 1, size, size]
+        # [token ids | positions | slots | sequence slots | offsets | starts | logit rows | rows of the tokens' source]
+        self.layout = [size, size, size, size, size + 1, size, size, size]
         total = sum(self.layout)
         self.ints = torch.zeros(total, dtype=torch.int32, device=device)
         cuts, at = [], 0
@@ -52,6 +52,7 @@ class DecodeGraph:
             sequence_slots=cuts[3], sequence_offsets=cuts[4], sequence_starts=cuts[5], logit_rows=cuts[6],
             n_logit_rows=size, host_slots=[-1] * size, host_counts=[1] * size, host_starts=[0] * size,
             is_decode=True, max_count=1, max_context=context)
+        self.source_rows = cuts[7]
         self.fill([-1] * size, [0] * size, [0] * size)      # all padding: a harmless first run
         # one run outside the graph first: one-time set-up inside kernels' launchers must not be captured
         stream = torch.cuda.Stream(device=device)
@@ -64,15 +65,21 @@ class DecodeGraph:
         with torch.cuda.graph(self.graph):
             self.logits = model.forward(self.batch, cache)
 
-    def fill(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int]) -> None:
+    def fill(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int], source=None) -> None:
+        """New contents for the step's arrays. With source = (tokens on the device, a row for each sequence)
+        the token ids are gathered from there, after the upload and before the replay."""
         size, count = self.size, len(slots)
         pad = size - count
+        rows = list(source[1]) if source is not None else [0] * count
         values = (list(tokens) + [0] * pad + list(starts) + [0] * pad + list(slots) + [-1] * pad
-                  + list(slots) + [-1] * pad + list(range(size + 1)) + list(starts) + [0] * pad + list(range(size)))
+                  + list(slots) + [-1] * pad + list(range(size + 1)) + list(starts) + [0] * pad + list(range(size))
+                  + rows + [0] * pad)
         staging_for(self.device).upload(values, out=self.ints)
+        if source is not None:
+            torch.index_select(source[0], 0, self.source_rows[:count], out=self.batch.token_ids[:count])
 
-    def run(self, slots, tokens, starts) -> torch.Tensor:
-        self.fill(slots, tokens, starts)
+    def run(self, slots, tokens, starts, source=None) -> torch.Tensor:
+        self.fill(slots, tokens, starts, source)
         self.graph.replay()
         return self.logits
 
@@ -84,11 +91,12 @@ class DecodeGraphs:
         self.device = device
         self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}
 
-    def step(self, slots: List[int], tokens: List[int], starts: List[int]) -> torch.Tensor:
-        """Logits [len(slots), vocab] of one decode step; a copy, valid until the caller drops it."""
+    def step(self, slots: List[int], tokens: List[int], starts: List[int], source=None) -> torch.Tensor:
+        """Logits [len(slots), vocab] of one decode step; a copy, valid until the caller drops it.
+        source: (int32 tokens on the device, a row of them for each sequence) instead of `tokens`."""
         size = batch_bucket(len(slots))
         context = context_bucket(max(starts) + 1, self.cache.max_context)
         key = (size, context)
         if key not in self.graphs:
             self.graphs[key] = DecodeGraph(self.model, self.cache, size, context, self.device)
-        return self.graphs[key].run(slots, tokens, starts)[:len(slots)].clone()
+        return self.graphs[key].run(slots, tokens, starts, source)[:len(slots)].clone()

@@ -67,8 +67,14 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, configs: Sequence[SamplerConfig],
                histories: Sequence[Sequence[int]], draws: Sequence[float]) -> List[int]:
+        """The token ids that `launch` chooses, on the host."""
+        return self.launch(logits, configs, histories, draws).tolist()
+
+    def launch(self, logits: torch.Tensor, configs: Sequence[SamplerConfig],
+               histories: Sequence[Sequence[int]], draws: Sequence[float]) -> torch.Tensor:
         """logits [rows, vocab] float32; for each row its options, the tokens of its sequence so
-        far (read only if its penalty is > 1) and its uniform number. Returns the token ids."""
+        far (read only if its penalty is > 1) and its uniform number. Returns the token ids as an
+        int32 tensor on the device, without waiting for them: a step can be started from them."""
         rows = logits.shape[0]
         if logits.dim() != 2 or logits.shape[1] == 0:
             raise ValueError("cannot sample from an empty logits vector")     # sampler.rs:56-60
@@ -87,9 +93,10 @@ class Sampler:
         if self._last is not None and self._last[0] == made_from:
             floats, ints = self._last[1]
         else:
-            floats = torch.tensor(
-                [[c.temperature for c in configs], [c.top_p for c in configs],
-                 [c.repetition_penalty for c in configs], list(draws)], dtype=torch.float32).to(self.device)
+            floats = staging_for(self.device).upload(
+                [c.temperature for c in configs] + [c.top_p for c in configs]
+                + [c.repetition_penalty for c in configs] + [float(d) for d in draws],
+                dtype=torch.float32).view(4, rows)
             ints = staging_for(self.device).upload([c.top_k for c in configs] + offsets + history)
             self._last = (made_from, (floats, ints))
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
@@ -97,4 +104,4 @@ class Sampler:
         small_top_k = any(not c.is_greedy() and (0 < c.top_k <= 64 or (c.top_k == 0 and c.top_p < 1.0)) for c in configs)
         self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2],
                         ints[2 * rows + 1:], ints[rows:2 * rows + 1], floats[3], small_top_k=small_top_k)
-        return out.tolist()
+        return out
