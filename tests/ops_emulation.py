@@ -138,12 +138,19 @@ class EmulatedOps:
                 out[t, head * head_dim:(head + 1) * head_dim] = (probs @ values[:, kvh, :]).to(out.dtype)
 
     # -- sampling ---------------------------------------------------------------
-    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms,
-               small_top_k=False):
+    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms,
+               small_top_k=False, append_at=None):
         rows, vocab = logits.shape
         for r in range(rows):
+            self._sample_row(r, logits, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms)
+            if append_at is not None and int(append_at[r]) >= 0:
+                history[int(append_at[r])] = out[r]
+
+    def _sample_row(self, r, logits, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms):
+        vocab = logits.shape[1]
+        for _ in range(1):
             row = logits[r].to(torch.float32).clone()
-            seen = history[int(history_offsets[r]):int(history_offsets[r + 1])].long()
+            seen = history[int(history_spans[2 * r]):int(history_spans[2 * r + 1])].long()
             pen = float(penalty[r])
             if pen > 1.0 and seen.numel() > 0:
                 seen = torch.unique(seen)

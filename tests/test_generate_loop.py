@@ -9,7 +9,7 @@ import plain_llama as P
 from xeno_rt_amd.engine import (Engine, GenerateRequest, StepError, decide, generate, plan_batches,
                                 resolve_prompt)
 from xeno_rt_amd.engine.generate import goes_on_whatever_it_draws
-from xeno_rt_amd.sampling import SamplerConfig, uniform
+from xeno_rt_amd.sampling import Sampler, SamplerConfig, TokenLog, uniform
 
 GREEDY = dict(temperature=0.0, repetition_penalty=1.0)
 
@@ -135,7 +135,7 @@ def test_a_step_from_tokens_on_the_device_is_the_step_from_the_same_tokens(pair)
     engine.cache.check()
 
 
-def test_the_loop_runs_a_step_ahead_unless_a_penalty_needs_the_history(pair, monkeypatch):
+def test_the_loop_runs_a_step_ahead_of_the_host(pair, monkeypatch):
     engine, plain = pair
     calls = {"step": 0, "step_from": 0}
     step, step_from = engine.step, engine.step_from
@@ -152,10 +152,24 @@ def test_the_loop_runs_a_step_ahead_unless_a_penalty_needs_the_history(pair, mon
     assert results[1].tokens == P.generate_greedy(plain, [50, 60], 6, stop_ids=[])
     # the prompts' step, then five steps for six tokens, none of them through the host
     assert calls == {"step": 1, "step_from": 5}
+    # with a repetition penalty too: the tokens it reads are kept on the device (the sampler appends them), and
+    # they are those that a loop through the host hands to the sampler at every step
     calls.update(step=0, step_from=0)
-    penalised = [GenerateRequest(prompt, max_tokens=4, stop_ids=[], temperature=0.0, repetition_penalty=1.3)]
-    generate(engine, penalised)
-    assert calls == {"step": 4, "step_from": 0}
+    prompt = [43, 44, 45]           # left alone, the model repeats its second token from here on
+    penalised = GenerateRequest(prompt, max_tokens=5, stop_ids=[], temperature=0.0, repetition_penalty=3.0)
+    got = generate(engine, [penalised, GenerateRequest([50, 60], max_tokens=3, stop_ids=[], **GREEDY)])
+    assert calls == {"step": 1, "step_from": 4}
+    sampler, slot, history = Sampler(engine.ops, engine.device), engine.alloc_slot(), list(prompt)
+    monkeypatch.undo()
+    logits = engine.step([(slot, history, [len(history) - 1])])
+    for _ in range(5):
+        history += sampler.sample(logits, [penalised.sampler_config()], [history], [0.0])
+        logits = engine.step([(slot, history[-1:], [0])])
+    engine.free_slot(slot)
+    assert got[0].tokens == history[len(prompt):]
+    free = P.generate_greedy(plain, prompt, 5, stop_ids=[])
+    assert free[1] == free[2] and got[0].tokens[:2] == free[:2] and got[0].tokens[2] != free[2]   # a token it chose itself is penalised
+    assert got[1].tokens == P.generate_greedy(plain, [50, 60], 3, stop_ids=[])
     engine.cache.check()
     assert engine.cache.slots.n_held == 0 and engine.cache.held_blocks() == 0
 

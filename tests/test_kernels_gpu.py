@@ -117,6 +117,33 @@ def test_linear_glu(ops, dtype, m, n, k):
     assert rel(out.cpu(), want) < ULP[dtype] * 2
 
 
+def test_linear_of_more_elements_than_32_bit_offsets_reach(ops):
+    """x with 2^31 elements and more (a step of many long prompts times a wide feed-forward) goes through the
+    matrix-core kernels in runs of rows: rows at the runs' edges are right, and the same as in a product of their own."""
+    k, n = 16384, 96
+    run = (2 ** 31 - 1) // k // 256 * 256
+    m = 2 ** 31 // k + 300                                      # two runs, the second short
+    assert run < m and m * k > 2 ** 31
+    generator = torch.Generator(device=DEV).manual_seed(3)
+    a = torch.empty(m, k, dtype=torch.bfloat16, device=DEV)
+    for begin in range(0, m, 16384):                             # filled piecewise: no float32 copy of 8 GB
+        a[begin:begin + 16384] = torch.randn(min(16384, m - begin), k, generator=generator, device=DEV) * 0.5
+    w = rand(2 * n, k, dtype=torch.bfloat16, seed=4, scale=0.05)
+    rows = [0, 1000, run - 1, run, run + 1, m - 1]
+    out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops.linear_glu(a, w, out)
+    acc = torch.zeros(m, 2 * n, device=DEV)
+    ops.linear(a, w, acc, accumulate=True)
+    torch.cuda.synchronize()
+    picked = a[rows].contiguous()
+    both = picked.double().cpu() @ w.double().cpu().t()
+    assert rel(acc[rows].cpu(), both) < 1e-5
+    assert rel(out[rows].cpu(), P.swiglu(both[:, :n], both[:, n:])) < ULP["bfloat16"] * 2
+    across = torch.zeros(512, 2 * n, device=DEV)                 # the rows on both sides of the edge, as one product
+    ops.linear(a[run - 256:run + 256].contiguous(), w, across, accumulate=True)
+    assert rel(across.cpu(), acc[run - 256:run + 256].cpu().double()) < 1e-5    # (split along k: another order of the sum)
+
+
 def test_linear_rows_do_not_depend_on_the_batch(ops):
     a = rand(70, 200, seed=3)
     w = rand(130, 200, seed=4)
@@ -525,7 +552,7 @@ def test_matrix_core_attention_finds_a_far_key(ops):
 def sample(ops, logits, temperature=0.0, top_k=0, top_p=1.0, penalty=1.0, history=(), draws=None):
     rows = logits.shape[0]
     f = lambda v: torch.full((rows,), float(v), device=DEV)
-    offsets = i32([len(history) * r for r in range(rows + 1)])
+    offsets = i32([len(history) * (r + e) for r in range(rows) for e in (0, 1)])   # a span (begin, end) per row
     out = torch.empty(rows, dtype=torch.int32, device=DEV)
     uniforms = torch.tensor(draws if draws is not None else [0.5] * rows, dtype=torch.float32, device=DEV)
     operands = (logits, out, f(temperature), torch.full((rows,), top_k, dtype=torch.int32, device=DEV), f(top_p),
@@ -610,6 +637,40 @@ def test_sample_with_ties_by_the_thousand_and_a_large_top_k(ops):
         assert set(torch.nonzero(counts).flatten().tolist()) <= set(torch.nonzero(dist).flatten().tolist())
 
 
+def test_sample_keeps_the_tokens_on_the_device_where_asked(ops):
+    """With append_at the chosen token is also written behind the row's span of the history, on every way
+    through the kernels (greedy, passes over the row, candidates from slices), and only for the rows
+    that ask for it; what it wrote is what the penalty of the next call reads."""
+    torch.manual_seed(5)
+    rows, vocab = 5, 40000
+    logits = (torch.randn(rows, vocab) * 3.0).to(DEV)
+    temperature = torch.tensor([0.0, 0.9, 0.9, 1.0, 0.0], device=DEV)
+    top_k = i32([0, 40, 0, 8, 0])
+    top_p = torch.tensor([1.0, 0.95, 1.0, 0.9, 1.0], device=DEV)
+    penalty = torch.tensor([1.0, 1.2, 1.0, 1.0, 1.0e9], device=DEV)
+    uniforms = torch.tensor([0.1, 0.5, 0.7, 0.3, 0.2], device=DEV)
+    room = 6
+    for small in (False, True):
+        history = torch.full((rows * room,), -7, dtype=torch.int32, device=DEV)
+        lengths = [0] * rows
+        picked = []
+        for step in range(3):
+            spans = i32([r * room + e * lengths[r] for r in range(rows) for e in (0, 1)])
+            append_at = i32([r * room + lengths[r] if r != 2 else -1 for r in range(rows)])   # row 2 keeps nothing
+            out = torch.empty(rows, dtype=torch.int32, device=DEV)
+            ops.sample(logits, out, temperature, top_k, top_p, penalty, history, spans, uniforms,
+                       small_top_k=small, append_at=append_at)
+            picked.append(out.tolist())
+            lengths = [n + (1 if r != 2 else 0) for r, n in enumerate(lengths)]
+        kept = history.view(rows, room).tolist()
+        for r in range(rows):
+            want = [step[r] for step in picked] if r != 2 else []
+            assert kept[r] == want + [-7] * (room - len(want)), (small, r)
+        # row 4 is greedy with a crushing penalty: it reads what it wrote and never takes a token twice
+        assert len(set(kept[4][:3])) == 3 and picked[0][4] == int(logits[4].argmax())
+        assert picked[0][0] == picked[1][0] == int(logits[0].argmax())      # no penalty: the same token again
+
+
 @pytest.mark.parametrize("vocab", [32768 - 4095, 40000, 151936])
 def test_sample_small_top_k_through_slices(ops, vocab):
     """Rows of every kind in one call (greedy, no top-k, top-k of 1, 40 and 64, a penalty, ties that overflow a
@@ -630,7 +691,7 @@ def test_sample_small_top_k_through_slices(ops, vocab):
     top_p = torch.tensor([1.0, 0.9, 1.0, 0.95, 0.5, 1.0, 1.0, 0.9, 1.0, 0.9, 0.95, 0.8], device=DEV)
     penalty = torch.tensor([1.0, 1.0, 1.0, 1.1, 2.0, 1.0, 1.0, 1.5, 1.0, 1.0, 1.0, 1.0], device=DEV)
     history = i32(list(range(0, vocab, 997)))
-    offsets = i32([0, 0, 0, 0] + [len(history)] * 9)               # the history is row 3's alone
+    offsets = i32([0, 0] * 3 + [0, len(history)] + [0, 0] * 8)     # the history is row 3's alone
     for draw in (0.03, 0.37, 0.71, 0.93, 0.999):
         uniforms = torch.full((rows,), draw, device=DEV)
         whole, sliced = torch.empty(rows, dtype=torch.int32, device=DEV), torch.full((rows,), -1, dtype=torch.int32, device=DEV)

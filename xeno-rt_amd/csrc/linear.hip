@@ -31,6 +31,18 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
     XRT_REQUIRE(mode != 1 || out_dtype == XRT_F32, "linear: accumulation needs a float32 output");
     XRT_REQUIRE(a && w && out, "linear: null operand");
     if (M == 0) return 0;
+    // The matrix-core kernels address their operands with 32-bit offsets. A step of so many tokens that x
+    // exceeds them (a batch of long prompts) goes in runs of rows; an output element's sum is the same.
+    if (dtype == XRT_BF16 && (long)M * K >= (1L << 31) && K <= (1 << 22)) {
+        const int run = (int)(((1L << 31) - 1) / K / 256 * 256);
+        const long out_row = (long)N * (out_dtype == XRT_F32 ? 4 : 2);
+        for (int m0 = 0; m0 < M; m0 += run) {
+            const int status = xrt_linear((const char*)a + (long)m0 * K * 2, w, dtype, (char*)out + m0 * out_row, out_dtype,
+                                          M - m0 < run ? M - m0 : run, N, K, mode, workspace, workspace_floats, stream);
+            if (status != 0) return status;
+        }
+        return 0;
+    }
     // bfloat16: the matrix-core kernels; float32, and shapes they refuse: the plain kernel
     if (dtype == XRT_BF16) {
         long need = 0;

@@ -95,12 +95,24 @@ __device__ __forceinline__ void block_sums(T (&v)[N], T* scratch) {
     for (int j = 0; j < N; ++j) v[j] = scratch[BLOCK_WAVES * N + j];
 }
 
+// Where a row's token goes: out[r], and, for a caller that keeps the sequences' tokens on the device (what
+// the penalty reads), the place behind the row's span of them.
+struct Chosen {
+    int* out;
+    int* history;
+    const int* append_at;
+    __device__ __forceinline__ void put(int r, int token) const {
+        out[r] = token;
+        if (append_at != nullptr && append_at[r] >= 0) history[append_at[r]] = token;
+    }
+};
+
 // The whole of it for row r, by one workgroup of THREADS threads; `seen` holds vocab bits of LDS.
 __device__ void sample_row(
     const int r, unsigned* seen,
-    const float* __restrict__ logits, int vocab, int* __restrict__ out, const float* __restrict__ temperature,
+    const float* __restrict__ logits, int vocab, const Chosen out, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ penalty,
-    const int* __restrict__ history, const int* __restrict__ history_offsets, const float* __restrict__ uniforms) {
+    const int* __restrict__ history, const int* __restrict__ history_spans, const float* __restrict__ uniforms) {
     __shared__ float scratch_f[(BLOCK_WAVES + 1) * SUMS];
     __shared__ unsigned scratch_u[(BLOCK_WAVES + 1) * SUMS];
     __shared__ int survivor_id[BLOCK_WAVES * SEGMENT];      // what top-k leaves, by wavefront run, in the order of ids
@@ -118,7 +130,7 @@ __device__ void sample_row(
     row.seen = seen;
     row.penalty = penalty[r];
     row.vocab = vocab;
-    const int h_begin = history_offsets[r], h_end = history_offsets[r + 1];
+    const int h_begin = history_spans[2 * r], h_end = history_spans[2 * r + 1];
     row.penalised = row.penalty > 1.0f && h_end > h_begin;
     if (row.penalised) {
         const int words = (vocab + 31) / 32;
@@ -155,7 +167,7 @@ __device__ void sample_row(
 
     const float temp = temperature[r];
     if (temp <= 1e-5f) {
-        if (tid == 0) out[r] = best_index;
+        if (tid == 0) out.put(r, best_index);
         return;
     }
     const float inv_temp = 1.0f / temp;
@@ -290,7 +302,7 @@ __device__ void sample_row(
                         }
                     }
                 if (pick < 0) pick = last_kept;         // rounding at the end: the last kept token
-                out[r] = pick >= 0 ? pick : best_index; // sampler.rs:195: fall back to the top candidate
+                out.put(r, pick >= 0 ? pick : best_index); // sampler.rs:195: fall back to the top candidate
             }
             return;
         }
@@ -398,15 +410,15 @@ __device__ void sample_row(
         if (lane == 0) chosen = pick;
     }
     __syncthreads();
-    if (tid == 0) out[r] = chosen >= 0 ? chosen : best_index;   // sampler.rs:195: fall back to the top candidate
+    if (tid == 0) out.put(r, chosen >= 0 ? chosen : best_index);   // sampler.rs:195: fall back to the top candidate
 }
 
 __global__ void __launch_bounds__(THREADS) sample_kernel(
-    const float* __restrict__ logits, int vocab, int* __restrict__ out, const float* __restrict__ temperature,
+    const float* __restrict__ logits, int vocab, const Chosen out, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ penalty,
-    const int* __restrict__ history, const int* __restrict__ history_offsets, const float* __restrict__ uniforms) {
+    const int* __restrict__ history, const int* __restrict__ history_spans, const float* __restrict__ uniforms) {
     extern __shared__ unsigned seen[];                 // vocab bits
-    sample_row(blockIdx.x, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms);
+    sample_row(blockIdx.x, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms);
 }
 
 // ---- a small top-k: candidates by slice, then the row ---------------------------------------------
@@ -464,7 +476,7 @@ __device__ __forceinline__ int place_of_maximum(unsigned mine, unsigned* maxima)
 __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
     const float* __restrict__ logits, int vocab, const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const float* __restrict__ penalty, const int* __restrict__ history,
-    const int* __restrict__ history_offsets, SliceCandidates* __restrict__ candidates, int slices) {
+    const int* __restrict__ history_spans, SliceCandidates* __restrict__ candidates, int slices) {
     __shared__ unsigned seen[SLICE / 32];
     __shared__ __attribute__((aligned(16))) unsigned maxima[SLICE_THREADS];
     __shared__ unsigned bound;
@@ -479,7 +491,7 @@ __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
     }
     const int first = slice * SLICE;
     const float factor = penalty[r];
-    const int h_begin = history_offsets[r], h_end = history_offsets[r + 1];
+    const int h_begin = history_spans[2 * r], h_end = history_spans[2 * r + 1];
     const bool penalised = factor > 1.0f && h_end > h_begin;
     if (tid < SLICE / 32) seen[tid] = 0u;
     if (tid == 0) held = 0;
@@ -550,9 +562,9 @@ __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
 }
 
 __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
-    const float* __restrict__ logits, int vocab, int* __restrict__ out, const float* __restrict__ temperature,
+    const float* __restrict__ logits, int vocab, const Chosen out, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ penalty,
-    const int* __restrict__ history, const int* __restrict__ history_offsets, const float* __restrict__ uniforms,
+    const int* __restrict__ history, const int* __restrict__ history_spans, const float* __restrict__ uniforms,
     const SliceCandidates* __restrict__ candidates, int slices) {
     extern __shared__ unsigned seen[];                 // vocab bits, for the rows that take the whole-row path
     __shared__ float scratch_f[(BLOCK_WAVES + 1) * SUMS];
@@ -613,7 +625,7 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
     __syncthreads();
     if (first_place[0] < 0) {                                   // the same for all threads
         __syncthreads();
-        sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms);
+        sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms);
         return;
     }
     const int total = first_place[slices];
@@ -648,7 +660,7 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
     const int listed = kept;
     if (listed > ROW_HOLDS) {                                   // ties by the thousand
         __syncthreads();
-        sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms);
+        sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms);
         return;
     }
     // ... in which the k-th largest is the one that k - 1 others come before (ties: lower id first); it and
@@ -696,7 +708,7 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
         block_sums(stayed, scratch_f);                          // has a barrier before row_mass is read
         if (!(stayed[0] >= p * row_mass)) {
             __syncthreads();
-            sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms);
+            sample_row(r, seen, logits, vocab, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms);
             return;
         }
     }
@@ -734,7 +746,7 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
             }
         }
         if (pick < 0) pick = last_kept;                         // rounding at the end: the last kept token
-        if (tid == 0) out[r] = sorted_id[pick];                 // n >= 1: the largest candidate has weight 1
+        if (tid == 0) out.put(r, sorted_id[pick]);                 // n >= 1: the largest candidate has weight 1
         return;
     }
     // top-p: the largest weight threshold whose kept mass reaches p * total, as on the whole row
@@ -771,7 +783,7 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
             }
         }
         if (pick < 0) pick = last_kept;                         // rounding at the end: the last kept token
-        out[r] = pick;                                          // n >= 1: the largest candidate has weight 1
+        out.put(r, pick);                                          // n >= 1: the largest candidate has weight 1
     }
 }
 
@@ -784,30 +796,32 @@ extern "C" long xrt_sample_workspace(int rows, int vocab) {
 }
 
 extern "C" int xrt_sample(const float* logits, int rows, int vocab, int* out, const float* temperature,
-                          const int* top_k, const float* top_p, const float* penalty, const int* history,
-                          const int* history_offsets, const float* uniforms, void* workspace, long workspace_bytes,
-                          void* stream) {
+                          const int* top_k, const float* top_p, const float* penalty, int* history,
+                          const int* history_spans, const int* append_at, const float* uniforms, void* workspace,
+                          long workspace_bytes, void* stream) {
     XRT_REQUIRE(rows >= 0, "sample: negative row count");
     XRT_REQUIRE(vocab > 0, "sample: cannot sample from an empty logits vector");          // sampler.rs:56-60
     XRT_REQUIRE(vocab <= MAX_VOCAB, "sample: vocabulary %d exceeds %d", vocab, MAX_VOCAB);
-    XRT_REQUIRE(logits && out && temperature && top_k && top_p && penalty && history_offsets && uniforms,
+    XRT_REQUIRE(logits && out && temperature && top_k && top_p && penalty && history_spans && uniforms,
                 "sample: null operand");
+    XRT_REQUIRE(append_at == nullptr || history != nullptr, "sample: tokens to append and no history to append them to");
     if (rows == 0) return 0;
+    const Chosen chosen{out, history, append_at};
     const size_t lds = (size_t)((vocab + 31) / 32) * sizeof(unsigned);
     const long need = xrt_sample_workspace(rows, vocab);
     if (workspace != nullptr && need > 0 && workspace_bytes >= need) {
         const int slices = (vocab + SLICE - 1) / SLICE;
         sample_slices_kernel<<<dim3(slices, rows), SLICE_THREADS, 0, (hipStream_t)stream>>>(
-            logits, vocab, temperature, top_k, top_p, penalty, history, history_offsets, (SliceCandidates*)workspace, slices);
+            logits, vocab, temperature, top_k, top_p, penalty, history, history_spans, (SliceCandidates*)workspace, slices);
         XRT_LAUNCH_CHECK("sample (slices)");
         sample_candidates_kernel<<<rows, THREADS, lds, (hipStream_t)stream>>>(
-            logits, vocab, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms,
+            logits, vocab, chosen, temperature, top_k, top_p, penalty, history, history_spans, uniforms,
             (const SliceCandidates*)workspace, slices);
         XRT_LAUNCH_CHECK("sample (candidates)");
         return 0;
     }
-    sample_kernel<<<rows, THREADS, lds, (hipStream_t)stream>>>(logits, vocab, out, temperature, top_k, top_p,
-                                                              penalty, history, history_offsets, uniforms);
+    sample_kernel<<<rows, THREADS, lds, (hipStream_t)stream>>>(logits, vocab, chosen, temperature, top_k, top_p,
+                                                              penalty, history, history_spans, uniforms);
     XRT_LAUNCH_CHECK("sample");
     return 0;
 }

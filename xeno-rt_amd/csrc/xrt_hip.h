@@ -81,10 +81,13 @@ int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_
 // one token per row of float32 logits. With a workspace of xrt_sample_workspace(rows, vocab) bytes (0: this
 // vocabulary gains nothing from it) rows with a top-k of 1 to 64 are sampled from candidates that
 // workgroups find slice by slice, instead of in eight passes over the row; without, all rows take the passes.
+// The penalty of row r reads history[history_spans[2r] .. history_spans[2r + 1]); with append_at (may be
+// null) the row's token is also written to history[append_at[r]] (nowhere if that is negative), so that a
+// caller can keep the sequences' tokens on the device.
 int xrt_sample(const float* logits, int rows, int vocab, int* out, const float* temperature,
-               const int* top_k, const float* top_p, const float* penalty, const int* history,
-               const int* history_offsets, const float* uniforms, void* workspace, long workspace_bytes,
-               void* stream);
+               const int* top_k, const float* top_p, const float* penalty, int* history,
+               const int* history_spans, const int* append_at, const float* uniforms, void* workspace,
+               long workspace_bytes, void* stream);
 long xrt_sample_workspace(int rows, int vocab);
 
 #ifdef __cplusplus

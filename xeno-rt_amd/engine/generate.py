@@ -122,6 +122,7 @@ def generate(engine, requests: Sequence[GenerateRequest], batch_size: Optional[i
     on_token(request_index, token_id) is called for every token kept, as it is produced.
     """
     from ..cache import BLOCK_TOKENS
+    from ..sampling import TokenLog
     from ..staging import staging_for
 
     config = engine.config
@@ -156,21 +157,24 @@ def generate(engine, requests: Sequence[GenerateRequest], batch_size: Optional[i
             # One step ahead of the host: the next step starts from the sampled tokens on the device, for
             # every request that only a stop token could end, and the host looks at the tokens while it
             # runs. A request that did draw a stop token has then been stepped once for nothing; its row
-            # of logits is dropped. A repetition penalty needs the history on the host first.
-            ahead = all(seq.request.repetition_penalty <= 1.0 for seq in running)
+            # of logits is dropped. The tokens that a repetition penalty reads are kept on the device.
+            log, place = None, {}
+            if any(seq.request.repetition_penalty > 1.0 for seq in running):
+                log = TokenLog(engine.device, [seq.history for seq in running],
+                               [seq.request.max_tokens + 1 for seq in running])
+                place = {seq.index: at for at, seq in enumerate(running)}
             while running:
                 drawn = sampler.launch(
                     logits, [seq.request.sampler_config() for seq in running],
                     [seq.history for seq in running],
-                    [uniform(seq.seed, 0, len(seq.produced)) for seq in running])
+                    [uniform(seq.seed, 0, len(seq.produced)) for seq in running],
+                    log=None if log is None else (log, [place[seq.index] for seq in running]))
                 fetched = staging_for(engine.device).fetch(drawn)
-                stepped, logits = [], None
-                if ahead:
-                    stepped = [(row, seq) for row, seq in enumerate(running)
-                               if goes_on_whatever_it_draws(len(seq.history), context, len(seq.produced),
-                                                            seq.request.max_tokens)]
-                    if stepped:
-                        logits = engine.step_from(drawn, [(seq.slot, row) for row, seq in stepped])
+                stepped = [(row, seq) for row, seq in enumerate(running)
+                           if goes_on_whatever_it_draws(len(seq.history), context, len(seq.produced),
+                                                        seq.request.max_tokens)]
+                if stepped:
+                    logits = engine.step_from(drawn, [(seq.slot, row) for row, seq in stepped])
                 still = []
                 for seq, token in zip(running, fetched.values()):
                     keep, reason = decide(token, seq.stops, len(seq.history), context,
@@ -185,14 +189,11 @@ def generate(engine, requests: Sequence[GenerateRequest], batch_size: Optional[i
                     seq.finish_reason = reason
                     if reason is None:
                         still.append(seq)
-                if ahead:
-                    kept = [i for i, (_, seq) in enumerate(stepped) if seq.finish_reason is None]
-                    if [stepped[i][1] for i in kept] != still:
-                        raise RuntimeError("a request went on that was not stepped ahead")
-                    if still and len(kept) < len(stepped):
-                        logits = logits.index_select(0, staging_for(engine.device).upload(kept))
-                elif still:
-                    logits = engine.step([(seq.slot, [seq.history[-1]], [0]) for seq in still])
+                kept = [i for i, (_, seq) in enumerate(stepped) if seq.finish_reason is None]
+                if [stepped[i][1] for i in kept] != still:
+                    raise RuntimeError("a request went on that was not stepped ahead")
+                if still and len(kept) < len(stepped):
+                    logits = logits.index_select(0, staging_for(engine.device).upload(kept))
                 running = still
         finally:
             for seq in live:

@@ -292,9 +292,11 @@ class HipOps:
             ctypes.c_float(scale), int(window or 0), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
 
-    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_offsets, uniforms,
-               small_top_k=False):
-        """small_top_k: some row has a temperature and a top-k of 1 to 64, or a top-p without top-k: worth the
+    def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms,
+               small_top_k=False, append_at=None):
+        """Row r's penalty reads history[history_spans[2r]:history_spans[2r + 1]]; with append_at, row r's
+        token is also written to history[append_at[r]] (nowhere if negative).
+        small_top_k: some row has a temperature and a top-k of 1 to 64, or a top-p without top-k: worth the
         kernels that look for candidates slice by slice."""
         if logits.dim() != 2:
             raise KernelError("sample: logits must be [rows, vocab]")
@@ -304,11 +306,13 @@ class HipOps:
         for what, tensor, dtype, shape in (
                 ("temperature", temperature, torch.float32, (rows,)), ("top_k", top_k, torch.int32, (rows,)),
                 ("top_p", top_p, torch.float32, (rows,)), ("penalty", penalty, torch.float32, (rows,)),
-                ("history_offsets", history_offsets, torch.int32, (rows + 1,)),
+                ("history_spans", history_spans, torch.int32, (2 * rows,)),
                 ("uniforms", uniforms, torch.float32, (rows,)), ("history", history, torch.int32, None)):
             self._require(tensor, f"sample {what}", dtype, shape, logits)
+        if append_at is not None:
+            self._require(append_at, "sample append_at", torch.int32, (rows,), logits)
         need = int(self.lib.xrt_sample_workspace(rows, vocab)) if small_top_k else 0
         workspace = torch.empty(need, dtype=torch.uint8, device=logits.device) if need > 0 else None
         self._check(self.lib.xrt_sample(_ptr(logits), rows, vocab, _ptr(out), _ptr(temperature), _ptr(top_k),
-                                        _ptr(top_p), _ptr(penalty), _ptr(history), _ptr(history_offsets),
-                                        _ptr(uniforms), _ptr(workspace), ctypes.c_long(need), self._stream(logits)))
+                                        _ptr(top_p), _ptr(penalty), _ptr(history), _ptr(history_spans),
+                                        _ptr(append_at), _ptr(uniforms), _ptr(workspace), ctypes.c_long(need), self._stream(logits)))

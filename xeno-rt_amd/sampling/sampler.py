@@ -57,6 +57,25 @@ def uniform(seed: int, request: int, step: int) -> float:
     return (word >> 40) / float(1 << 24)
 
 
+class TokenLog:
+    """The tokens of some sequences on the device, for the repetition penalty: what each has when the log is
+    made is uploaded once, and the sampling kernel itself appends what it chooses. Without a log the whole
+    history of every penalised row goes to the device at every step."""
+
+    def __init__(self, device, sequences: Sequence[Sequence[int]], room: Sequence[int]):
+        """room[i]: tokens that sequence i may still get."""
+        self.begin: List[int] = []
+        at = 0
+        for tokens, more in zip(sequences, room):
+            self.begin.append(at)
+            at += len(tokens) + max(0, int(more))
+        host = torch.zeros(max(at, 1), dtype=torch.int32)
+        for begin, tokens in zip(self.begin, sequences):
+            host[begin:begin + len(tokens)] = torch.tensor(list(tokens), dtype=torch.int32)
+        self.end = self.begin[1:] + [at]
+        self.tokens = staging_for(device).upload(host)
+
+
 class Sampler:
     """Samples one token for each row of a batch of logits, on the device."""
 
@@ -66,30 +85,43 @@ class Sampler:
         self._last = None           # (what the operands were made from, the operands): a decode loop asks the same again
 
     def sample(self, logits: torch.Tensor, configs: Sequence[SamplerConfig],
-               histories: Sequence[Sequence[int]], draws: Sequence[float]) -> List[int]:
+               histories: Sequence[Sequence[int]], draws: Sequence[float], log=None) -> List[int]:
         """The token ids that `launch` chooses, on the host."""
-        return self.launch(logits, configs, histories, draws).tolist()
+        return self.launch(logits, configs, histories, draws, log).tolist()
 
     def launch(self, logits: torch.Tensor, configs: Sequence[SamplerConfig],
-               histories: Sequence[Sequence[int]], draws: Sequence[float]) -> torch.Tensor:
+               histories: Sequence[Sequence[int]], draws: Sequence[float], log=None) -> torch.Tensor:
         """logits [rows, vocab] float32; for each row its options, the tokens of its sequence so
         far (read only if its penalty is > 1) and its uniform number. Returns the token ids as an
-        int32 tensor on the device, without waiting for them: a step can be started from them."""
+        int32 tensor on the device, without waiting for them: a step can be started from them.
+
+        log: (a TokenLog, for each row its sequence's index there). The penalty then reads the tokens
+        from the log, of which `histories` only tell the count, and the chosen token is appended."""
         rows = logits.shape[0]
         if logits.dim() != 2 or logits.shape[1] == 0:
             raise ValueError("cannot sample from an empty logits vector")     # sampler.rs:56-60
         if not (rows == len(configs) == len(histories) == len(draws)):
             raise ValueError("one config, history and draw per row of logits")
         history: List[int] = []
-        offsets = [0]
-        for config, tokens in zip(configs, histories):
-            if config.repetition_penalty > 1.0:
+        spans: List[int] = []
+        append_at: List[int] = []
+        for row, (config, tokens) in enumerate(zip(configs, histories)):
+            if config.repetition_penalty <= 1.0:
+                spans += [0, 0]
+                append_at.append(-1)
+            elif log is not None:
+                begin = log[0].begin[log[1][row]]
+                if begin + len(tokens) >= log[0].end[log[1][row]]:
+                    raise ValueError(f"row {row}: the log has no room for another token")
+                spans += [begin, begin + len(tokens)]
+                append_at.append(begin + len(tokens))
+            else:
+                spans += [len(history), len(history) + len(tokens)]
                 history.extend(int(t) for t in tokens)
-            offsets.append(len(history))
         # Rows that take the largest logit read no uniform number; when every row does, and nothing is
         # penalised, the operands of the step before serve again and nothing is uploaded.
         greedy = all(c.is_greedy() for c in configs)
-        made_from = (tuple(configs), None if greedy else tuple(draws), tuple(history), tuple(offsets))
+        made_from = (tuple(configs), None if greedy else tuple(draws), tuple(history), tuple(spans), log is not None)
         if self._last is not None and self._last[0] == made_from:
             floats, ints = self._last[1]
         else:
@@ -97,11 +129,16 @@ class Sampler:
                 [c.temperature for c in configs] + [c.top_p for c in configs]
                 + [c.repetition_penalty for c in configs] + [float(d) for d in draws],
                 dtype=torch.float32).view(4, rows)
-            ints = staging_for(self.device).upload([c.top_k for c in configs] + offsets + history)
+            ints = staging_for(self.device).upload([c.top_k for c in configs] + spans
+                                                   + (append_at if log is not None else history))
             self._last = (made_from, (floats, ints))
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
         # rows that the kernels can sample from a few candidates instead of passes over the whole row
         small_top_k = any(not c.is_greedy() and (0 < c.top_k <= 64 or (c.top_k == 0 and c.top_p < 1.0)) for c in configs)
-        self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2],
-                        ints[2 * rows + 1:], ints[rows:2 * rows + 1], floats[3], small_top_k=small_top_k)
+        if log is not None:
+            self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2], log[0].tokens,
+                            ints[rows:3 * rows], floats[3], small_top_k=small_top_k, append_at=ints[3 * rows:])
+        else:
+            self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2],
+                            ints[3 * rows:], ints[rows:3 * rows], floats[3], small_top_k=small_top_k)
         return out
