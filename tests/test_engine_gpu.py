@@ -254,28 +254,34 @@ def test_a_batch_of_forty_sequences(dtype, arch, head_dim, tmp_path):
     assert engine.cache.slots.n_held == 0
 
 
+@pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_generation_a_step_ahead_equals_generation_through_the_host(dtype, models, engines):
+def test_generation_a_step_ahead_equals_generation_through_the_host(dtype, graphs, models, engines):
     """The loop starts a step from the sampled tokens on the device before it has seen them. The same
     requests, sampled with a temperature, through a loop written here that brings every token to the
     host first, with the same uniform numbers: the same tokens, also where a request draws a stop token
     (and has been stepped once for nothing) while the others go on."""
     from xeno_rt_amd.engine import GenerateRequest, generate
+    from xeno_rt_amd.engine import Engine
     from xeno_rt_amd.sampling import Sampler, uniform
-    engine = engines("llama", dtype)
+    # with recorded decode steps, and with every step run directly (as models do whose parts cannot be recorded)
+    engine = engines("llama", dtype) if graphs else Engine.load(models["llama"][0], dtype=dtype, max_tokens=64 * 8,
+                                                                max_slots=3, graphs=False)
     vocab = engine.config.vocab_size
     prompts = [token_ids(vocab, n, seed=300 + n) for n in (9, 3, 14)]
-    options = dict(temperature=0.9, top_k=12, top_p=0.9, repetition_penalty=1.0)
+    # the second request has a repetition penalty: the loop keeps its tokens on the device, the loop below hands
+    # them to the sampler at every step
+    options = [dict(temperature=0.9, top_k=12, top_p=0.9, repetition_penalty=penalty) for penalty in (1.0, 1.3, 1.0)]
 
     def through_the_host(stops):
         sampler = Sampler(engine.ops, engine.device)
-        config = GenerateRequest([], **options).sampler_config()
+        configs = [GenerateRequest([], **o).sampler_config() for o in options]
         slots = [engine.alloc_slot() for _ in prompts]
         produced = [[] for _ in prompts]
         live = list(range(len(prompts)))
         logits = engine.step([(slots[i], prompts[i], [len(prompts[i]) - 1]) for i in live])
         while live:
-            tokens = sampler.sample(logits, [config] * len(live), [[]] * len(live),
+            tokens = sampler.sample(logits, [configs[i] for i in live], [prompts[i] + produced[i] for i in live],
                                     [uniform(70 + i, 0, len(produced[i])) for i in live])
             still = []
             for i, token in zip(live, tokens):
@@ -296,7 +302,7 @@ def test_generation_a_step_ahead_equals_generation_through_the_host(dtype, model
     stop = free[1][10]
     want = through_the_host((stop,))
     assert len(want[1]) <= 10 and max(len(tokens) for tokens in want) > len(want[1]) + 1
-    requests = [GenerateRequest(prompt, max_tokens=24, seed=70 + i, stop_ids=[stop], **options)
+    requests = [GenerateRequest(prompt, max_tokens=24, seed=70 + i, stop_ids=[stop], **options[i])
                 for i, prompt in enumerate(prompts)]
     got = generate(engine, requests)
     assert [result.tokens for result in got] == want

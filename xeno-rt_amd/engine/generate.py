@@ -161,7 +161,7 @@ def generate(engine, requests: Sequence[GenerateRequest], batch_size: Optional[i
             log, place = None, {}
             if any(seq.request.repetition_penalty > 1.0 for seq in running):
                 log = TokenLog(engine.device, [seq.history for seq in running],
-                               [seq.request.max_tokens + 1 for seq in running])
+                               [min(seq.request.max_tokens, context - len(seq.history)) + 1 for seq in running])
                 place = {seq.index: at for at, seq in enumerate(running)}
             while running:
                 drawn = sampler.launch(
