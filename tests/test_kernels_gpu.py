@@ -301,12 +301,17 @@ def test_qkv_prepare_of_many_tokens(ops, dtype, nh, nkv, hd, rope_dim):
 
 @pytest.mark.parametrize("nh,nkv,hd,rope_dim,k,tokens", [(32, 8, 128, 128, 4096, 8), (4, 2, 64, 64, 200, 9), (3, 3, 48, 32, 96, 16),
                                                           (2, 1, 256, 256, 72, 1), (5, 1, 16, 16, 64, 3), (4, 2, 64, 0, 128, 9),
-                                                          (4, 4, 80, 48, 264, 7)])
+                                                          (4, 4, 80, 48, 264, 7),
+                                                          # 17 to 64 tokens: the product is split along k, and the kernel that
+                                                          # adds the partial sums does the rest (the third: two kernels)
+                                                          (32, 8, 128, 128, 4096, 40), (4, 2, 64, 64, 256, 17),
+                                                          (3, 3, 48, 32, 192, 33), (4, 2, 64, 0, 128, 64), (6, 2, 96, 96, 320, 64)])
 def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens):
     """The projection of a short step with the rotation and the cache write in its epilogue, against the two
     kernels one after the other; without a norm before it and with one."""
-    positions = i32([0, 1, 63, 64, 65, 127, 128, 500, 1000, 2, 3, 4, 5, 6, 7, 8][:tokens])
-    slots = i32([0, 0, 0, 0, 1, 1, -1, 1, 0, 1, 1, 1, 1, 1, 1, 1][:tokens])                # one token is padding
+    positions = ([0, 1, 63, 64, 65, 127, 128, 500, 1000, 2, 3, 4, 5, 6, 7, 8] + list(range(9, 57)))[:tokens]
+    slots = ([0, 0, 0, 0, 1, 1, -1, 1, 0, 1, 1, 1, 1, 1, 1, 1] + [0] * 48)[:tokens]                # one token is padding
+    positions, slots = i32(positions), i32(slots)
     width = (nh + 2 * nkv) * hd
     a = rand(tokens, k, dtype=torch.bfloat16, seed=hd)
     w = rand(width, k, dtype=torch.bfloat16, seed=k, scale=1.0 / math.sqrt(k))
@@ -318,7 +323,8 @@ def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens):
     # the norm before the projection, handed over by the product before it
     x = rand(tokens, k, seed=3, scale=2.0)
     gain = (rand(k, seed=4) + 1.0).to(torch.bfloat16)
-    scaled = ops.linear(rand(tokens, 64, dtype=torch.bfloat16, seed=5), rand(k, 64, dtype=torch.bfloat16, seed=6), x,
+    inner = 64 if tokens <= 16 else 256
+    scaled = ops.linear(rand(tokens, inner, dtype=torch.bfloat16, seed=5), rand(k, inner, dtype=torch.bfloat16, seed=6), x,
                         accumulate=True, then_norm=(gain, 1e-4))
     assert scaled is not None
     for rows in (a, scaled):

@@ -20,6 +20,7 @@
 #include <cstdlib>
 #include "common.h"
 #include "xrt_hip.h"
+#include "gemm_skinny.h"
 
 namespace {
 
@@ -621,13 +622,86 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restri
     }
 }
 
+// The second kernel of a q/k/v projection split along k (no head norms, the rotation over the whole head):
+// a thread adds up the two outputs that the rotation pairs (dims d and d + head_dim / 2 of one head), for
+// NORM 1 scales them by the row's 1 / rms, rotates q and k by the token's position, writes bfloat16 q/k/v and
+// puts k and v into the cache. One thread per (token, head, d).
+template <int NORM>
+__global__ void __launch_bounds__(256) split_reduce_qkv_kernel(const float* __restrict__ parts, int splits, int M, int N,
+                                                                bf16* __restrict__ qkv, const xrt_linear_norm norm,
+                                                                const QkvAfter after) {
+    __shared__ float wave_sums[256 / XRT_WAVE];
+    const int half = after.head_dim / 2;
+    const long per_token = (long)(N / 2);
+    const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool inside = index < (long)M * per_token;
+    const long m = inside ? index / per_token : M - 1;
+    const int pair = inside ? (int)(index % per_token) : 0;
+    const int head = pair / half, d = pair % half;
+    const long n = (long)head * after.head_dim + d;
+    float mine = 0.f;
+    if constexpr (NORM == 1) {
+        // a block lies within one token if a token's pairs are a multiple of 256: then its threads share the work
+        if (per_token % 256 == 0)
+            for (int t = threadIdx.x; t < norm.tiles_in; t += 256) mine += norm.squares_in[(long)t * XRT_SQUARES_STRIDE + m];
+        else
+            for (int t = 0; t < norm.tiles_in; ++t) mine += norm.squares_in[(long)t * XRT_SQUARES_STRIDE + m];
+    }
+    float lower = 0.f, upper = 0.f;
+    for (int p = 0; p < splits; ++p) {
+        const float* part = parts + ((long)p * M + m) * N;
+        lower += part[n];
+        upper += part[n + half];
+    }
+    const int pos = after.positions[m];
+    const bool is_q = head < after.n_heads, is_v = head >= after.n_heads + after.n_kv_heads;
+    float sine = 0.f, cosine = 1.f;
+    if (after.rope_theta != nullptr && !is_v) sincosf((float)pos * after.rope_scale / after.rope_theta[d], &sine, &cosine);
+    if constexpr (NORM == 1) {
+        float total = mine;
+        if (per_token % 256 == 0) {
+            mine = wave_sum(mine);
+            if (threadIdx.x % XRT_WAVE == 0) wave_sums[threadIdx.x / XRT_WAVE] = mine;
+            __syncthreads();
+            total = 0.f;
+            for (int w = 0; w < 256 / XRT_WAVE; ++w) total += wave_sums[w];
+        }
+        const float by = 1.0f / sqrtf(total / (float)norm.width_in + norm.eps);
+        lower *= by;
+        upper *= by;
+    }
+    if (!inside) return;
+    // rounded as the product alone would have stored them, then rotated: the same values as from two kernels
+    lower = to_float(from_float<bf16>(lower));
+    upper = to_float(from_float<bf16>(upper));
+    const bf16 out_lower = from_float<bf16>(lower * cosine - upper * sine);
+    const bf16 out_upper = from_float<bf16>(lower * sine + upper * cosine);
+    qkv[m * N + n] = out_lower;
+    qkv[m * N + n + half] = out_upper;
+    if (is_q || after.k_cache == nullptr) return;
+    const int kv_head = head - after.n_heads - (is_v ? after.n_kv_heads : 0);
+    const long base = cache_block_base(after.block_table, after.table_stride, after.n_blocks, after.slots[m], pos,
+                                       after.n_kv_heads, kv_head, after.head_dim);
+    if (base < 0) return;
+    const int within = pos % XRT_BLOCK_TOKENS;
+    if (is_v) {
+        after.v_cache[base + (long)d * XRT_BLOCK_TOKENS + within] = out_lower;
+        after.v_cache[base + (long)(d + half) * XRT_BLOCK_TOKENS + within] = out_upper;
+    } else {
+        after.k_cache[base + (long)within * after.head_dim + d] = out_lower;
+        after.k_cache[base + (long)within * after.head_dim + d + half] = out_upper;
+    }
+}
+
 template <typename TO>
 int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, float* workspace,
-                 const xrt_linear_norm* norm, hipStream_t s) {
+                 const xrt_linear_norm* norm, const QkvAfter* after, hipStream_t s) {
     const SplitPlan plan = split_plan(M, N, K, mode);
     const bool scaled = norm && norm->squares_in, emits = norm && norm->squares_out;
     XRT_REQUIRE(!norm || M <= SPLIT_BM, "linear (mfma): the norm around a product takes at most %d rows here", SPLIT_BM);
     const RowScale scale = scaled ? RowScale{norm->squares_in, norm->tiles_in, norm->width_in, norm->eps} : RowScale{};
+    XRT_REQUIRE(!after || (plan.splits > 1 && mode == MODE_STORE && sizeof(TO) == 2),
+                "linear (mfma): only a bfloat16 product split along k does what follows a q/k/v projection");
     if (M <= SPLIT_BM && plan.splits == 1) {                   // tiles enough: each applies the epilogue itself
         XRT_REQUIRE(!emits, "linear (mfma): only a product split along k writes what the norm after it needs");
         if (mode == MODE_STORE) return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s, 1, 0, scale);
@@ -648,6 +722,15 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
     const xrt_linear_norm none = {};
     const xrt_linear_norm& around = norm ? *norm : none;
     XRT_REQUIRE(!(scaled && emits), "linear (mfma): one product does one half of a norm");
+    if (after != nullptr) {
+        if constexpr (sizeof(TO) == 2) {
+            const unsigned pair_blocks = (unsigned)(((long)M * (N / 2) + 255) / 256);
+            if (scaled) split_reduce_qkv_kernel<1><<<pair_blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around, *after);
+            else split_reduce_qkv_kernel<0><<<pair_blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around, *after);
+            XRT_LAUNCH_CHECK("linear (split reduce, q/k/v)");
+        }
+        return 0;
+    }
 #define XRT_REDUCE(MODE_, NORM_) split_reduce_kernel<MODE_, TO, NORM_><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around)
     if (mode == MODE_STORE) { if (scaled) XRT_REDUCE(MODE_STORE, 1); else XRT_REDUCE(MODE_STORE, 0); }
     else if (mode == MODE_GATED) { if (scaled) XRT_REDUCE(MODE_GATED, 1); else XRT_REDUCE(MODE_GATED, 0); }
@@ -698,6 +781,20 @@ bool xrt_linear_split_takes_norm(const void* a, const void* w, int M, int N, int
 
 int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                      float* workspace, const xrt_linear_norm* norm, hipStream_t s) {
-    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, workspace, norm, s);
-    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, workspace, norm, s);
+    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, workspace, norm, nullptr, s);
+    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, workspace, norm, nullptr, s);
+}
+
+// Whether the q/k/v projection of a step of 17 to 64 tokens can also do what follows it (rotation over the
+// whole head or none, no head norms, cache write) in the kernel that adds up its partial sums.
+bool xrt_linear_split_takes_qkv(const void* a, const void* w, int M, int N, int K, const QkvAfter& after, long* workspace_floats) {
+    *workspace_floats = 0;
+    if (M > SPLIT_BM || after.head_dim % 2 != 0 || N != (after.n_heads + 2 * after.n_kv_heads) * after.head_dim) return false;
+    if (after.rope_theta != nullptr && after.rope_dim != after.head_dim) return false;
+    return xrt_linear_split_takes(a, w, M, N, K, MODE_STORE, workspace_floats) && *workspace_floats > 0;
+}
+
+int xrt_linear_split_qkv(const void* a, const void* w, void* qkv, int M, int N, int K, float* workspace,
+                         const xrt_linear_norm* norm, const QkvAfter& after, hipStream_t s) {
+    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)qkv, M, N, K, MODE_STORE, workspace, norm, &after, s);
 }

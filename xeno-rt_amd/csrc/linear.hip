@@ -11,6 +11,9 @@ int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int 
 
 bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats);
 bool xrt_linear_split_takes_norm(const void* a, const void* w, int M, int N, int K, int mode);
+bool xrt_linear_split_takes_qkv(const void* a, const void* w, int M, int N, int K, const QkvAfter& after, long* workspace_floats);
+int xrt_linear_split_qkv(const void* a, const void* w, void* qkv, int M, int N, int K, float* workspace,
+                         const xrt_linear_norm* norm, const QkvAfter& after, hipStream_t s);
 int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
                      float* workspace, const xrt_linear_norm* norm, hipStream_t s);
 
@@ -109,6 +112,14 @@ extern "C" int xrt_linear_qkv(const void* a, const void* w, int dtype, void* qkv
         (k_cache == nullptr || (block_table && slots && table_stride > 0 && n_blocks > 0)) &&
         (rope_theta == nullptr || rope_dim > 0))
         return xrt_linear_skinny(a, w, qkv, XRT_BF16, M, N, K, 0, norm, &after, (hipStream_t)stream);
+    // 17 to 64 tokens, the product split along k: the kernel that adds the partial sums does the rest
+    long need = 0;
+    if (dtype == XRT_BF16 && a && w && qkv && M > 0 && K > 0 && !q_norm && !k_norm && positions &&
+        (k_cache == nullptr) == (v_cache == nullptr) &&
+        (k_cache == nullptr || (block_table && slots && table_stride > 0 && n_blocks > 0)) &&
+        (!norm || (norm->squares_in && !norm->squares_out && xrt_linear_split_takes_norm(a, w, M, N, K, 0))) &&
+        xrt_linear_split_takes_qkv(a, w, M, N, K, after, &need) && workspace != nullptr && workspace_floats >= need)
+        return xrt_linear_split_qkv(a, w, qkv, M, N, K, workspace, norm, after, (hipStream_t)stream);
     const int status = norm ? xrt_linear_normed(a, w, dtype, qkv, dtype, M, N, K, 0, norm, workspace, workspace_floats, stream)
                             : xrt_linear(a, w, dtype, qkv, dtype, M, N, K, 0, workspace, workspace_floats, stream);
     if (status != 0) return status;
