@@ -19,9 +19,9 @@ from ..cache import BLOCK_TOKENS, CacheError, CacheFull, SequenceCache
 from ..config import architecture, load_config
 from ..models import DecoderModel, ModelSpec
 from ..parts.base import Runtime
-from ..weights import check_names, load_tensors, random_tensors
+from ..weights import load_tensors
 from ..staging import staging_for
-from .batch import StepBatch, build_batch
+from .batch import build_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
            "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32}

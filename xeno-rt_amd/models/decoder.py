@@ -7,7 +7,7 @@ cache entry of an earlier call instead of owning one.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional
 
 import torch

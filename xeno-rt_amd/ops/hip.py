@@ -7,7 +7,6 @@ kernel could read outside of it.
 from __future__ import annotations
 
 import ctypes
-import os
 from dataclasses import dataclass
 from typing import Optional, Tuple
 
