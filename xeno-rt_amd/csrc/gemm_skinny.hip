@@ -165,24 +165,20 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
             }
         }
     }
+    int early_pos = 0, early_slot = -1, early_block = -1;
+    float early_theta = 1.f;
     // (what the accumulating epilogue reads is asked for behind the first loads of w: those have the longer way)
     auto ask_early = [&]() {
         if constexpr (QKV) {
+            // only asked for here: a wavefront that waited for them now would have one step of w in flight meanwhile
             const int token = min(r, M - 1);
             if (rotates && wave < 4) {                          // the lane's four angles, one per wavefront; read by wavefront 0
-                const float angle = (float)after.positions[token] * after.rope_scale / after.rope_theta[lower_dim + (c % 2) * 4 + wave];
-                sincosf(angle, &early_sin[lane][wave], &early_cos[lane][wave]);     // lanes c and c ^ 2 hold the two halves of a pair
+                early_pos = after.positions[token];
+                early_theta = after.rope_theta[lower_dim + (c % 2) * 4 + wave];
             }
             if (wave == 4 && c == 0) {
-                const int pos = after.positions[token];
-                long base = -1;
-                if (after.k_cache && head >= after.n_heads) {
-                    const int kv_head = (head - after.n_heads) % after.n_kv_heads;
-                    base = cache_block_base(after.block_table, after.table_stride, after.n_blocks, after.slots[token],
-                                            pos, after.n_kv_heads, kv_head, after.head_dim);
-                }
-                early_base[r] = base;
-                early_within[r] = pos % XRT_BLOCK_TOKENS;
+                early_pos = after.positions[token];
+                if (after.k_cache && head >= after.n_heads) early_slot = after.slots[token];
             }
         }
         if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
@@ -196,6 +192,33 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                                                                    : (unsigned)min(n0 + 2 * lane, (long)N - 2) * 2u;
                     load_dword_to_lds(norm.gain, at, lds_address(&early_gain[0]));
                 }
+            }
+        }
+    };
+    // After the first step of w has been multiplied, what was asked for above has arrived as well (loads come
+    // back in order): sine and cosine are worked out, and the cache block's number is asked for, while the
+    // next steps are in flight.
+    auto use_early = [&]() {
+        if constexpr (QKV) {
+            if (rotates && wave < 4) {
+                const float angle = (float)early_pos * after.rope_scale / early_theta;
+                sincosf(angle, &early_sin[lane][wave], &early_cos[lane][wave]);     // lanes c and c ^ 2 hold the two halves of a pair
+            }
+            if (wave == 4 && c == 0 && early_slot >= 0)
+                early_block = after.block_table[(long)early_slot * after.table_stride + early_pos / XRT_BLOCK_TOKENS];
+        }
+    };
+    // when the stream of w has run through: where the lane's token lies in the cache (-1: nowhere)
+    auto place_in_cache = [&]() {
+        if constexpr (QKV) {
+            if (wave == 4 && c == 0) {
+                long base = -1;
+                if (early_block >= 0 && early_block < after.n_blocks) {
+                    const int kv_head = (head - after.n_heads) % after.n_kv_heads;
+                    base = ((long)early_block * after.n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * after.head_dim;
+                }
+                early_base[r] = base;
+                early_within[r] = early_pos % XRT_BLOCK_TOKENS;
             }
         }
     };
@@ -234,6 +257,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
             load_x(x_b, k_begin + (i + 1) * KSTEP);
             load_w(w_b, k_begin + (i + 1) * KSTEP);
             multiply(w_a, x_a);
+            if constexpr (QKV) if (i == 0) use_early();
             load_x(x_a, k_begin + (i + 2) * KSTEP);
             load_w(w_a, k_begin + (i + 2) * KSTEP);
             multiply(w_b, x_b);
@@ -246,8 +270,10 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
         } else {
             multiply(w_a, x_a);
         }
+        if constexpr (QKV) if (full <= 2) use_early();         // the loop above did not run
     } else {
         ask_early();
+        use_early();
     }
     // what is left of K when it is no multiple of the step: one guarded step, in the wavefront that owns it
     const int tail_begin = k_begin + full * KSTEP;
@@ -268,6 +294,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
             }
         }
     }
+    place_in_cache();
     add_squares();
     floatx4 acc[WT][MT];
 #pragma unroll
