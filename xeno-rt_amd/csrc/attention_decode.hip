@@ -281,16 +281,29 @@ __global__ void __launch_bounds__(HD) attention_decode_merge_kernel(
 // (each from the four wavefronts of a workgroup) per (token, head).
 struct Cut { int chunk_blocks, n_parts; };
 
-Cut cut_for(int tokens, int n_kv_heads, int q_tiles, int max_context) {
+Cut cut_for(int tokens, int n_kv_heads, int q_tiles, int max_context, int head_dim) {
     const int max_blocks = (max_context + XRT_BLOCK_TOKENS - 1) / XRT_BLOCK_TOKENS;
-    // Two workgroups of four wavefronts fit a compute unit. With that many (token, key/value head) pairs a
-    // workgroup takes all keys of its pair: nothing is left to merge, and the merge kernel is not launched.
-    if ((long)tokens * n_kv_heads * q_tiles >= 512) return Cut{(max_blocks + WAVES - 1) / WAVES, 1};
-    // else: enough wavefronts to fill the chip, but chunks as long as that allows
-    long chunk_blocks = ((long)tokens * n_kv_heads * q_tiles * max_blocks) / 4096;
-    chunk_blocks = chunk_blocks < 1 ? 1 : (chunk_blocks > 16 ? 16 : chunk_blocks);
-    const int n_chunks = (int)((max_blocks + chunk_blocks - 1) / chunk_blocks);
-    return Cut{(int)chunk_blocks, (n_chunks + WAVES - 1) / WAVES};
+    // How long the kernel takes is set by the compute unit with the most to do: workgroups are dealt out to
+    // the 256 compute units in turn, and a compute unit works off its share at its own pace (two workgroups
+    // at a time are no faster than one after the other). Measured at head size 128: 6.3 us for a block of 64
+    // keys per wavefront, 0.7 us per workgroup, about 5 us for the merge kernel. So the cut is chosen for
+    // the fewest blocks per compute unit: 384 workgroups of 16 blocks (two on every second compute unit) are
+    // slower than 768 of 8. The longer chunk wins among equals (less to merge); with one workgroup per (token,
+    // key/value head) pair nothing is left to merge and the merge kernel is not launched.
+    const long pairs = (long)tokens * n_kv_heads * q_tiles;
+    const long block_ns = 6300L * head_dim / 128, group_ns = 700, merge_ns = 5000;
+    const int longest = (max_blocks + WAVES - 1) / WAVES;
+    long best_ns = -1;
+    Cut best{longest, 1};
+    for (int chunk_blocks = longest; chunk_blocks >= 1; --chunk_blocks) {
+        const int n_chunks = (max_blocks + chunk_blocks - 1) / chunk_blocks;
+        const int n_parts = (n_chunks + WAVES - 1) / WAVES;
+        if ((long)(n_parts - 1) * WAVES * chunk_blocks >= max_blocks) continue;         // a part without keys: a shorter chunk does the same
+        const long per_unit = (pairs * n_parts + 255) / 256;
+        const long ns = per_unit * (chunk_blocks * block_ns + group_ns) + (n_parts > 1 ? merge_ns : 0);
+        if (best_ns < 0 || ns < best_ns) { best_ns = ns; best = Cut{chunk_blocks, n_parts}; }
+    }
+    return best;
 }
 
 template <int HD>
@@ -299,7 +312,7 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
            float scale, int max_context, float* workspace, long workspace_floats, hipStream_t s) {
     const int group = n_heads / n_kv_heads;
     const int q_tiles = (group + 15) / 16;
-    const Cut cut = cut_for(tokens, n_kv_heads, q_tiles, max_context);
+    const Cut cut = cut_for(tokens, n_kv_heads, q_tiles, max_context, HD);
     const long need = (long)tokens * n_heads * cut.n_parts * (HD + 2);
     XRT_REQUIRE(workspace != nullptr && workspace_floats >= need,
                 "attention (decode): workspace of %ld floats given, %ld needed", workspace_floats, need);

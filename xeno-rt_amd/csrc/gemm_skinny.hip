@@ -53,8 +53,10 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 // registers for the stream.
 template <int MT, int RT, int MODE, typename TO, int EXTRA = 0>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skinny_kernel(
-    const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
+    const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K, int rows,
     const LinearNorm norm, const QkvAfter after) {
+    // rows: rows of w that a workgroup's tile holds, 16 or fewer (with RT == 1): the host picks them so that
+    // the workgroups divide evenly among the compute units. Lanes beyond read the tile's last row again.
     constexpr bool AROUND = EXTRA != 0, QKV = EXTRA == 2;
     static_assert(!AROUND || (MT == 1 && RT == 1), "the norm around a product: one tile of x, one of w per wavefront");
     static_assert(!QKV || (MODE == MODE_STORE && sizeof(TO) == 2), "after a q/k/v projection: a bfloat16 store");
@@ -74,19 +76,21 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 
     const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
     const int r = lane % 16, c = lane / 16;
-    const long n0 = (long)blockIdx.x * (16 * RT);
+    const long n0 = (long)blockIdx.x * (RT == 1 ? rows : 16 * RT);
     // after a q/k/v projection: the tile's head, and the dims of the head its rows 0..7 and 8..15 make
     int head = 0, lower_dim = 0, upper_dim = 8;
     bool rotates = false;
     if constexpr (QKV) {
-        const int tiles_per_head = after.head_dim / 16;
+        // a tile: rows / 2 dims and the rows / 2 that the rotation pairs them with (beyond rope_dim and in
+        // value heads: the rows / 2 dims that follow), in lanes r = 0.. and r = 8..
+        const int tiles_per_head = after.head_dim / rows;
         head = blockIdx.x / tiles_per_head;
         const int s = blockIdx.x % tiles_per_head;
         const bool is_value = head >= after.n_heads + after.n_kv_heads;
-        const int rotated_tiles = (after.rope_theta && !is_value) ? after.rope_dim / 16 : 0;
+        const int rotated_tiles = (after.rope_theta && !is_value) ? after.rope_dim / rows : 0;
         rotates = s < rotated_tiles;
-        lower_dim = rotates ? 8 * s : 16 * s;
-        upper_dim = rotates ? after.rope_dim / 2 + 8 * s : 16 * s + 8;
+        lower_dim = rotates ? rows / 2 * s : rows * s;
+        upper_dim = rotates ? after.rope_dim / 2 + rows / 2 * s : rows * s + rows / 2;
     }
 
     const int steps = (K + KSTEP - 1) / KSTEP;
@@ -110,8 +114,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 #pragma unroll
     for (int t = 0; t < WT; ++t) {
         const int rt = t % RT, half = t / RT;                   // half 1: the "up" rows of a gated product
-        long n = min(n0 + rt * 16 + r, (long)N - 1);
-        if constexpr (QKV) n = (long)head * after.head_dim + (r < 8 ? lower_dim + r : upper_dim + r - 8);
+        long n = min(n0 + rt * 16 + min(r, rows - 1), (long)N - 1);
+        if constexpr (QKV) n = (long)head * after.head_dim + (r < 8 ? lower_dim + min(r, rows / 2 - 1) : upper_dim + min(r - 8, rows / 2 - 1));
         w_ptr[t] = w + (n + (long)half * N) * K + c * 8;
     }
     const bf16* x_ptr[MT];
@@ -174,7 +178,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
             const int token = min(r, M - 1);
             if (rotates && wave < 4) {                          // the lane's four angles, one per wavefront; read by wavefront 0
                 early_pos = after.positions[token];
-                early_theta = after.rope_theta[lower_dim + (c % 2) * 4 + wave];
+                early_theta = after.rope_theta[min(lower_dim + (c % 2) * 4 + wave, after.rope_dim / 2 - 1)];   // (lanes beyond a tile of 8 rows: unused)
             }
             if (wave == 4 && c == 0) {
                 early_pos = after.positions[token];
@@ -361,7 +365,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                     }
                     packed.e[i] = from_float<bf16>(value);
                 }
-                if (mm < M) {
+                if (mm < M && (c % 2) * 4 < rows / 2) {          // (rows / 2 is 8 or 4: all four of a lane's dims or none)
                     const int dim = (c < 2 ? lower_dim : upper_dim) + (c % 2) * 4;
                     *reinterpret_cast<Four*>((bf16*)out + (long)mm * N + (long)head * after.head_dim + dim) = packed;
                     const long base = early_base[r];
@@ -392,7 +396,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
             if (mm < M && !written) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if (nn + i >= N) continue;
+                    if (nn + i >= N || c * 4 + i >= rows) continue;
                     TO* dst = out + (long)mm * N + nn + i;
                     if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(g[i]);
                     if constexpr (MODE == MODE_ACCUMULATE) {
@@ -430,23 +434,36 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 template <int MT, int RT, typename TO>
 int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
                 const QkvAfter* after, hipStream_t s) {
-    const unsigned grid = (unsigned)((N + 16 * RT - 1) / (16 * RT));
+    // Workgroups are dealt out to the 256 compute units in turn, and the kernel takes about as long as the
+    // compute unit with the most of them: 384 tiles of 16 rows take as long as 512. So, with as many rounds
+    // over the compute units as tiles of 16 rows make, a tile gets the fewest rows (8 at least) that still fit
+    // those rounds: 512 tiles of 12 rows instead of 384 of 16. (More rounds of still smaller tiles lose to what
+    // every workgroup costs, about as much as three rows.) Accumulating products keep 16 (what they hand to a
+    // norm is laid out by tiles of 16 columns), and so does the tile that the rotation after a q/k/v
+    // projection pairs (768 tiles of 8 rows were slower than 384 of 16).
+    int rows = 16;
+    if (RT == 1 && mode != MODE_ACCUMULATE && !after) {
+        const long rounds = ((N + 15) / 16 + 255) / 256;
+        rows = (int)((N + 256 * rounds - 1) / (256 * rounds));
+        rows = rows < 8 ? 8 : rows;
+    }
+    const unsigned grid = (unsigned)(RT == 1 ? (N + rows - 1) / rows : (N + 16 * RT - 1) / (16 * RT));
     const dim3 block(WAVES * XRT_WAVE);
     const QkvAfter none = {};
     if constexpr (MT == 1 && RT == 1) {
         if (after) {
             if constexpr (sizeof(TO) == 2) {
-                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, *after);
+                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, *after);
                 XRT_LAUNCH_CHECK("linear (skinny, q/k/v)");
                 return 0;
             }
         } else if (norm.squares_in || norm.squares_out) {
             if (mode == MODE_STORE)
-                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
+                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
             else if (mode == MODE_ACCUMULATE)
-                gemm_skinny_kernel<1, 1, MODE_ACCUMULATE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
+                gemm_skinny_kernel<1, 1, MODE_ACCUMULATE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
             else
-                gemm_skinny_kernel<1, 1, MODE_GATED, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
+                gemm_skinny_kernel<1, 1, MODE_GATED, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
             XRT_LAUNCH_CHECK("linear (skinny, with norm)");
             return 0;
         }
@@ -456,11 +473,11 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
         return 1;
     }
     if (mode == MODE_STORE)
-        gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
+        gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
     else if (mode == MODE_ACCUMULATE)
-        gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
+        gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
     else if constexpr (RT == 1)
-        gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, norm, none);
+        gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
     else {
         xrt_set_error("linear (skinny): a gated product takes one row tile per wavefront");
         return 1;
