@@ -174,10 +174,12 @@ def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n):
     scaled = ops.linear(a, w, x, accumulate=True, then_norm=(gain, eps))
     assert scaled is not None and scaled.shape == (m, hidden)
     assert rel(x.cpu(), fresh) < 1e-5
-    tiles = (hidden + 15) // 16
-    padded = torch.zeros(m, tiles * 16, dtype=torch.float64)
+    tiles = scaled.squares.shape[0]                 # the product cuts its columns into tiles of 16 or fewer, all alike
+    width = -(-hidden // tiles)
+    assert 8 <= width <= 16 and tiles == -(-hidden // width)
+    padded = torch.zeros(m, tiles * width, dtype=torch.float64)
     padded[:, :hidden] = x.double().cpu() ** 2
-    assert rel(scaled.squares[:, :m].t().cpu(), padded.reshape(m, tiles, 16).sum(-1)) < 1e-6
+    assert rel(scaled.squares[:, :m].t().cpu(), padded.reshape(m, tiles, width).sum(-1)) < 1e-6
     assert rel(scaled.values.cpu(), x.double().cpu() * gain.double().cpu()) < ULP["bfloat16"]
 
     want = normed @ v.double().cpu().t()

@@ -19,7 +19,7 @@
 //
 // Around an RMSNorm between two products (x += a w^T; y = rmsnorm(x) * gain; z = y v^T) a step of
 // up to 16 rows needs no kernel for the norm: the accumulating product also writes
-// bfloat16(x * gain) and, for every tile of 16 columns, each row's sum of squares; the product
+// bfloat16(x * gain) and, for every tile of columns, each row's sum of squares; the product
 // after it takes those as its activations and multiplies its rows by 1 / sqrt(sum / width + eps).
 // The sums are added in a fixed order (tiles in eighths by wavefront, then wavefront by wavefront).
 //
@@ -385,7 +385,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
             float fresh[4] = {0.f, 0.f, 0.f, 0.f};              // what out holds now, 0 outside of it
             bool written = false;
             if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
-                if (out_ahead && mm < M && nn < N) {            // the four values in one piece, as they came
+                if (out_ahead && mm < M && nn < N && c * 4 < rows) {   // the four values in one piece, as they came (rows is a multiple of 4 here)
                     const floatx4 before = early_out[lane];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) fresh[i] = before[i] + g[i];
@@ -396,7 +396,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
             if (mm < M && !written) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if (nn + i >= N || c * 4 + i >= rows) continue;
+                    if (nn + i >= N || c * 4 + i >= rows) continue;        // (fresh stays 0: it counts for nothing below)
                     TO* dst = out + (long)mm * N + nn + i;
                     if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(g[i]);
                     if constexpr (MODE == MODE_ACCUMULATE) {
@@ -413,7 +413,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                     sum += __shfl_xor(sum, 32);
                     if (mm < M) {
                         if (c == 0) norm.squares_out[(long)blockIdx.x * XRT_SQUARES_STRIDE + mm] = sum;
-                        if (nn < N) {                           // N is a multiple of 8: all four or none
+                        if (nn < N && c * 4 < rows) {           // N is a multiple of 8 and rows one of 4: all four or none
                             struct alignas(8) Four { bf16 e[4]; } scaled;
 #pragma unroll
                             for (int i = 0; i < 4; ++i) {
@@ -431,22 +431,25 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     }
 }
 
+// Rows of w in a workgroup's tile (one tile of 16 or fewer per wavefront).
+// Workgroups are dealt out to the 256 compute units in turn, and the kernel takes about as long as the
+// compute unit with the most of them: 384 tiles of 16 rows take as long as 512. So, with as many rounds
+// over the compute units as tiles of 16 rows make, a tile gets the fewest rows (8 at least) that still fit
+// those rounds: 512 tiles of 12 rows instead of 384 of 16. (More rounds of still smaller tiles lose to what
+// every workgroup costs, about as much as three rows.) Accumulating products take a multiple of 4 (their
+// epilogue moves four values at a time). The tile that the rotation after a q/k/v projection pairs stays at
+// 16 (768 tiles of 8 rows were slower than 384 of 16).
+int balanced_rows(int N, int mode) {
+    const long rounds = ((N + 15) / 16 + 255) / 256;
+    int rows = (int)((N + 256 * rounds - 1) / (256 * rounds));
+    if (mode == MODE_ACCUMULATE) rows = (rows + 3) / 4 * 4;
+    return rows < 8 ? 8 : (rows > 16 ? 16 : rows);
+}
+
 template <int MT, int RT, typename TO>
 int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
                 const QkvAfter* after, hipStream_t s) {
-    // Workgroups are dealt out to the 256 compute units in turn, and the kernel takes about as long as the
-    // compute unit with the most of them: 384 tiles of 16 rows take as long as 512. So, with as many rounds
-    // over the compute units as tiles of 16 rows make, a tile gets the fewest rows (8 at least) that still fit
-    // those rounds: 512 tiles of 12 rows instead of 384 of 16. (More rounds of still smaller tiles lose to what
-    // every workgroup costs, about as much as three rows.) Accumulating products keep 16 (what they hand to a
-    // norm is laid out by tiles of 16 columns), and so does the tile that the rotation after a q/k/v
-    // projection pairs (768 tiles of 8 rows were slower than 384 of 16).
-    int rows = 16;
-    if (RT == 1 && mode != MODE_ACCUMULATE && !after) {
-        const long rounds = ((N + 15) / 16 + 255) / 256;
-        rows = (int)((N + 256 * rounds - 1) / (256 * rounds));
-        rows = rows < 8 ? 8 : rows;
-    }
+    const int rows = RT == 1 && !after ? balanced_rows(N, mode) : 16;
     const unsigned grid = (unsigned)(RT == 1 ? (N + rows - 1) / rows : (N + 16 * RT - 1) / (16 * RT));
     const dim3 block(WAVES * XRT_WAVE);
     const QkvAfter none = {};
@@ -515,6 +518,9 @@ bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K) {
 
 // The norm around a product needs one tile of x.
 bool xrt_linear_skinny_takes_norm(int M) { return M <= 16; }
+
+// Tiles of columns for which an accumulating product of N columns writes sums of squares.
+int xrt_linear_skinny_norm_tiles(int N) { const int rows = balanced_rows(N, MODE_ACCUMULATE); return (N + rows - 1) / rows; }
 
 // So does what follows a q/k/v projection; and the rotation must pair whole groups of 8 dims.
 bool xrt_linear_skinny_takes_qkv(int M, int N, const QkvAfter& after) {

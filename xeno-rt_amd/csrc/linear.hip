@@ -65,6 +65,14 @@ extern "C" int xrt_linear_takes_norm(const void* a, const void* w, int dtype, in
     return xrt_linear_split_takes_norm(a, w, M, N, K, mode) ? 1 : 0;
 }
 
+// Tiles of columns for which an accumulating product that xrt_linear_takes_norm accepts writes sums of
+// squares: the rows of the table that the caller provides (and hands to the product after the norm).
+extern "C" int xrt_linear_norm_tiles(const void* a, const void* w, int dtype, int M, int N, int K) {
+    if (dtype == XRT_BF16 && xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_norm(M))
+        return xrt_linear_skinny_norm_tiles(N);
+    return (N + 15) / 16;
+}
+
 extern "C" int xrt_linear_normed(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N,
                                  int K, int mode, const xrt_linear_norm* norm, float* workspace,
                                  long workspace_floats, void* stream) {
@@ -74,7 +82,7 @@ extern "C" int xrt_linear_normed(const void* a, const void* w, int dtype, void* 
     XRT_REQUIRE(out_dtype == XRT_F32 || out_dtype == XRT_BF16, "linear with norm: unknown output dtype %d", out_dtype);
     XRT_REQUIRE(mode != 1 || out_dtype == XRT_F32, "linear with norm: accumulation needs a float32 output");
     if (norm->squares_in)
-        XRT_REQUIRE(norm->width_in == K && norm->tiles_in == (K + 15) / 16,
+        XRT_REQUIRE(norm->width_in == K && norm->tiles_in >= (K + 15) / 16 && norm->tiles_in <= (K + 7) / 8,     // tiles of 8 to 16 columns
                     "linear with norm: sums of squares of %d tiles over %d columns for a of %d columns",
                     norm->tiles_in, norm->width_in, K);
     const bool emits = norm->squares_out || norm->scaled_out || norm->gain;

@@ -31,7 +31,7 @@ long xrt_linear_workspace(const void* a, const void* w, int dtype, int M, int N,
 
 // An RMSNorm between two products, x += a w^T; y = rmsnorm(x) * gain; z = y v^T, without a kernel of
 // its own. The first product (mode 1) also writes scaled_out[m, n] = bfloat16(x[m, n] * gain[n]) and
-// squares_out[t * XRT_SQUARES_STRIDE + m], the sum of x[m, n]^2 over the 16 columns n of tile t. The
+// squares_out[t * XRT_SQUARES_STRIDE + m], the sum of x[m, n]^2 over the columns n of tile t (xrt_linear_norm_tiles of them, 16 columns or fewer each). The
 // second takes scaled_out as its a, squares_in (tiles_in = ceil(width_in / 16) tiles) and multiplies its
 // rows by 1 / sqrt(sum of squares / width_in + eps) before its epilogue. A half left all zero is not done.
 // xrt_linear_takes_norm says whether an accumulating product can write these (bfloat16 operands, up to 64 rows,
@@ -43,6 +43,7 @@ typedef struct xrt_linear_norm {
     void* scaled_out; const void* gain; int gain_dtype; float* squares_out;
 } xrt_linear_norm;
 int xrt_linear_takes_norm(const void* a, const void* w, int dtype, int M, int N, int K, int mode);
+int xrt_linear_norm_tiles(const void* a, const void* w, int dtype, int M, int N, int K);   // rows of the table at squares_out
 int xrt_linear_normed(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
                       int mode, const xrt_linear_norm* norm, float* workspace, long workspace_floats, void* stream);
 

@@ -37,9 +37,10 @@ SQUARES_STRIDE = 64         # rows of a table of sums of squares (XRT_SQUARES_ST
 @dataclass
 class Prescaled:
     """Rows of the residual stream on their way through an RMSNorm whose division is still to do:
-    values[m, k] = bfloat16(x[m, k] * gain[k]) and squares[t, m] = the sum of x[m, k]^2 over the 16
-    columns k of tile t. `linear` and `linear_glu` take it in place of the normed rows and divide
-    the rows of their result by the rms; nothing else can read it."""
+    values[m, k] = bfloat16(x[m, k] * gain[k]) and squares[t, m] = the sum of x[m, k]^2 over the
+    columns k of tile t (16 or fewer a tile, as the product that wrote them cut its columns). `linear`
+    and `linear_glu` take it in place of the normed rows and divide the rows of their result by the
+    rms; nothing else can read it."""
     values: torch.Tensor
     squares: torch.Tensor
     eps: float
@@ -81,7 +82,7 @@ class HipOps:
         self.path = path
         self.lib.xrt_last_error.restype = ctypes.c_char_p
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
-                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_normed", "xrt_linear_qkv"):
+                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
         self.lib.xrt_sample_workspace.restype = ctypes.c_long
@@ -157,12 +158,13 @@ class HipOps:
             gain, eps = then_norm
             self._require(gain, "norm gain", None, (n,), a)
             emit = Prescaled(torch.empty((m, n), dtype=torch.bfloat16, device=a.device),
-                             torch.empty(((n + 15) // 16, SQUARES_STRIDE), dtype=torch.float32, device=a.device),
+                             torch.empty((int(self.lib.xrt_linear_norm_tiles(*sizes, m, n, k)), SQUARES_STRIDE),
+                                         dtype=torch.float32, device=a.device),
                              float(eps))
         if scaled is not None or emit is not None:
             norm = _LinearNorm()
             if scaled is not None:
-                tiles = (k + 15) // 16
+                tiles = scaled.squares.shape[0]         # as many as the product that wrote them had tiles of columns
                 self._require(scaled.squares, "sums of squares", torch.float32, (tiles, SQUARES_STRIDE), a)
                 norm.squares_in, norm.tiles_in, norm.width_in, norm.eps = scaled.squares.data_ptr(), tiles, k, scaled.eps
             if emit is not None:
@@ -238,7 +240,7 @@ class HipOps:
                                           norm_eps, rope_theta, rope_dim, rope_scale, kv, longest_run)
         norm = None
         if scaled is not None:
-            tiles = (k + 15) // 16
+            tiles = scaled.squares.shape[0]
             self._require(scaled.squares, "sums of squares", torch.float32, (tiles, SQUARES_STRIDE), a)
             norm = _LinearNorm()
             norm.squares_in, norm.tiles_in, norm.width_in, norm.eps = scaled.squares.data_ptr(), tiles, k, scaled.eps
