@@ -277,7 +277,9 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
     // Tiles of 128 queries (four wavefronts, two workgroups to a compute unit) would spread the
     // uneven work of causal tiles better, but were measured slower at 2048 tokens (121 against
     // 101 us): every workgroup moves all its cache blocks through LDS, and with half the
-    // wavefronts per block that work doubles.
+    // wavefronts per block that work doubles. Nor do they help where tiles of 256 leave compute
+    // units empty, with a tile of many keys and one of few sharing a compute unit: 50.6 against
+    // 48.3 us at 1024 tokens, 93.6 against 93.2 at 2048.
     return launch_waves<HD, 8>(qkv, tokens, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks,
                                seq_offsets, seq_slots, seq_starts, n_seqs, out, scale, s);
 }
