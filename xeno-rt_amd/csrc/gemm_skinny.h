@@ -10,6 +10,7 @@ struct QkvAfter {
     const float* rope_theta; int rope_dim; float rope_scale;      // rope_theta null: no rotation
     int n_heads, n_kv_heads, head_dim;
     bf16* k_cache; bf16* v_cache; const int* block_table; int table_stride, n_blocks;     // k_cache null: no write
+    int kv_rows = 16;                                              // rows of a key or value head's tile: set by the kernel's launcher
 };
 
 bool xrt_linear_skinny_accepts(const void* a, const void* w, int M, int K);

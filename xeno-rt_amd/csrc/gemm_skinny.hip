@@ -53,10 +53,12 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 // registers for the stream.
 template <int MT, int RT, int MODE, typename TO, int EXTRA = 0>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skinny_kernel(
-    const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K, int rows,
+    const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K, int given_rows,
     const LinearNorm norm, const QkvAfter after) {
-    // rows: rows of w that a workgroup's tile holds, 16 or fewer (with RT == 1): the host picks them so that
-    // the workgroups divide evenly among the compute units. Lanes beyond read the tile's last row again.
+    // given_rows: rows of w that a workgroup's tile holds, 16 or fewer (with RT == 1): the host picks them so
+    // that the workgroups divide evenly among the compute units. Lanes beyond read the tile's last row again.
+    // After a q/k/v projection the tiles of the query heads have 16 rows and come first; those of the key
+    // and value heads have after.kv_rows (16 or 8).
     constexpr bool AROUND = EXTRA != 0, QKV = EXTRA == 2;
     static_assert(!AROUND || (MT == 1 && RT == 1), "the norm around a product: one tile of x, one of w per wavefront");
     static_assert(!QKV || (MODE == MODE_STORE && sizeof(TO) == 2), "after a q/k/v projection: a bfloat16 store");
@@ -76,6 +78,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 
     const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
     const int r = lane % 16, c = lane / 16;
+    int rows = given_rows;
     const long n0 = (long)blockIdx.x * (RT == 1 ? rows : 16 * RT);
     // after a q/k/v projection: the tile's head, and the dims of the head its rows 0..7 and 8..15 make
     int head = 0, lower_dim = 0, upper_dim = 8;
@@ -83,9 +86,16 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
     if constexpr (QKV) {
         // a tile: rows / 2 dims and the rows / 2 that the rotation pairs them with (beyond rope_dim and in
         // value heads: the rows / 2 dims that follow), in lanes r = 0.. and r = 8..
+        const int query_tiles = after.n_heads * (after.head_dim / 16);
+        int tile = blockIdx.x;
+        rows = 16;
+        if (tile >= query_tiles) {
+            tile -= query_tiles;
+            rows = after.kv_rows;
+        }
         const int tiles_per_head = after.head_dim / rows;
-        head = blockIdx.x / tiles_per_head;
-        const int s = blockIdx.x % tiles_per_head;
+        head = (blockIdx.x >= query_tiles ? after.n_heads : 0) + tile / tiles_per_head;
+        const int s = tile % tiles_per_head;
         const bool is_value = head >= after.n_heads + after.n_kv_heads;
         const int rotated_tiles = (after.rope_theta && !is_value) ? after.rope_dim / rows : 0;
         rotates = s < rotated_tiles;
@@ -450,13 +460,27 @@ template <int MT, int RT, typename TO>
 int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
                 const QkvAfter* after, hipStream_t s) {
     const int rows = RT == 1 && !after ? balanced_rows(N, mode) : 16;
-    const unsigned grid = (unsigned)(RT == 1 ? (N + rows - 1) / rows : (N + 16 * RT - 1) / (16 * RT));
+    unsigned grid = (unsigned)(RT == 1 ? (N + rows - 1) / rows : (N + 16 * RT - 1) / (16 * RT));
+    QkvAfter then = after ? *after : QkvAfter{};
+    if (after) {
+        // tiles of 8 rows for the key and value heads, if the compute unit with the most rows then has fewer
+        // (32 query heads and 8 key/value heads of 128: 256 + 256 tiles, 24 rows each, instead of 384 of 16)
+        const long query_tiles = (long)after->n_heads * (after->head_dim / 16), kv_tiles = 2L * after->n_kv_heads * (after->head_dim / 16);
+        auto most = [&](int kv_rows) {                          // rows of the fullest compute unit (the first)
+            const long kv = kv_tiles * (16 / kv_rows);
+            long sum = 0;
+            for (long group = 0; group < query_tiles + kv; group += 256) sum += group < query_tiles ? 16 : kv_rows;
+            return sum;
+        };
+        then.kv_rows = most(8) < most(16) ? 8 : 16;
+        grid = (unsigned)(query_tiles + kv_tiles * (16 / then.kv_rows));
+    }
     const dim3 block(WAVES * XRT_WAVE);
     const QkvAfter none = {};
     if constexpr (MT == 1 && RT == 1) {
         if (after) {
             if constexpr (sizeof(TO) == 2) {
-                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, *after);
+                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, then);
                 XRT_LAUNCH_CHECK("linear (skinny, q/k/v)");
                 return 0;
             }
