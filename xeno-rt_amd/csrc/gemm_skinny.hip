@@ -2,7 +2,7 @@
 // float32 accumulation on the matrix cores: out[m, n] = sum_k x[m, k] * w[n, k].
 //
 // Such a product is bound by reading w once from HBM, so the kernel is built around that
-// stream. A workgroup of 8 wavefronts owns 16 (or 32) rows of w. Each wavefront takes one
+// stream. A workgroup of 8 wavefronts owns 16 (or 32, or fewer than 16: see balanced_rows) rows of w. Each wavefront takes one
 // eighth of K and streams its part of those rows straight from global memory into the A
 // operand of v_mfma_f32_16x16x32_bf16: a 64-wide K step is two load instructions, and in each
 // the four lanes (r, 0..3) of a row read 64 contiguous bytes of it, so that a step takes one
