@@ -645,6 +645,27 @@ def test_sample_with_ties_by_the_thousand_and_a_large_top_k(ops):
         assert set(torch.nonzero(counts).flatten().tolist()) <= set(torch.nonzero(dist).flatten().tolist())
 
 
+def test_sample_largest_logit_slice_by_slice(ops):
+    """Rows that take the largest logit, in a vocabulary large enough for the way through slices: the first
+    index among equals, also when they lie in different slices; NaN never wins; a row of nothing but NaN
+    or -inf gives index 0; the penalty counts. (The helper checks both ways against each other.)"""
+    vocab = 50000
+    torch.manual_seed(11)
+    logits = torch.randn(7, vocab)
+    logits[0, [40000, 123, 4096 * 5 + 7]] = 9.0                    # equal maxima in three slices: the first index
+    logits[1, ::3] = float("nan"); logits[1, 30001] = 8.0          # NaN all over
+    logits[2] = float("nan")
+    logits[3] = float("-inf")
+    logits[4, 49999] = 20.0                                        # the very last token, in the last, partly filled slice
+    logits[5, 7] = 5.0; logits[5, 20000] = 4.9                     # the penalty takes the first one down
+    logits[6] = -logits[6].abs() - 1.0; logits[6, 33333] = -0.5    # all negative
+    logits = logits.to(DEV)
+    picked = sample(ops, logits)
+    assert picked[:5] == [123, 30001, 0, 0, 49999] and picked[6] == 33333
+    assert picked[5] == 7
+    assert sample(ops, logits, penalty=1.5, history=[7, 8, 9])[5] == 20000
+
+
 def test_sample_keeps_the_tokens_on_the_device_where_asked(ops):
     """With append_at the chosen token is also written behind the row's span of the history, on every way
     through the kernels (greedy, passes over the row, candidates from slices), and only for the rows

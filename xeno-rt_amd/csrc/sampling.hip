@@ -435,7 +435,8 @@ constexpr int SLICE_TOPS = 8;          // of a slice's largest values, one per t
 constexpr int LEAST_SLICES = 8;        // with fewer slices their tops are too few to bound a top-k of FAST_TOP_K
 
 struct SliceCandidates {
-    int count;                         // -1: this row does not go this way; more than SLICE_HOLDS: they did not fit
+    int count;                         // -1: this row does not go this way; more than SLICE_HOLDS: they did not fit;
+                                       // -2: a row that takes the largest logit: `largest` is the slice's, `unused` its first index (0x7fffffff: none)
     float largest, mass;               // for a row without top-k: the slice's largest value, and the sum of exp((value - largest) / temperature)
     int unused;
     unsigned top[SLICE_TOPS];          // keys of SLICE_TOPS different tokens of the slice, the largest first (0: none)
@@ -484,8 +485,9 @@ __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
     __shared__ int held;
     const int r = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
     SliceCandidates& mine = candidates[(long)r * slices + slice];
+    const bool greedy = temperature[r] <= 1e-5f;                // the largest logit, first index: the slices' largest, then the first of those
     const int k = top_k_by_slices(temperature[r], top_k[r], top_p[r], vocab);
-    if (k == 0) {
+    if (k == 0 && !greedy) {
         if (tid == 0) mine.count = -1;
         return;
     }
@@ -517,6 +519,33 @@ __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
         value[e] = (seen[local >> 5] >> (local & 31)) & 1u ? changed : v;
         // key 0 stands for "no token"; no float maps to it but a NaN with all bits set, which can go without loss
         key[e] = first + local < vocab ? order_key(value[e]) : 0u;
+    }
+    if (greedy) {
+        // strict >, so NaN never wins (sampler.rs:83-98); a thread's tokens come in the order of their indices
+        float best = -INFINITY;
+        int best_index = 0x7fffffff;
+#pragma unroll
+        for (int e = 0; e < SLICE_EACH; ++e)
+            if (key[e] != 0u && value[e] > best) { best = value[e]; best_index = first + e * SLICE_THREADS + tid; }
+#pragma unroll
+        for (int offset = XRT_WAVE / 2; offset > 0; offset >>= 1) {
+            const float other = __shfl_xor(best, offset, XRT_WAVE);
+            const int other_index = __shfl_xor(best_index, offset, XRT_WAVE);
+            if (other > best || (other == best && other_index < best_index)) { best = other; best_index = other_index; }
+        }
+        if (tid % XRT_WAVE == 0) { wave_mass[tid / XRT_WAVE] = best; maxima[tid / XRT_WAVE] = (unsigned)best_index; }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < SLICE_WAVES; ++w) {
+                const float other = wave_mass[w];
+                const int other_index = (int)maxima[w];
+                if (other > best || (other == best && other_index < best_index)) { best = other; best_index = other_index; }
+            }
+            mine.count = -2;
+            mine.largest = best;
+            mine.unused = best_index;
+        }
+        return;
     }
     unsigned largest = 0u;
     float largest_value = -INFINITY;
@@ -581,6 +610,20 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
     const SliceCandidates* mine = candidates + (long)r * slices;
     // where every slice's candidates start in the row's list (one lane per slice; an inclusive sum over the
     // lanes); a slice that says "not this way" or "they did not fit" sends the row to the whole-row path
+    if (temperature[r] <= 1e-5f) {                              // the largest logit: the largest of the slices', the first among equals
+        if (tid < XRT_WAVE) {
+            float best = tid < slices ? mine[tid].largest : -INFINITY;
+            int best_index = tid < slices ? mine[tid].unused : 0x7fffffff;
+#pragma unroll
+            for (int offset = XRT_WAVE / 2; offset > 0; offset >>= 1) {
+                const float other = __shfl_xor(best, offset, XRT_WAVE);
+                const int other_index = __shfl_xor(best_index, offset, XRT_WAVE);
+                if (other > best || (other == best && other_index < best_index)) { best = other; best_index = other_index; }
+            }
+            if (tid == 0) out.put(r, best_index == 0x7fffffff ? 0 : best_index);   // nothing compared greater (all NaN or -inf): index 0
+        }
+        return;
+    }
     const bool no_top_k = top_k[r] == 0;                        // a top-p alone: see top_k_by_slices
     const int k = no_top_k ? FAST_TOP_K : top_k[r];
     if (tid < XRT_WAVE) {

@@ -133,8 +133,9 @@ class Sampler:
                                                    + (append_at if log is not None else history))
             self._last = (made_from, (floats, ints))
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
-        # rows that the kernels can sample from a few candidates instead of passes over the whole row
-        small_top_k = any(not c.is_greedy() and (0 < c.top_k <= 64 or (c.top_k == 0 and c.top_p < 1.0)) for c in configs)
+        # rows that the kernels can sample from a few candidates instead of passes over the whole row, and rows
+        # that take the largest logit (many workgroups look for it slice by slice, instead of one over the row)
+        small_top_k = any(c.is_greedy() or 0 < c.top_k <= 64 or (c.top_k == 0 and c.top_p < 1.0) for c in configs)
         if log is not None:
             self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2], log[0].tokens,
                             ints[rows:3 * rows], floats[3], small_top_k=small_top_k, append_at=ints[3 * rows:])
