@@ -365,3 +365,42 @@ def test_norms_are_handed_to_the_products_only_where_every_part_agrees(pair, tmp
     # layer 0's o is no longer followed by a handed norm, and nothing is handed on behind its down
     assert sum(1 for _, then in handed if then) == 2 * layers - 1 - 2
     assert sum(1 for scaled, _ in handed if scaled) == layers - 2
+
+
+def test_buckets_of_recorded_decode_steps():
+    from xeno_rt_amd.engine.graphs import batch_bucket, context_bucket
+    sizes = [batch_bucket(n) for n in range(1, 130)]
+    assert all(size >= n for n, size in enumerate(sizes, start=1))            # a bucket holds its batch
+    assert sizes == sorted(sizes)
+    assert sorted(set(sizes)) == [1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192]
+    assert [context_bucket(n, 5000) for n in (1, 1024, 1025, 4096, 4097, 5000)] == [1024, 1024, 2048, 4096, 5000, 5000]
+
+
+def test_staging_on_the_host_stand_in():
+    """Without a GPU the staging area hands the values through: copies, never views of what it was given."""
+    from xeno_rt_amd.staging import staging_for
+    staging = staging_for("cpu")
+    assert staging.upload([3, 1, 2]).tolist() == [3, 1, 2]
+    assert staging.upload([0.5, 2.0], dtype=torch.float32).dtype == torch.float32
+    table = torch.arange(6, dtype=torch.int32).view(2, 3)
+    copy = staging.upload(table[1:2])
+    table[1, 0] = 99
+    assert copy.tolist() == [[3, 4, 5]]
+    out = torch.zeros(2, 3, dtype=torch.int32)
+    staging.upload(table, out=out)
+    assert out.tolist() == [[0, 1, 2], [99, 4, 5]]
+    assert staging.fetch(torch.tensor([7, 8], dtype=torch.int32)).values() == [7, 8]
+
+
+def test_token_log_lays_sequences_out_with_room():
+    log = TokenLog("cpu", [[5, 6, 7], [], [9]], [2, 4, 0])
+    assert log.begin == [0, 5, 9] and log.end == [5, 9, 10]
+    assert log.tokens[:3].tolist() == [5, 6, 7] and int(log.tokens[9]) == 9
+    # the sampler refuses a row whose log is full, before any kernel runs
+    sampler = Sampler(EmulatedOps(), "cpu")
+    config = SamplerConfig(temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.5)
+    logits = torch.zeros(1, 16)
+    with pytest.raises(ValueError, match="no room"):
+        sampler.launch(logits, [config], [[9]], [0.0], log=(log, [2]))
+    picked = sampler.launch(logits, [config], [[5, 6, 7]], [0.0], log=(log, [0]))
+    assert int(log.tokens[3]) == int(picked[0])                 # the chosen token was appended behind the sequence's three
