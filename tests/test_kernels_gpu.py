@@ -106,7 +106,9 @@ def test_linear(ops, dtype, m, n, k):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("m,n,k", [(1, 176, 64), (9, 100, 96), (64, 520, 200), (200, 1000, 72), (48, 2000, 520),
                                    (2048, 3100, 64), (300, 130, 1032), (2048, 3072, 128), (2000, 3000, 192), (2048, 4224, 64),
-                                   (64, 520, 256), (50, 1000, 1024), (200, 1000, 512)])
+                                   (64, 520, 256), (50, 1000, 1024), (200, 1000, 512),
+                                   # 17 to 64 rows and tiles enough without a split along k
+                                   (40, 14336, 256), (64, 9002, 128), (33, 20000, 192)])
 def test_linear_glu(ops, dtype, m, n, k):
     a = rand(m, k, dtype=DT[dtype], seed=1)
     w = rand(2 * n, k, dtype=DT[dtype], seed=2, scale=0.3)
