@@ -29,6 +29,16 @@ int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype
                int mode, float* workspace, long workspace_floats, void* stream);
 long xrt_linear_workspace(const void* a, const void* w, int dtype, int M, int N, int K, int mode);
 
+// xrt_linear for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+// loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. The partial sums of a
+// product split along k go to a fixed array of XRT_LINEAR_STATIC_FLOATS floats (16 MiB) that the library
+// holds in device memory on every GPU it is used on; the call allocates nothing and refuses a product
+// whose partial sums do not fit (xrt_linear_workspace says how many floats a product needs). Calls on one
+// GPU share that array: calls that overlap there (different streams) race.
+#define XRT_LINEAR_STATIC_FLOATS (4L << 20)
+int xrt_linear_static(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
+                      int mode, void* stream);
+
 // An RMSNorm between two products, x += a w^T; y = rmsnorm(x) * gain; z = y v^T, without a kernel of
 // its own. The first product (mode 1) also writes scaled_out[m, n] = bfloat16(x[m, n] * gain[n]) and
 // squares_out[t * XRT_SQUARES_STRIDE + m], the sum of x[m, n]^2 over the columns n of tile t (xrt_linear_norm_tiles of them, 16 columns or fewer each). The
