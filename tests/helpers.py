@@ -20,9 +20,14 @@ def errors(got: torch.Tensor, want: torch.Tensor):
     return float(diff.abs().max()) / scale, float(diff.pow(2).mean().sqrt()) / scale
 
 
+SEEN = {}       # dtype -> [largest max error, largest rms error] that passed: printed at the end of a run
+
+
 def assert_logits(got, want, dtype, what=""):
     assert torch.isfinite(got).all(), f"{what}: logits are not finite"
     worst, rms = errors(got, want)
+    seen = SEEN.setdefault(dtype, [0.0, 0.0])
+    seen[0], seen[1] = max(seen[0], worst), max(seen[1], rms)
     limit = TOLERANCE[dtype]
     assert worst <= limit["max"] and rms <= limit["rms"], \
         f"{what} [{dtype}]: max error {worst:.3e} (limit {limit['max']:.1e}), rms {rms:.3e} (limit {limit['rms']:.1e})"

@@ -1,7 +1,7 @@
 """Plain, slow implementation of the Llama / Qwen3 dense decoder.
 
 Whole sequences, no cache, one function for each part, written from the
-formulas of the reference (cited as file:line under /root/reference). It
+formulas of the reference (cited as file:line of the reference's own tree). It
 shares no code with the engine: it reads the model folder with the
 `safetensors` package and `json`, and computes with elementary torch tensor
 operations on the CPU (float32 by default, float64 on request).
@@ -123,13 +123,13 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_heads:
     kh = k.reshape(k.shape[0], n_kv_heads, head_dim)
     vh = v.reshape(v.shape[0], n_kv_heads, head_dim)
     out = torch.zeros_like(qh)
-    for t in range(tokens):
-        attend_len = start_position + t + 1                      # llama.rs:736
-        for head in range(n_heads):
-            kv_head = head // group                              # llama.rs:741
-            scores = (kh[:attend_len, kv_head, :] @ qh[t, head, :]) * scale   # :744-751
-            probs = softmax(scores)                              # :753
-            out[t, head, :] = probs @ vh[:attend_len, kv_head, :]  # :756-768
+    # attend_len = start_position + t + 1 (llama.rs:736): key j is hidden from query t if j > start_position + t
+    hidden = torch.arange(k.shape[0])[None, :] > (start_position + torch.arange(tokens))[:, None]
+    for head in range(n_heads):
+        kv_head = head // group                                  # llama.rs:741
+        scores = (qh[:, head, :] @ kh[:, kv_head, :].t()) * scale            # :744-751, all queries of the head at once
+        probs = softmax(scores.masked_fill(hidden, -math.inf))   # :753 over the keys each query sees
+        out[:, head, :] = probs @ vh[:, kv_head, :]              # :756-768
     return out.reshape(tokens, n_heads * head_dim)
 
 
@@ -174,33 +174,49 @@ class PlainModel:
             for name in handle.keys():
                 self.weights[name] = handle.get_tensor(name).to(dtype)
 
+    @classmethod
+    def from_weights(cls, raw_config: dict, weights: dict, dtype=torch.float32) -> "PlainModel":
+        """From config.json's contents and tensors by checkpoint name (any float type)."""
+        model = cls.__new__(cls)
+        model.config = PlainConfig(raw_config)
+        model.dtype = dtype
+        model.weights = {name: tensor.to(dtype) for name, tensor in weights.items()}
+        return model
+
     def w(self, name: str) -> torch.Tensor:
         return self.weights[name]
 
     # -- one block: norm -> attention -> add -> norm -> feed-forward -> add ----
-    def block(self, layer: int, x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
-        """crates/xrt-models/src/llama.rs:433-602 (decode) / 676-810 (prefill)."""
+    def block(self, layer: int, x: torch.Tensor, positions: torch.Tensor, tail: int = 0) -> torch.Tensor:
+        """crates/xrt-models/src/llama.rs:433-602 (decode) / 676-810 (prefill).
+
+        With tail = n only the last n positions are returned: keys and values are made for every
+        position, queries and everything after the attention only for those n (what the reference's
+        decode step computes for one position, llama.rs:447-602, against the keys before it)."""
         c = self.config
         p = f"model.layers.{layer}."
+        first = x.shape[0] - tail if tail else 0
         normed = rmsnorm(x, self.w(p + "input_layernorm.weight"), c.eps)           # :441-442
-        q = linear(normed, self.w(p + "self_attn.q_proj.weight"))                 # :447-486
+        q = linear(normed[first:], self.w(p + "self_attn.q_proj.weight"))         # :447-486
         k = linear(normed, self.w(p + "self_attn.k_proj.weight"))
         v = linear(normed, self.w(p + "self_attn.v_proj.weight"))
         if c.qk_norm:                                                              # :489-496
             q = head_rmsnorm(q, c.n_heads, c.head_dim, self.w(p + "self_attn.q_norm.weight"), c.eps)
             k = head_rmsnorm(k, c.n_kv_heads, c.head_dim, self.w(p + "self_attn.k_norm.weight"), c.eps)
-        q = rope(q, c.n_heads, c.head_dim, positions, c.rope_dim, c.rope_theta)    # :498-500
+        q = rope(q, c.n_heads, c.head_dim, positions[first:], c.rope_dim, c.rope_theta)    # :498-500
         k = rope(k, c.n_kv_heads, c.head_dim, positions, c.rope_dim, c.rope_theta)
-        attn = causal_attention(q, k, v, c.n_heads, c.n_kv_heads, c.head_dim)      # :504-574
-        x = x + linear(attn, self.w(p + "self_attn.o_proj.weight"))               # :576-577
+        attn = causal_attention(q, k, v, c.n_heads, c.n_kv_heads, c.head_dim, start_position=first)   # :504-574
+        x = x[first:] + linear(attn, self.w(p + "self_attn.o_proj.weight"))       # :576-577
         normed = rmsnorm(x, self.w(p + "post_attention_layernorm.weight"), c.eps)  # :579-580
         gate = linear(normed, self.w(p + "mlp.gate_proj.weight"))                 # :584-598
         up = linear(normed, self.w(p + "mlp.up_proj.weight"))
         x = x + linear(swiglu(gate, up), self.w(p + "mlp.down_proj.weight"))      # :599-601
         return x
 
-    def logits(self, token_ids) -> torch.Tensor:
-        """Logits [T, V] at every position of one whole sequence, positions 0..T-1.
+    def logits(self, token_ids, tail: int = 0) -> torch.Tensor:
+        """Logits [T, V] at every position of one whole sequence, positions 0..T-1; with tail = n only
+        at the last n positions (the layers before the last still run every position: their outputs
+        make the next layer's keys and values).
 
         crates/xrt-models/src/llama.rs:830-1009 (forward_batch_all_logits).
         """
@@ -212,8 +228,9 @@ class PlainModel:
             raise ValueError("token id exceeds embedding rows")                   # :1044-1049
         positions = torch.arange(ids.numel())
         x = self.w("model.embed_tokens.weight")[ids]                              # :666-669
+        tail = min(int(tail), ids.numel())
         for layer in range(c.layers):
-            x = self.block(layer, x, positions)
+            x = self.block(layer, x, positions, tail=tail if layer == c.layers - 1 else 0)
         normed = rmsnorm(x, self.w("model.norm.weight"), c.eps)                   # :604-609
         head = self.w("model.embed_tokens.weight") if c.tied else self.w("lm_head.weight")  # :301-305
         return linear(normed, head)                                               # :613

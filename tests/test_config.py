@@ -37,6 +37,18 @@ def test_defaults_of_absent_keys_are_the_references():
     assert config.rope_dim == config.head_dim
 
 
+def test_rotary_base_inside_rope_parameters_is_read_not_ignored():
+    raw = {k: v for k, v in TINY["qwen3"].items() if k != "rope_theta"}
+    raw["rope_parameters"] = {"rope_theta": 1000000.0, "rope_type": "default"}
+    assert parse_config(raw).rope_theta == 1000000.0
+    assert parse_config(raw) == parse_config(TINY["qwen3"])
+
+
+def test_written_config_names_its_model_type(tmp_path):
+    for name, model_type in (("llama", "llama"), ("qwen3", "qwen3")):
+        assert parse_config(TINY[name]).to_dict()["model_type"] == model_type
+
+
 def test_eos_may_be_a_number_or_a_list():
     assert parse_config(TINY["llama"]).eos_token_ids == (1,)
     assert parse_config(TINY["qwen3"]).eos_token_ids == (2, 5)
@@ -58,6 +70,11 @@ def test_eos_may_be_a_number_or_a_list():
     ({"eos_token_id": 9999}, "outside the vocabulary"),
     ({"rms_norm_eps": 0.0}, "rms_norm_eps"),
     ({"vocab_size": "many"}, "vocab_size"),
+    ({"model_type": "qwen3"}, "model_type"),
+    ({"rope_parameters": {"rope_theta": 10000.0, "rope_type": "yarn"}}, "rope_type"),
+    ({"rope_parameters": {"rope_theta": 10000.0, "factor": 4.0}}, "rope_parameters"),
+    ({"rope_parameters": {"rope_theta": 500000.0}}, "disagree"),
+    ({"partial_rotary_factor": 0.5}, "partial_rotary_factor"),
 ])
 def test_bad_configs_are_refused(change, text):
     with pytest.raises(ConfigError, match=text):

@@ -155,7 +155,9 @@ def test_the_loop_runs_a_step_ahead_of_the_host(pair, monkeypatch):
     # with a repetition penalty too: the tokens it reads are kept on the device (the sampler appends them), and
     # they are those that a loop through the host hands to the sampler at every step
     calls.update(step=0, step_from=0)
-    prompt = [43, 44, 45]           # left alone, the model repeats its second token from here on
+    # a prompt after which the model, left alone, repeats its second token
+    prompt = next(p for p in ([a, a + 1, a + 2] for a in range(3, 250))
+                  if (lambda free: free[1] == free[2] and free[0] != free[1])(P.generate_greedy(plain, p, 3, stop_ids=[])))
     penalised = GenerateRequest(prompt, max_tokens=5, stop_ids=[], temperature=0.0, repetition_penalty=3.0)
     got = generate(engine, [penalised, GenerateRequest([50, 60], max_tokens=3, stop_ids=[], **GREEDY)])
     assert calls == {"step": 1, "step_from": 4}

@@ -226,6 +226,72 @@ def test_norm_weights_and_qk_norm_matter(tmp_path):
     assert float((model.logits(ids) - base).abs().max()) > 1e-2
 
 
+def test_a_block_sees_positions_only_as_distances(tmp_path):
+    """Keys and queries are normed per head and then rotated, values are not rotated at all: then every
+    score depends on the distance between query and key alone, and a block gives the same output when all
+    positions are shifted. The head norm after the rotation (its weights differ along the head, so they
+    would break the pairs' rotation) or a rotated value fails this."""
+    model = _model(tmp_path, "qwen3")
+    c = model.config
+    p = "model.layers.1.self_attn."
+    assert float((model.w(p + "q_norm.weight") - 1).abs().max()) > 0.05         # the fixture's head norms are not ones
+    x = torch.randn(9, c.hidden, generator=torch.Generator().manual_seed(4))
+    positions = torch.arange(9)
+    base = model.block(1, x, positions)
+    close(model.block(1, x, positions + 37), base, 1e-5 * float(base.abs().max()))     # float32 angles round differently
+    # the guard: the same parts with the norm after the rotation do depend on absolute positions
+    def scores_with_norm_last(at):
+        normed = P.rmsnorm(x, model.w("model.layers.1.input_layernorm.weight"), c.eps)
+        q = P.rope(P.linear(normed, model.w(p + "q_proj.weight")), c.n_heads, c.head_dim, at, c.rope_dim, c.rope_theta)
+        k = P.rope(P.linear(normed, model.w(p + "k_proj.weight")), c.n_kv_heads, c.head_dim, at, c.rope_dim, c.rope_theta)
+        q = P.head_rmsnorm(q, c.n_heads, c.head_dim, model.w(p + "q_norm.weight"), c.eps)
+        k = P.head_rmsnorm(k, c.n_kv_heads, c.head_dim, model.w(p + "k_norm.weight"), c.eps)
+        return q[:, :c.head_dim] @ k[:, :c.head_dim].t()
+    assert float((scores_with_norm_last(positions) - scores_with_norm_last(positions + 37)).abs().max()) > 1e-3
+
+
+def test_the_feed_forward_reads_the_stream_after_the_attention_was_added(tmp_path):
+    """norm, attention, add, norm, feed-forward, add: with the feed-forward silenced a block returns
+    x1 = x + attention; with both live it returns x1 + feed_forward(norm2(x1)). A block whose two halves
+    both read the incoming stream (a parallel block), or a norm after the sum, fails this."""
+    model = _model(tmp_path, "llama")
+    c = model.config
+    p = "model.layers.0."
+    x = torch.randn(6, c.hidden, generator=torch.Generator().manual_seed(8))
+    positions = torch.arange(6)
+    both = model.block(0, x, positions)
+    kept = model.w(p + "mlp.down_proj.weight").clone()
+    model.weights[p + "mlp.down_proj.weight"].zero_()
+    x1 = model.block(0, x, positions)
+    model.weights[p + "mlp.down_proj.weight"].copy_(kept)
+    normed = P.rmsnorm(x1, model.w(p + "post_attention_layernorm.weight"), c.eps)
+    want = x1 + P.linear(P.swiglu(P.linear(normed, model.w(p + "mlp.gate_proj.weight")),
+                                  P.linear(normed, model.w(p + "mlp.up_proj.weight"))), kept)
+    close(both, want, 1e-5)
+    parallel = P.rmsnorm(x, model.w(p + "post_attention_layernorm.weight"), c.eps)
+    wrong = x1 + P.linear(P.swiglu(P.linear(parallel, model.w(p + "mlp.gate_proj.weight")),
+                                   P.linear(parallel, model.w(p + "mlp.up_proj.weight"))), kept)
+    assert float((both - wrong).abs().max()) > 1e-2
+
+
+def test_logits_of_the_last_positions_alone_are_those_of_the_whole(tmp_path):
+    for name in ("llama", "qwen3"):
+        model = _model(tmp_path, name)
+        ids = list(range(20, 61))
+        whole = model.logits(ids)
+        for tail in (1, 5, len(ids), len(ids) + 3):
+            close(model.logits(ids, tail=tail), whole[-tail:], 1e-5)
+
+
+def test_model_from_tensors_is_the_model_from_the_folder(tmp_path):
+    import json, os
+    model = _model(tmp_path, "qwen3")
+    raw = json.load(open(os.path.join(str(tmp_path / "qwen3"), "config.json")))
+    again = P.PlainModel.from_weights(raw, {name: tensor.clone() for name, tensor in model.weights.items()})
+    ids = [3, 1, 4, 1, 5, 9, 2, 6]
+    assert torch.equal(again.logits(ids), model.logits(ids))
+
+
 # ---- sampling and the loop -------------------------------------------------------------
 
 def test_greedy_and_penalty_reference_cases():

@@ -118,8 +118,82 @@ def test_stored_precision_is_kept(tmp_path):
     tensors = load_tensors(folder, spec.weight_specs())
     assert tensors["model.norm.weight"].dtype == torch.float32                 # 32-bit stays 32-bit
     assert float(tensors["model.norm.weight"][0]) == pytest.approx(1.001, abs=1e-7)
-    assert tensors["model.layers.0.mlp.up_proj.weight"].dtype == torch.bfloat16
+    assert tensors["model.layers.0.mlp.up_proj.weight"].dtype == torch.float16    # as stored: the binder converts
     assert tensors["model.embed_tokens.weight"].dtype == torch.bfloat16
+
+
+def test_float16_checkpoint_widens_exactly_on_the_32_bit_path_and_is_rounded_only_on_the_other(tmp_path):
+    """What the parts bind: a float32 model holds float16(w) exactly, a bfloat16 model its rounding."""
+    from ops_emulation import EmulatedOps
+    from xeno_rt_amd.engine import Engine
+
+    stored = {}
+
+    def edit(t):
+        for name in list(t):
+            t[name] = (t[name].float() * 1.37).to(torch.float16)     # values that bfloat16 cannot hold
+        stored.update({name: value.clone() for name, value in t.items()})
+    folder, spec = folder_with(tmp_path, "llama", edit)
+    engine = Engine.load(folder, dtype="float32", max_tokens=128, device="cpu", ops=EmulatedOps())
+    mixer, mlp = engine.model.spec.layers[1].mixer, engine.model.spec.layers[1].feed_forward
+    p = "model.layers.1."
+    want_qkv = torch.cat([stored[p + f"self_attn.{n}_proj.weight"].float() for n in "qkv"])
+    assert mixer.w_qkv.dtype == torch.float32 and torch.equal(mixer.w_qkv, want_qkv)
+    assert torch.equal(mlp.w_down, stored[p + "mlp.down_proj.weight"].float())
+    norm = engine.model.spec.final_norm.weight
+    assert norm.dtype == torch.float32 and torch.equal(norm, stored["model.norm.weight"].float())
+    assert torch.equal(engine.get_tensor(p + "mlp.up_proj.weight"), stored[p + "mlp.up_proj.weight"])
+    rounded = Engine.load(folder, dtype="bfloat16", max_tokens=128, device="cpu", ops=EmulatedOps())
+    assert torch.equal(rounded.model.spec.layers[1].mixer.w_qkv, want_qkv.to(torch.bfloat16))
+    assert not torch.equal(want_qkv.to(torch.bfloat16).float(), want_qkv)
+    # a float16 vector is never squeezed into bfloat16: it widens
+    assert rounded.model.spec.final_norm.weight.dtype == torch.float32
+
+
+def test_random_weights_are_the_same_in_the_file_in_memory_and_in_any_pieces(tmp_path):
+    """Every element depends on (seed, tensor name, element index) alone."""
+    from ops_emulation import EmulatedOps
+    from xeno_rt_amd.engine import Engine
+    from xeno_rt_amd.weights import make_tensor
+    from xeno_rt_amd.weights import random_init
+    from xeno_rt_amd.parts.base import WeightSpec
+
+    config = parse_config(TINY["qwen3"])
+    folder = write_random_model(config, str(tmp_path / "m"), seed=5, std=0.05, gain_std=0.1)
+    engine = Engine.random(config, seed=5, std=0.05, gain_std=0.1, dtype="bfloat16", max_tokens=128, device="cpu",
+                           ops=EmulatedOps())
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as file:
+        for name in file.names():
+            assert torch.equal(file.read(name), engine.get_tensor(name)), name
+        gains = file.read("model.layers.0.input_layernorm.weight").float()
+        assert 0.05 < float((gains - 1).abs().mean()) < 0.15
+    p = "model.layers.2.self_attn."
+    bound = engine.model.spec.layers[2].mixer.w_qkv
+    assert torch.equal(bound, torch.cat([engine.get_tensor(p + f"{n}_proj.weight") for n in "qkv"]))
+    # float32 and bfloat16 models of one seed hold the same numbers before rounding
+    wide = Engine.random(config, seed=5, std=0.05, dtype="float32", max_tokens=128, device="cpu", ops=EmulatedOps())
+    name = "model.layers.1.mlp.gate_proj.weight"
+    assert torch.equal(wide.get_tensor(name).to(torch.bfloat16), engine.get_tensor(name))
+    # pieces: elements 1000 .. 1010 made alone equal those of the whole; another name or seed gives other values
+    key = random_init.tensor_key(5, name)
+    whole = random_init.normal_values(key, 0, 5000, 1.0)
+    assert torch.equal(random_init.normal_values(key, 1000, 10, 1.0), whole[1000:1010])
+    # the tensor arithmetic against the generator written out on Python integers
+    for i in (0, 1, 999, 4999):
+        words = [random_init._mix((key + (2 * i + j) * random_init._GOLDEN) & random_init._MASK) for j in (0, 1)]
+        total = sum((word >> (10 * field)) & 1023 for word in words for field in range(6))
+        assert float(whole[i]) == float(2 * total - 12 * 1023)
+    assert not (random_init.normal_values(random_init.tensor_key(5, name + "x"), 0, 5000, 1.0) == whole).all()
+    assert not (random_init.normal_values(random_init.tensor_key(6, name), 0, 5000, 1.0) == whole).all()
+    # a tensor's values do not depend on the other tensors of the model, nor on its shape's cut
+    spec = WeightSpec((50, 100))
+    assert torch.equal(make_tensor(spec, 5, name, 0.05, torch.float32).reshape(-1),
+                       make_tensor(WeightSpec((5000,)), 5, name, 0.05, torch.float32))
+    # and they are normal enough: moments of a large sample
+    sample = random_init.normal_values(key, 0, 1 << 20, random_init.normal_scale(1.0)).double()
+    assert abs(float(sample.mean())) < 4e-3 and abs(float(sample.std()) - 1.0) < 4e-3
+    assert abs(float((sample ** 4).mean()) - 3.0) < 0.15          # twelve uniforms: kurtosis 2.9
+    assert 0.0015 < float((sample.abs() > 3.0).double().mean()) < 0.0035      # normal: 0.0027
 
 
 def test_random_weights_follow_seed_and_rule(tmp_path):

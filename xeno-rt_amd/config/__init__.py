@@ -58,6 +58,8 @@ class LlamaConfig:
 
     # Architectures that this class parses, and whether each norms q and k per head.
     QK_NORM_BY_ARCHITECTURE = {"LlamaForCausalLM": False, "Qwen3ForCausalLM": True}
+    # what checkpoint folders of these architectures carry under `model_type`
+    MODEL_TYPE_BY_ARCHITECTURE = {"LlamaForCausalLM": "llama", "Qwen3ForCausalLM": "qwen3"}
 
     @property
     def q_width(self) -> int:            # llama.rs:130-132
@@ -103,8 +105,30 @@ class LlamaConfig:
         if head_dim % 2 != 0:
             raise ConfigError(f"config.json: head_dim {head_dim} must be even (rotary pairs)")
 
+        model_type = raw.get("model_type")
+        if model_type is not None and model_type != cls.MODEL_TYPE_BY_ARCHITECTURE[architecture]:
+            raise ConfigError(f"config.json: model_type {model_type!r} does not belong to {architecture}")
         if raw.get("rope_scaling") not in (None, {}):
             raise ConfigError("config.json: 'rope_scaling' is not supported (must be null or absent)")
+        # newer checkpoint folders carry the rotary base inside `rope_parameters`; anything there that would
+        # change the angles (a scaling rule, a factor) is refused, never ignored
+        rope_parameters = raw.get("rope_parameters")
+        if rope_parameters is not None:
+            if not isinstance(rope_parameters, dict):
+                raise ConfigError("config.json: 'rope_parameters' must be an object")
+            unknown = sorted(set(rope_parameters) - {"rope_theta", "rope_type"})
+            if unknown:
+                raise ConfigError(f"config.json: 'rope_parameters' has keys that are not supported: {unknown}")
+            if rope_parameters.get("rope_type") not in (None, "default"):
+                raise ConfigError(f"config.json: rope_type {rope_parameters.get('rope_type')!r} is not supported "
+                                  "(only 'default')")
+            inner = rope_parameters.get("rope_theta")
+            if inner is not None:
+                if raw.get("rope_theta") is not None and float(raw["rope_theta"]) != float(inner):
+                    raise ConfigError("config.json: 'rope_theta' and 'rope_parameters.rope_theta' disagree")
+                raw = dict(raw, rope_theta=inner)
+        if raw.get("partial_rotary_factor") not in (None, 1, 1.0):
+            raise ConfigError("config.json: 'partial_rotary_factor' must be 1 or absent (the whole head is rotated)")
         activation = raw.get("hidden_act", "silu")
         if activation != "silu":
             raise ConfigError(f"config.json: hidden_act must be 'silu', found {activation!r}")
@@ -158,6 +182,7 @@ class LlamaConfig:
         eos = list(self.eos_token_ids)
         return {
             "architectures": [self.architecture],
+            "model_type": self.MODEL_TYPE_BY_ARCHITECTURE[self.architecture],
             "vocab_size": self.vocab_size,
             "hidden_size": self.hidden_size,
             "intermediate_size": self.intermediate_size,

@@ -13,6 +13,11 @@ const char* xrt_last_error(void);
 int xrt_embed(const void* table, int table_dtype, const int* ids, float* out, int tokens, int hidden,
               int vocab, void* stream);
 
+// out[i] = element i of the random-weights stream `key`: float(2 * (sum of twelve 10-bit fields of two
+// splitmix64 words) - 12 * 1023) * scale + offset, the same values as the host-side generator gives
+int xrt_random_normal(void* out, int dtype, long count, unsigned long long key, float scale, float offset,
+                      void* stream);
+
 // residual[i] += delta[i]
 int xrt_add(float* residual, const void* delta, int delta_dtype, long count, void* stream);
 

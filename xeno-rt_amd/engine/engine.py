@@ -19,7 +19,7 @@ from ..cache import BLOCK_TOKENS, CacheError, CacheFull, SequenceCache
 from ..config import architecture, load_config
 from ..models import DecoderModel, ModelSpec
 from ..parts.base import Runtime
-from ..weights import load_tensors
+from ..weights import CheckpointSource, RandomSource
 from ..staging import staging_for
 from .batch import build_batch
 
@@ -53,7 +53,9 @@ class Engine:
         self.ops = ops
         self.runtime = Runtime(ops, self.dtype, self.device)
         self.config = spec.config
-        self.tensors = tensors          # by checkpoint name, as loaded (or made on demand): see get_tensor
+        # by checkpoint name: a dict, or a source that reads or makes a tensor when a part asks for it and
+        # keeps none, so that the device holds every weight once, in the form the parts bound it
+        self.tensors = tensors
         self.model = DecoderModel(spec, tensors, self.runtime)
         model_context = getattr(spec.config, "max_position_embeddings", None)
         limit = max_context if max_context is not None else model_context
@@ -81,20 +83,23 @@ class Engine:
         """From a folder with config.json and model.safetensors (or shards with an index)."""
         config = load_config(folder)
         spec = architecture(config.architecture).build(config)
-        device = options.get("device", "cuda:0")
-        tensors = load_tensors(folder, spec.weight_specs(), spec.ignored_names(), device=device)
+        tensors = CheckpointSource(folder, spec.weight_specs(), spec.ignored_names())
         return cls(spec, tensors, dtype=dtype, **options)
 
     @classmethod
-    def random(cls, config, seed: int = 0, dtype="bfloat16", std: float = 0.02, **options) -> "Engine":
-        """With random weights made on the device; no file is written."""
+    def random(cls, config, seed: int = 0, dtype="bfloat16", std: float = 0.02, gain_std: float = 0.0,
+               **options) -> "Engine":
+        """With random weights made on the device; no file is written. The values are those of the folder
+        that `write_random_model` writes for the same configuration, seed and deviations, in the compute
+        dtype (`get_tensor` makes them again on the host)."""
         spec = architecture(config.architecture).build(config)
         device = options.get("device", "cuda:0")
-        stored = torch.bfloat16 if compute_dtype(dtype) == torch.bfloat16 else torch.float32
-        engine = cls.__new__(cls)
-        tensors = LazyRandom(spec.weight_specs(), seed, std, stored, device)
-        cls.__init__(engine, spec, tensors, dtype=dtype, **options)
-        return engine
+        ops = options.get("ops")
+        if ops is None:
+            from ..ops import load_ops
+            ops = options["ops"] = load_ops()
+        tensors = RandomSource(spec.weight_specs(), seed, std, compute_dtype(dtype), device, ops, gain_std)
+        return cls(spec, tensors, dtype=dtype, **options)
 
     # -- slots -------------------------------------------------------------------
     def alloc_slot(self) -> int:
@@ -128,6 +133,8 @@ class Engine:
         on the host: what a reference computation outside this library needs."""
         if name not in self.tensors:
             raise KeyError(f"no tensor named '{name}'")
+        if hasattr(self.tensors, "host"):
+            return self.tensors.host(name)
         return self.tensors[name].detach().to("cpu")
 
     # -- the step ----------------------------------------------------------------
@@ -218,21 +225,3 @@ class Engine:
             raise StepError(f"the cache cannot hold this step: {error}") from None
         self.cache.sync()
         return slots, tokens, wants, starts
-
-
-class LazyRandom(dict):
-    """Random tensors by name, each made on the device when a part asks for it."""
-
-    def __init__(self, specs, seed, std, dtype, device):
-        super().__init__()
-        self._specs = specs
-        self._index = {name: i for i, name in enumerate(specs)}
-        self._args = (seed, std, dtype, device)
-
-    def __missing__(self, name):
-        from ..weights.random_init import _make
-        seed, std, dtype, device = self._args
-        return _make(self._specs[name], seed, self._index[name], std, dtype, device)
-
-    def __contains__(self, name):
-        return name in self._specs

@@ -82,7 +82,7 @@ class HipOps:
         self.path = path
         self.lib.xrt_last_error.restype = ctypes.c_char_p
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
-                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv"):
+                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv", "xrt_random_normal"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
         self.lib.xrt_sample_workspace.restype = ctypes.c_long
@@ -118,6 +118,13 @@ class HipOps:
         self._require(out, "embed out", torch.float32, (tokens, hidden), table)
         self._check(self.lib.xrt_embed(_ptr(table), _code(table), _ptr(ids), _ptr(out), tokens, hidden, vocab,
                                        self._stream(out)))
+
+    def random_normal(self, out, key: int, scale: float, offset: float = 0.0):
+        """out[i] = element i of the random-weights stream `key` (weights/random_init.py), times scale, plus offset."""
+        self._require(out, "random_normal out")
+        self._check(self.lib.xrt_random_normal(_ptr(out), _code(out), ctypes.c_long(out.numel()),
+                                               ctypes.c_ulonglong(key & ((1 << 64) - 1)), ctypes.c_float(scale),
+                                               ctypes.c_float(offset), self._stream(out)))
 
     def add(self, residual, delta):
         self._require(residual, "add residual", torch.float32)

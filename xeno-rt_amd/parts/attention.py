@@ -74,9 +74,7 @@ class Attention(Mixer):
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         p = self.prefix
-        self.w_qkv = torch.cat([runtime.matrix(tensors[p + name])
-                                for name in ("q_proj.weight", "k_proj.weight", "v_proj.weight")],
-                               dim=0).contiguous()
+        self.w_qkv = runtime.stacked(tensors[p + name] for name in ("q_proj.weight", "k_proj.weight", "v_proj.weight"))
         self.w_o = runtime.matrix(tensors[p + "o_proj.weight"])
         if self.qk_norm:
             self.q_norm = runtime.vector(tensors[p + "q_norm.weight"])

@@ -70,14 +70,34 @@ class Runtime:
         self.device = torch.device(device)
 
     def matrix(self, tensor: torch.Tensor) -> torch.Tensor:
-        """A weight matrix in the compute dtype, contiguous, on the device."""
+        """A weight matrix in the compute dtype, contiguous, on the device. A tensor that comes from the
+        host in another type is converted there, so that the device never holds it twice."""
+        if tensor.device != self.device and tensor.dtype != self.dtype:
+            tensor = tensor.to(self.dtype)
         return tensor.to(device=self.device, dtype=self.dtype).contiguous()
 
+    def stacked(self, tensors) -> torch.Tensor:
+        """Matrices of equal width one below the other, as one matrix in the compute dtype on the device:
+        allocated once, each piece copied into its rows."""
+        tensors = list(tensors)
+        width = tensors[0].shape[1]
+        if any(t.dim() != 2 or t.shape[1] != width for t in tensors):
+            raise ValueError(f"stacked matrices need one width, found {[tuple(t.shape) for t in tensors]}")
+        out = torch.empty((sum(t.shape[0] for t in tensors), width), dtype=self.dtype, device=self.device)
+        at = 0
+        for tensor in tensors:
+            if tensor.device != self.device and tensor.dtype != self.dtype:
+                tensor = tensor.to(self.dtype)
+            out[at:at + tensor.shape[0]].copy_(tensor)
+            at += tensor.shape[0]
+        return out
+
     def vector(self, tensor: torch.Tensor) -> torch.Tensor:
-        """A small float vector: float32 on the 32-bit path, else as the file stores it."""
-        if self.dtype == torch.float32 or tensor.dtype == torch.float32:
-            return tensor.to(device=self.device, dtype=torch.float32).contiguous()
-        return tensor.to(device=self.device, dtype=torch.bfloat16).contiguous()
+        """A small float vector: bfloat16 if the file stores it so and the model computes in bfloat16,
+        float32 otherwise (a float16 vector widens exactly)."""
+        if self.dtype == torch.bfloat16 and tensor.dtype == torch.bfloat16:
+            return tensor.to(device=self.device).contiguous()
+        return tensor.to(device=self.device, dtype=torch.float32).contiguous()
 
     def empty(self, shape, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)

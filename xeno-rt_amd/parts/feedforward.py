@@ -42,8 +42,7 @@ class GatedMLP(FeedForward):
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         p = self.prefix
-        self.w_gate_up = torch.cat([runtime.matrix(tensors[p + "gate_proj.weight"]),
-                                    runtime.matrix(tensors[p + "up_proj.weight"])], dim=0).contiguous()
+        self.w_gate_up = runtime.stacked(tensors[p + name] for name in ("gate_proj.weight", "up_proj.weight"))
         self.w_down = runtime.matrix(tensors[p + "down_proj.weight"])
 
     def forward(self, h, batch, residual: torch.Tensor, then=None):

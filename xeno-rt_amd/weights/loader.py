@@ -5,9 +5,15 @@ first that is missing (crates/xrt-models/src/llama.rs:286-337,
 crates/xrt-gguf/src/lib.rs:532-541). Here the whole set is compared at once:
 one error lists the missing tensors, the unexpected ones and the wrong shapes.
 
-Kept precision: BF16 and F16 tensors are held as bfloat16, F32 tensors stay
-float32, integer tables become int32. Conversion to the compute dtype is the
-business of the part that binds the tensor.
+Kept precision: tensors are handed on as the file stores them (BF16, F16, F32;
+64-bit integer tables become int32). Conversion to the compute dtype is the
+business of the part that binds the tensor, so that the 32-bit path widens an
+F16 checkpoint exactly and only the bfloat16 path rounds it.
+
+`CheckpointSource` hands out one tensor at a time, read from the mapped file
+when a part asks for it and kept by nobody: a model's weights are on the device
+once, in the form the parts bound them, and `Engine.get_tensor` reads the file
+again.
 """
 from __future__ import annotations
 
@@ -48,8 +54,6 @@ _INTEGER = ("I32", "I64")
 
 
 def _kept(tensor: torch.Tensor) -> torch.Tensor:
-    if tensor.dtype == torch.float16:
-        return tensor.to(torch.bfloat16)
     if tensor.dtype == torch.int64:
         if tensor.numel() and (int(tensor.max()) > 2**31 - 1 or int(tensor.min()) < -2**31):
             raise SafetensorsError("integer table does not fit int32")
@@ -111,6 +115,41 @@ def check_names(where: str, expected: Dict[str, WeightSpec], found: Dict[str, tu
             wrong_dtype.append((name, spec.kind, dtype, "/".join(_FLOAT)))
     if missing or unexpected or wrong_shape or wrong_dtype:
         raise WeightError(where, missing, unexpected, wrong_shape, wrong_dtype)
+
+
+class CheckpointSource:
+    """The tensors of a model folder by name, each read when it is asked for (on the host, as stored).
+
+    The whole set of names, shapes and dtypes is checked against `expected` when the source is made."""
+
+    def __init__(self, folder: str, expected: Dict[str, WeightSpec], ignored: Iterable[str] = ()):
+        self.folder = folder
+        self.expected = dict(expected)
+        self.files = CheckpointFiles(folder)
+        try:
+            found = {name: (file.entries[name].dtype, file.entries[name].shape)
+                     for name, file in self.files.where.items()}
+            check_names(folder, self.expected, found, ignored)
+        except Exception:
+            self.files.close()
+            raise
+
+    def __contains__(self, name: str) -> bool:
+        return name in self.expected
+
+    def keys(self):
+        return self.expected.keys()
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        if name not in self.expected:
+            raise KeyError(name)
+        return _kept(self.files.where[name].read(name))
+
+    def host(self, name: str) -> torch.Tensor:
+        return self[name]
+
+    def close(self) -> None:
+        self.files.close()
 
 
 def load_tensors(folder: str, expected: Dict[str, WeightSpec], ignored: Iterable[str] = (),
