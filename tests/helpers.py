@@ -8,7 +8,10 @@ import torch
 #   bfloat16: activations are rounded to 8 bits (2^-9 relative) about six times per layer;
 #            with the tests' weights (std 0.2: sharp attention, gains above one) that comes
 #            to one or two percent of the largest logit. The root-mean-square bound is
-#            tighter because it does not ride on the single worst element.
+#            tighter because it does not ride on the single worst element. Largest errors seen over all
+#            tests (printed at the end of every run): max 3.4e-2, rms 7.0e-3 with the tiny models' weights
+#            of std 0.2; max 1.5e-2, rms 2.9e-3 at real layer sizes with std 0.02. The limits are
+#            1.5 and 2 times the former.
 TOLERANCE = {"float32": dict(max=2e-5, rms=5e-6), "bfloat16": dict(max=5e-2, rms=1.5e-2)}
 
 

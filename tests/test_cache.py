@@ -105,6 +105,24 @@ def test_groups_with_a_window_keep_only_what_is_still_seen():
     assert ring.pool.n_held == 0 and full.pool.n_held == 0
 
 
+def test_truncation_below_what_a_window_has_released_is_refused():
+    needs = [CacheNeeds(kv=KVSpec(2, 16, window=100))]
+    cache = SequenceCache(needs, [0], 1024, 2, 1024, torch.float32, "cpu")
+    ring = cache.groups[0]
+    a = cache.alloc_slot()
+    cache.reserve(a, 600); cache.commit(a, 600)           # a query at 600 sees keys 501..: blocks 0..6 are gone
+    held = ring.pool.n_held
+    with pytest.raises(CacheError, match="released"):
+        cache.truncate(a, 300)                            # a query at 300 would see keys 201..299: released long ago
+    assert cache.length(a) == 600 and ring.pool.n_held == held
+    cache.truncate(a, 590)                                # a query at 590 sees keys 491..: block 7 is still held
+    assert cache.length(a) == 590
+    cache.reserve(a, 591); cache.commit(a, 591)
+    cache.check()
+    cache.free_slot(a)
+    assert ring.pool.n_held == 0
+
+
 def test_state_is_zero_for_every_new_sequence():
     cache = make_cache(state=True)
     a = cache.alloc_slot()

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from conftest import TINY, make_folder
-from helpers import (TOLERANCE, assert_logits, first_bad_position, run_batched, run_tail_decoded, run_whole,
+from helpers import (TOLERANCE, assert_logits, errors, first_bad_position, run_batched, run_tail_decoded, run_whole,
                      token_ids)
 import plain_llama as P
 
@@ -149,13 +149,26 @@ def test_greedy_generation_through_the_entry_point(name, dtype, models, engines)
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_far_keys_among_hundreds(dtype, tmp_path):
     """Several hundred tokens of context with weights that make attention sharp: the keys that
-    matter lie far back, in other cache blocks than the query."""
+    matter lie far back, in other cache blocks than the query.
+
+    Weights this sharp (std 0.3) turn the rounding of q and k to bfloat16 into errors of up to 6 % of
+    the largest logit, whatever computes them: the stand-in for the kernels, which rounds where they
+    round and otherwise computes in float32 on the host, is as far from the plain model as the kernels
+    are. The bfloat16 engine is therefore compared with that stand-in (a key that is missed or read from
+    the wrong block moves logits by far more than the orders of summation do), the 32-bit engine with
+    the plain model."""
+    from ops_emulation import EmulatedOps
     from xeno_rt_amd.engine import Engine
     raw = dict(TINY["llama"], max_position_embeddings=1024, num_hidden_layers=1, rope_theta=50000.0)
     folder = make_folder(raw, tmp_path / "far", seed=5, std=0.3)
     plain = P.PlainModel(folder)
     ids = token_ids(plain.config.vocab_size, 700, seed=3)
     want = plain.logits(ids)
+    if dtype == "bfloat16":
+        rounded = run_whole(Engine.load(folder, dtype=dtype, max_tokens=1024, device="cpu", ops=EmulatedOps()), ids)
+        worst, rms = errors(rounded, want)
+        assert worst < 0.1 and rms < 0.01, "the stand-in itself is off"
+        want = rounded
     engine = Engine.load(folder, dtype=dtype, max_tokens=1024)
     assert_logits(run_whole(engine, ids), want, dtype, "700 tokens whole")
     got = run_tail_decoded(engine, ids)
@@ -196,6 +209,61 @@ def test_replayed_decode_steps_equal_direct_ones(dtype, models):
     assert len(recorded.graphs.graphs) >= 2
     for index, (a, b) in enumerate(zip(*outputs)):
         assert torch.equal(a, b), f"step {index}: a replayed graph differs from the direct step"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_recorded_steps_share_memory_and_make_room_for_each_other(dtype, models, monkeypatch):
+    """All recorded steps draw on one memory pool and at most MAX_GRAPHS are kept: steps of three
+    shapes taken in turn (each replay between replays of the others, each shape recorded again after
+    it had to make room) give the bits of direct steps."""
+    from xeno_rt_amd.engine import Engine, graphs
+    monkeypatch.setattr(graphs, "MAX_GRAPHS", 2)
+    folder, plain, _ = models["llama"]
+    vocab = plain.config.vocab_size
+    recorded = Engine.load(folder, dtype=dtype, max_tokens=64 * 16, max_slots=8)
+    direct = Engine.load(folder, dtype=dtype, max_tokens=64 * 16, max_slots=8, graphs=False)
+    outputs = []
+    for engine in (recorded, direct):
+        rows = []
+        slots = [engine.alloc_slot() for _ in range(7)]
+        engine.step([(slot, token_ids(vocab, 5 + 9 * i, seed=i), []) for i, slot in enumerate(slots)])
+        for step in range(24):
+            live = slots[:(1, 3, 7)[step % 3]]                   # batch buckets 1, 4 and 8 in turn
+            tokens = token_ids(vocab, len(live), seed=300 + step)
+            rows.append(engine.step([(slot, [token], [0]) for slot, token in zip(live, tokens)]))
+        for slot in slots:
+            engine.free_slot(slot)
+        outputs.append(rows)
+    assert len(recorded.graphs.graphs) == 2
+    for index, (a, b) in enumerate(zip(*outputs)):
+        assert torch.equal(a, b), f"step {index}: a replayed graph differs from the direct step"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["llama", "qwen3"])
+def test_a_step_may_mix_sequences_that_start_with_sequences_that_go_on(name, dtype, models, engines):
+    """One step with a whole prompt of a new sequence, one token of a sequence under way, and several
+    tokens of another one under way (its start not on a block's boundary)."""
+    engine = engines(name, dtype)
+    _, plain, cases = models[name]
+    lengths = LENGTHS[name]
+    a, b, c = (cases[n] for n in (lengths[3], lengths[4], lengths[5]))     # (ids, plain logits)
+    slots = [engine.alloc_slot() for _ in range(3)]
+    cut_b, cut_c = len(b[0]) - 1, len(c[0]) - 37
+    first = engine.step([(slots[1], b[0][:cut_b], list(range(cut_b))), (slots[2], c[0][:cut_c], list(range(cut_c)))])
+    mixed = engine.step([(slots[0], a[0], list(range(len(a[0])))),
+                         (slots[1], b[0][cut_b:], [0]),
+                         (slots[2], c[0][cut_c:], list(range(37)))])
+    for slot in slots:
+        engine.free_slot(slot)
+    got_a = mixed[:len(a[0])]
+    got_b = torch.cat([first[:cut_b], mixed[len(a[0]):len(a[0]) + 1]])
+    got_c = torch.cat([first[cut_b:], mixed[len(a[0]) + 1:]])
+    for what, got, (ids, want) in (("starting", got_a, a), ("one more token", got_b, b), ("37 more tokens", got_c, c)):
+        assert_logits(got, want, dtype, f"{name} mixed step, the sequence {what}, first bad row {first_bad_position(got, want, dtype)}")
+        if dtype == "float32":
+            assert torch.equal(got, run_whole(engine, ids)), f"{name}: a mixed step changed float32 bits ({what})"
+    engine.cache.check()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -235,6 +235,11 @@ class SequenceCache:
             raise CacheError(f"slot {slot}: cannot truncate {self.lengths[slot]} tokens to {length}")
         if self.states and length != self.lengths[slot]:
             raise CacheError("a cache with per-sequence state cannot be truncated")
+        for group in self.groups:
+            # a window has let go of the blocks below its floor: a shorter sequence that would look there again cannot be had
+            if group.spec.window is not None and group.first_needed_block(length) < group._floor.get(slot, 0):
+                raise CacheError(f"slot {slot}: cannot truncate to {length} tokens: a window of {group.spec.window} has "
+                                 f"released the keys before {group._floor[slot] * BLOCK_TOKENS}, which a query there would see")
         self.lengths[slot] = length
         for group in self.groups:
             group.shrink_to(slot, length)

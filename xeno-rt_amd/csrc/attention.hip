@@ -10,6 +10,7 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
                           int window, hipStream_t s);
 bool xrt_attention_decode_accepts(int head_dim);
+long xrt_attention_decode_workspace(int tokens, int n_heads, int n_kv_heads, int head_dim, int max_context);
 int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
                          const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                          const int* positions, const int* slots, void* out, float scale, int max_context,
@@ -19,6 +20,17 @@ int xrt_attention_prefill(const void* qkv, int tokens, int n_heads, int n_kv_hea
                           const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                           const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
                           float scale, hipStream_t s);
+
+static bool takes_decode_kernel(int dtype, int n_heads, int n_kv_heads, int head_dim, int window, int max_count, int max_context) {
+    return dtype == XRT_BF16 && window == 0 && max_count == 1 && max_context > 0 && n_heads > 0 && n_kv_heads > 0 &&
+           n_heads % n_kv_heads == 0 && xrt_attention_decode_accepts(head_dim);
+}
+
+extern "C" long xrt_attention_workspace(int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int window,
+                                        int max_count, int max_context) {
+    if (tokens <= 0 || !takes_decode_kernel(dtype, n_heads, n_kv_heads, head_dim, window, max_count, max_context)) return 0;
+    return xrt_attention_decode_workspace(tokens, n_heads, n_kv_heads, head_dim, max_context);
+}
 
 extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                              const void* k_cache, const void* v_cache, const int* block_table,
@@ -37,7 +49,9 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
     hipStream_t s = (hipStream_t)stream;
     const bool described = seq_offsets && seq_slots && seq_starts && n_seqs > 0 && max_count > 0 && max_context > 0;
     if (dtype == XRT_BF16 && window == 0 && described) {
-        if (max_count == 1 && workspace != nullptr && xrt_attention_decode_accepts(head_dim))
+        const long need = xrt_attention_workspace(dtype, tokens, n_heads, n_kv_heads, head_dim, window, max_count, max_context);
+        if (takes_decode_kernel(dtype, n_heads, n_kv_heads, head_dim, window, max_count, max_context) &&
+            (need == 0 || (workspace != nullptr && workspace_floats >= need)))
             return xrt_attention_decode(qkv, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
                                         table_stride, n_blocks, positions, slots, out, scale, max_context, workspace,
                                         workspace_floats, s);

@@ -313,8 +313,8 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
     const int group = n_heads / n_kv_heads;
     const int q_tiles = (group + 15) / 16;
     const Cut cut = cut_for(tokens, n_kv_heads, q_tiles, max_context, HD);
-    const long need = (long)tokens * n_heads * cut.n_parts * (HD + 2);
-    XRT_REQUIRE(workspace != nullptr && workspace_floats >= need,
+    const long need = cut.n_parts == 1 ? 0 : (long)tokens * n_heads * cut.n_parts * (HD + 2);
+    XRT_REQUIRE(need == 0 || (workspace != nullptr && workspace_floats >= need),
                 "attention (decode): workspace of %ld floats given, %ld needed", workspace_floats, need);
     float* part_o = workspace;
     float* part_ml = workspace + (long)tokens * n_heads * cut.n_parts * HD;
@@ -337,10 +337,12 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
 
 bool xrt_attention_decode_accepts(int head_dim) { return head_dim == 64 || head_dim == 128; }
 
-// floats of workspace that a decode step of `tokens` sequences may need
+// floats of workspace that a decode step of `tokens` sequences needs: the partial results of the cut that
+// the launcher will choose (none where one workgroup sees all keys of a sequence)
 long xrt_attention_decode_workspace(int tokens, int n_heads, int n_kv_heads, int head_dim, int max_context) {
-    const int max_blocks = (max_context + XRT_BLOCK_TOKENS - 1) / XRT_BLOCK_TOKENS;
-    return (long)tokens * n_heads * max_blocks * (head_dim + 2);     // chunks of one block: the most there can be
+    const int q_tiles = (n_heads / n_kv_heads + 15) / 16;
+    const Cut cut = cut_for(tokens, n_kv_heads, q_tiles, max_context, head_dim);
+    return cut.n_parts == 1 ? 0 : (long)tokens * n_heads * cut.n_parts * (head_dim + 2);
 }
 
 int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,

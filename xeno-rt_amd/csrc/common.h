@@ -96,12 +96,12 @@ __device__ __forceinline__ long cache_block_base(const int* block_table, int tab
 // compiler, when it knows of such a load, waits for all of them at every barrier.
 __device__ __forceinline__ void load_to_lds(const void* base, unsigned byte_offset, unsigned lds_base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_base), "v"(byte_offset), "s"(base) : "memory");
+                 :: "s"(lds_base), "v"(byte_offset), "s"(base) : "memory", "m0");
 }
 // The same with 4 bytes per lane: lane l writes LDS byte address lds_base + 4 * l.
 __device__ __forceinline__ void load_dword_to_lds(const void* base, unsigned byte_offset, unsigned lds_base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-                 :: "s"(lds_base), "v"(byte_offset), "s"(base) : "memory");
+                 :: "s"(lds_base), "v"(byte_offset), "s"(base) : "memory", "m0");
 }
 // Waits until at most `pending` of this wavefront's loads (the newest ones) are outstanding and
 // its LDS reads are done, then meets the workgroup's other wavefronts. __syncthreads() cannot

@@ -86,8 +86,11 @@ int xrt_linear_qkv(const void* a, const void* w, int dtype, void* qkv, int M, in
 
 // causal attention of every token of a step over its sequence's cache. The sequences of the
 // step may be described (seq_* arrays, n_seqs, the largest token count of a sequence and the
-// longest sequence after the step): then the matrix-core kernels can be used; decode needs a
-// workspace of tokens * n_heads * ceil(max_context / 64) * (head_dim + 2) floats.
+// longest sequence after the step): then the matrix-core kernels can be used; a decode step (max_count 1)
+// then needs a workspace of xrt_attention_workspace(...) floats for the partial results of the parts that
+// its keys are cut into (0: none), and takes the general kernel without it.
+long xrt_attention_workspace(int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int window,
+                             int max_count, int max_context);
 int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                   const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                   int n_blocks, const int* positions, const int* slots, void* out, float scale, int window,

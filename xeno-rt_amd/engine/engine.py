@@ -142,8 +142,8 @@ class Engine:
         """Run the next tokens of some sequences; return logits [wanted, vocab] (float32, on the device).
 
         entries: (slot, tokens, want) per sequence; `want` are indices into `tokens`, in the order
-        in which their logits are returned (entries first, then want). The sequences of a step either
-        all start (length 0) or all continue; their token counts may differ.
+        in which their logits are returned (entries first, then want). The sequences of a step may
+        start (length 0) or continue, with any token counts, in any mixture.
         """
         slots, tokens, wants, starts = self.prepare(entries)
         try:

@@ -6,6 +6,11 @@ bring one token has a fixed shape once its batch size and the longest context ar
 rounded up to buckets, so its kernels are captured once per bucket and replayed with
 new contents in the same buffers. Sequences that fill a bucket up are padding (slot -1):
 computed, cached nowhere, read by nothing.
+
+All recorded steps take their buffers from one memory pool: the steps are replayed one after
+another, never at once, so what one used for its activations serves the next, and only the
+inputs and logits of each stay its own. At most MAX_GRAPHS steps are kept; the one replayed
+longest ago makes room.
 """
 from __future__ import annotations
 
@@ -17,6 +22,7 @@ from ..staging import staging_for
 from .batch import StepBatch
 
 CONTEXT_BUCKET = 1024
+MAX_GRAPHS = 32
 
 
 def batch_bucket(count: int) -> int:
@@ -35,7 +41,7 @@ def context_bucket(length: int, limit: int) -> int:
 class DecodeGraph:
     """One captured decode step for `size` sequences whose contexts reach at most `context`."""
 
-    def __init__(self, model, cache, size: int, context: int, device):
+    def __init__(self, model, cache, size: int, context: int, device, pool=None):
         self.size = size
         self.context = context
         self.device = device
@@ -62,7 +68,7 @@ class DecodeGraph:
         torch.cuda.current_stream(device).wait_stream(stream)
         torch.cuda.synchronize(device)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with torch.cuda.graph(self.graph, pool=pool):
             self.logits = model.forward(self.batch, cache)
 
     def fill(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int], source=None) -> None:
@@ -89,7 +95,8 @@ class DecodeGraphs:
         self.model = model
         self.cache = cache
         self.device = device
-        self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}
+        self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}       # in the order of their last use
+        self.pool = torch.cuda.graph_pool_handle() if torch.device(device).type == "cuda" else None
 
     def step(self, slots: List[int], tokens: List[int], starts: List[int], source=None) -> torch.Tensor:
         """Logits [len(slots), vocab] of one decode step; a copy, valid until the caller drops it.
@@ -97,6 +104,10 @@ class DecodeGraphs:
         size = batch_bucket(len(slots))
         context = context_bucket(max(starts) + 1, self.cache.max_context)
         key = (size, context)
-        if key not in self.graphs:
-            self.graphs[key] = DecodeGraph(self.model, self.cache, size, context, self.device)
-        return self.graphs[key].run(slots, tokens, starts, source)[:len(slots)].clone()
+        graph = self.graphs.pop(key, None)
+        if graph is None:
+            while len(self.graphs) >= MAX_GRAPHS:
+                del self.graphs[next(iter(self.graphs))]
+            graph = DecodeGraph(self.model, self.cache, size, context, self.device, self.pool)
+        self.graphs[key] = graph
+        return graph.run(slots, tokens, starts, source)[:len(slots)].clone()

@@ -85,6 +85,7 @@ class HipOps:
                      "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv", "xrt_random_normal"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
+        self.lib.xrt_attention_workspace.restype = ctypes.c_long
         self.lib.xrt_sample_workspace.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
@@ -290,9 +291,9 @@ class HipOps:
             self._require(starts, "sequence starts", torch.int32, (n_seqs,), qkv)
             if max_context > stride * BLOCK_TOKENS:
                 raise KernelError(f"attention: a sequence of {max_context} tokens exceeds the block table")
-            if max_count == 1 and qkv.dtype == torch.bfloat16 and not window:
-                blocks = (max_context + BLOCK_TOKENS - 1) // BLOCK_TOKENS
-                workspace_floats = tokens * n_heads * blocks * (head_dim + 2)
+            workspace_floats = int(self.lib.xrt_attention_workspace(_code(qkv), tokens, n_heads, n_kv_heads, head_dim,
+                                                                    int(window or 0), max_count, max_context))
+            if workspace_floats > 0:
                 workspace = torch.empty(workspace_floats, dtype=torch.float32, device=qkv.device)
         self._check(self.lib.xrt_attention(
             _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(k_cache), _ptr(v_cache),
