@@ -86,6 +86,7 @@ class HipOps:
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
         self.lib.xrt_attention_workspace.restype = ctypes.c_long
+        self.lib.xrt_probe_read_bytes.restype = ctypes.c_long
         self.lib.xrt_sample_workspace.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
@@ -126,6 +127,21 @@ class HipOps:
         self._check(self.lib.xrt_random_normal(_ptr(out), _code(out), ctypes.c_long(out.numel()),
                                                ctypes.c_ulonglong(key & ((1 << 64) - 1)), ctypes.c_float(scale),
                                                ctypes.c_float(offset), self._stream(out)))
+
+    def probe_read(self, buffer, nontemporal: bool = False) -> int:
+        """Read `buffer` once and write nothing; returns the bytes read (a little under the buffer's size)."""
+        self._require(buffer, "probe buffer")
+        sink = torch.zeros(1, dtype=torch.int32, device=buffer.device)
+        size = buffer.numel() * buffer.element_size()
+        self._check(self.lib.xrt_probe_read(_ptr(buffer), ctypes.c_long(size), int(nontemporal), _ptr(sink),
+                                            self._stream(buffer)))
+        return int(self.lib.xrt_probe_read_bytes(ctypes.c_long(size)))
+
+    def probe_mfma(self, iterations: int, device) -> int:
+        """Matrix-core products on tiles held in registers; returns the flops done."""
+        sink = torch.zeros(1, dtype=torch.float32, device=device)
+        self._check(self.lib.xrt_probe_mfma(ctypes.c_long(iterations), _ptr(sink), self._stream(sink)))
+        return 512 * 4 * iterations * 4 * 2 * 32 * 32 * 16
 
     def add(self, residual, delta):
         self._require(residual, "add residual", torch.float32)
