@@ -47,6 +47,11 @@ def first_bad_position(got, want, dtype):
     return None
 
 
+def plain_matrix(weight):
+    """A bound weight as a matrix with rows contiguous along k, whichever layout the kernels keep it in."""
+    return weight.unpacked() if hasattr(weight, "unpacked") else weight
+
+
 def token_ids(vocab, length, seed):
     return torch.randint(0, vocab, (length,), generator=torch.Generator().manual_seed(seed)).tolist()
 

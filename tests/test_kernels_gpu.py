@@ -33,6 +33,15 @@ def rand(*shape, dtype=torch.float32, seed=0, scale=1.0):
     return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
 
 
+def packed_or_not(ops, w, packed, kind="tiles", **details):
+    """w as the products take it: as it is, or in the tiled layout (bfloat16, k a multiple of 32)."""
+    if not packed:
+        return w
+    if w.dtype != torch.bfloat16 or w.shape[1] % 32 != 0:
+        pytest.skip("only bfloat16 matrices whose k is a multiple of 32 are packed")
+    return ops.pack(w, kind, **details)
+
+
 def rel(got, want):
     return float((got.double() - want.double()).abs().max()) / max(1e-30, float(want.double().abs().max()))
 
@@ -85,12 +94,14 @@ SHAPES = [(1, 64, 64), (3, 200, 96), (8, 1000, 176), (17, 96, 192), (64, 333, 52
           (2100, 8300, 128), (40, 4100, 1024), (64, 333, 640), (33, 130, 128), (17, 700, 192)]
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16 packed"])
 @pytest.mark.parametrize("m,n,k", SHAPES)
 def test_linear(ops, dtype, m, n, k):
+    dtype, packed = dtype.split()[0], dtype.endswith("packed")
     a = rand(m, k, dtype=DT[dtype], seed=m)
     w = rand(n, k, dtype=DT[dtype], seed=n, scale=0.1)
     want = a.double().cpu() @ w.double().cpu().t()
+    w = packed_or_not(ops, w, packed)
     out32 = torch.empty(m, n, device=DEV)
     ops.linear(a, w, out32)
     assert rel(out32.cpu(), want) < 1e-5                        # float32 accumulation in both paths
@@ -103,17 +114,22 @@ def test_linear(ops, dtype, m, n, k):
     assert rel(acc.cpu(), base.double().cpu() + want) < 1e-5
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16 packed"])
 @pytest.mark.parametrize("m,n,k", [(1, 176, 64), (9, 100, 96), (64, 520, 200), (200, 1000, 72), (48, 2000, 520),
+                                   (3, 8, 32), (16, 24, 160), (30, 1000, 96), (64, 4104, 224), (8, 14336, 4096),
                                    (2048, 3100, 64), (300, 130, 1032), (2048, 3072, 128), (2000, 3000, 192), (2048, 4224, 64),
                                    (64, 520, 256), (50, 1000, 1024), (200, 1000, 512),
                                    # 17 to 64 rows and tiles enough without a split along k
                                    (40, 14336, 256), (64, 9002, 128), (33, 20000, 192)])
 def test_linear_glu(ops, dtype, m, n, k):
+    dtype, packed = dtype.split()[0], dtype.endswith("packed")
+    if packed and n % 8 != 0:
+        pytest.skip("gate and up rows are paired in groups of 8")
     a = rand(m, k, dtype=DT[dtype], seed=1)
     w = rand(2 * n, k, dtype=DT[dtype], seed=2, scale=0.3)
     both = a.double().cpu() @ w.double().cpu().t()
     want = P.swiglu(both[:, :n], both[:, n:])
+    w = packed_or_not(ops, w, packed, "gated", gated_n=n)
     out = torch.empty(m, n, dtype=DT[dtype], device=DEV)
     ops.linear_glu(a, w, out)
     assert rel(out.cpu(), want) < ULP[dtype] * 2
@@ -160,7 +176,8 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
 @pytest.mark.parametrize("m,hidden,k,n", [(1, 4096, 512, 1024), (8, 4096, 14336, 6144), (16, 200, 96, 72),
                                           (5, 1000, 136, 333), (13, 8200, 64, 48),
                                           (17, 4096, 512, 1024), (40, 1024, 256, 333), (64, 4096, 14336, 6144), (33, 512, 128, 20000)])
-def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n):
+@pytest.mark.parametrize("packed", [False, True])
+def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n, packed):
     # x += a w^T; y = rmsnorm(x) * gain; z = y v^T (and the gated pair), the norm without a kernel of its own:
     # up to 16 rows in the kernel that streams w, 17 to 64 rows in the tiles split along k and their second kernel
     a = rand(m, k, dtype=torch.bfloat16, seed=1)
@@ -172,8 +189,17 @@ def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n):
     eps = 1e-3
     fresh = x.double().cpu() + a.double().cpu() @ w.double().cpu().t()
     normed = P.rmsnorm(fresh, gain.double().cpu(), eps)
+    plain_v = v
+    if packed and (hidden % 32 != 0 or n % 8 != 0):
+        pytest.skip("sizes that are not packed")
+    w = packed_or_not(ops, w, packed)
+    v_glu = packed_or_not(ops, v, packed, "gated", gated_n=n)
+    v = packed_or_not(ops, v, packed)
 
     scaled = ops.linear(a, w, x, accumulate=True, then_norm=(gain, eps))
+    if packed and hidden % 16 != 0 and m <= 16:
+        assert scaled is None                                   # a packed w writes sums of squares per tile of 16 columns
+        return
     assert scaled is not None and scaled.shape == (m, hidden)
     assert rel(x.cpu(), fresh) < 1e-5
     tiles = scaled.squares.shape[0]                 # the product cuts its columns into tiles of 16 or fewer, all alike
@@ -184,20 +210,21 @@ def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n):
     assert rel(scaled.squares[:, :m].t().cpu(), padded.reshape(m, tiles, width).sum(-1)) < 1e-6
     assert rel(scaled.values.cpu(), x.double().cpu() * gain.double().cpu()) < ULP["bfloat16"]
 
-    want = normed @ v.double().cpu().t()
+    want = normed @ plain_v.double().cpu().t()
     for out_dtype in (torch.float32, torch.bfloat16):
         out = torch.empty(m, 2 * n, dtype=out_dtype, device=DEV)
         ops.linear(scaled, v, out)
         # the rows of y are rounded to bfloat16 before the product, by either way of doing the norm
         unfused = torch.empty(m, hidden, dtype=torch.bfloat16, device=DEV)
         ops.rmsnorm(x, gain, eps, unfused)
-        spread = rel(unfused.double().cpu() @ v.double().cpu().t(), want)
+        spread = rel(unfused.double().cpu() @ plain_v.double().cpu().t(), want)
         assert rel(out.cpu(), want) < 2 * spread + ULP["bfloat16" if out_dtype == torch.bfloat16 else "float32"] * 2
     glu = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
-    ops.linear_glu(scaled, v, glu)
+    ops.linear_glu(scaled, v_glu, glu)
     assert rel(glu.cpu(), P.swiglu(want[:, :n], want[:, n:])) < 2e-2
     # and once more into the residual stream, with the norm after it handed on again
-    again = ops.linear(scaled, v[:hidden % 64 + 64], torch.zeros(m, hidden % 64 + 64, device=DEV), accumulate=True,
+    again = ops.linear(scaled, packed_or_not(ops, plain_v[:hidden % 64 + 64].contiguous(), packed),
+                       torch.zeros(m, hidden % 64 + 64, device=DEV), accumulate=True,
                        then_norm=((rand(hidden % 64 + 64, seed=6) + 1.0), eps))
     assert (again is not None) == (m <= 16)                     # 64 to 127 columns: only the kernel for up to 16 rows writes them
 
@@ -310,7 +337,8 @@ def test_qkv_prepare_of_many_tokens(ops, dtype, nh, nkv, hd, rope_dim):
                                                           # adds the partial sums does the rest (the third: two kernels)
                                                           (32, 8, 128, 128, 4096, 40), (4, 2, 64, 64, 256, 17),
                                                           (3, 3, 48, 32, 192, 33), (4, 2, 64, 0, 128, 64), (6, 2, 96, 96, 320, 64)])
-def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens):
+@pytest.mark.parametrize("packed", [False, True])
+def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens, packed):
     """The projection of a short step with the rotation and the cache write in its epilogue, against the two
     kernels one after the other; without a norm before it and with one."""
     positions = ([0, 1, 63, 64, 65, 127, 128, 500, 1000, 2, 3, 4, 5, 6, 7, 8] + list(range(9, 57)))[:tokens]
@@ -331,12 +359,15 @@ def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens):
     scaled = ops.linear(rand(tokens, inner, dtype=torch.bfloat16, seed=5), rand(k, inner, dtype=torch.bfloat16, seed=6), x,
                         accumulate=True, then_norm=(gain, 1e-4))
     assert scaled is not None
+    # packed as the attention part packs it: the pairs of a rotation over whole heads side by side
+    plain_w = w
+    w = packed_or_not(ops, w, packed, "rotary", head_dim=hd, rotated_heads=nh + nkv if rope_dim == hd else 0)
     for rows in (a, scaled):
         got = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
         want = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
         kv_got, kv_want = clone_cache(kv), clone_cache(kv)
         ops.linear_qkv(rows, w, got, nh, nkv, hd, positions, slots, kv=kv_got, **args)
-        ops.linear(rows, w, want)
+        ops.linear(rows, plain_w, want)
         ops.qkv_prepare(want, nh, nkv, hd, positions, slots, kv=kv_want, **args)
         # the same sums, roundings and formulas in both: at most the contraction of a multiply-add may differ
         assert rel(got.float(), want.float()) < ULP["bfloat16"]
@@ -348,7 +379,7 @@ def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens):
     got = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
     want = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
     ops.linear_qkv(a, w, got, nh, nkv, hd, positions, slots, **args)
-    ops.linear(a, w, want)
+    ops.linear(a, plain_w, want)
     ops.qkv_prepare(want, nh, nkv, hd, positions, slots, **args)
     assert rel(got.float(), want.float()) < ULP["bfloat16"]
     qn, kn = rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0
@@ -357,6 +388,10 @@ def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens):
     ops.linear(a, w, want)
     ops.qkv_prepare(want, nh, nkv, hd, positions, slots, q_norm=qn, k_norm=kn, norm_eps=1e-4, kv=kv_want, **args)
     assert torch.equal(got, want) and torch.equal(kv_got.k, kv_want.k) and torch.equal(kv_got.v, kv_want.v)
+    if packed:          # and the packed projection alone against the plain one
+        ops.linear(a, w, want)
+        ops.linear(a, plain_w, got)
+        assert rel(want.float(), got.float()) < ULP["bfloat16"] * 2
 
 
 def test_rope_reference_vector_and_pairing(ops):

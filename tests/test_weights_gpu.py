@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from conftest import TINY, make_folder
-from helpers import assert_logits, run_whole, token_ids
+from helpers import assert_logits, plain_matrix, run_whole, token_ids
 import plain_llama as P
 
 pytestmark = pytest.mark.gpu
@@ -73,7 +73,7 @@ def test_a_loaded_model_holds_every_weight_once(tmp_path):
         assert held - cache_bytes <= 1.02 * factor * file_bytes + (1 << 20), (dtype, held, cache_bytes, file_bytes)
         assert peak - cache_bytes <= 1.05 * factor * file_bytes + (4 << 20), (dtype, peak, file_bytes)
         name = "model.layers.4.self_attn.k_proj.weight"
-        assert torch.equal(engine.get_tensor(name).to(engine.dtype), engine.model.spec.layers[4].mixer.w_qkv[
+        assert torch.equal(engine.get_tensor(name).to(engine.dtype), plain_matrix(engine.model.spec.layers[4].mixer.w_qkv)[
             config.q_width:config.q_width + config.kv_width].cpu())
         del engine
 

@@ -6,6 +6,7 @@
 // same in any batch.
 #include "common.h"
 #include "xrt_hip.h"
+#include "packing.h"
 
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
@@ -14,6 +15,15 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
     const T* row = table + (long)ids[token] * hidden;
     float* dst = out + token * hidden;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]);
+}
+
+// the same from a table kept in tiles (a table that is also the output head's weight)
+__global__ void embed_packed_kernel(const bf16* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ out, int hidden, const Packing packing) {
+    const long token = blockIdx.x;
+    const long row = packed_row(packing, ids[token]);
+    float* dst = out + token * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(table[packed_offset(row, i / 8 * 8, hidden) + i % 8]);
 }
 
 template <typename T>
@@ -82,12 +92,19 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
         dst[i] = from_float<TO>((row[i] * inv_rms) * to_float(weight[i]));
 }
 
-extern "C" int xrt_embed(const void* table, int table_dtype, const int* ids, float* out, int tokens,
+extern "C" int xrt_embed(const void* table, int table_dtype, const xrt_packing* packing, const int* ids, float* out, int tokens,
                          int hidden, int vocab, void* stream) {
     XRT_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes tokens=%d hidden=%d vocab=%d", tokens, hidden, vocab);
     XRT_REQUIRE(table_dtype == XRT_F32 || table_dtype == XRT_BF16, "embed: unknown dtype %d", table_dtype);
     if (tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    if (packing && is_packed(*packing)) {
+        XRT_REQUIRE(packing->kind == XRT_PACK_TILES && table_dtype == XRT_BF16 && hidden % 32 == 0,
+                    "embed: a packed table is bfloat16 in plain tiles with a width that is a multiple of 32");
+        embed_packed_kernel<<<tokens, 256, 0, s>>>((const bf16*)table, ids, out, hidden, *packing);
+        XRT_LAUNCH_CHECK("embed (packed)");
+        return 0;
+    }
     if (table_dtype == XRT_F32)
         embed_kernel<float><<<tokens, 256, 0, s>>>((const float*)table, ids, out, hidden);
     else

@@ -18,8 +18,7 @@
 // them (rows n and n + N of w), arranged so that each wavefront holds both of a pair.
 #include <climits>
 #include <cstdlib>
-#include "common.h"
-#include "xrt_hip.h"
+#include "packing.h"
 #include "gemm_skinny.h"
 
 namespace {
@@ -43,7 +42,7 @@ struct RowScale { const float* squares; int tiles; int width; float eps; };
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __device__ __forceinline__ void gemm_tile(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int id, int tiles_m, int tiles_n, int n_first, int k_per_split, const RowScale scale = RowScale{}) {
+    int id, int tiles_m, int tiles_n, int n_first, int k_per_split, const Packing packing, const RowScale scale = RowScale{}) {
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr int WAVE_M = BM / WM, WAVE_N = BN / WN;        // part of the tile owned by one wavefront
     constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;        // 32x32 accumulator tiles of a wavefront
@@ -149,11 +148,28 @@ __device__ __forceinline__ void gemm_tile(
             const int r = min(i * WAVES + wave, BLOCKS_A - 1) * ROWS + sub;
             off_a[i] = (unsigned)(min(m0 + r, (long)M - 1) * K + chunk_of(r)) * 2u;
         }
+        // A packed w is copied as it lies: an instruction takes one whole tile of the packing (16 packed rows x 32
+        // columns, a contiguous kilobyte, lane by lane), and the stage holds the tile's groups of 16 packed rows
+        // one after another, two tiles of 32 columns each. The 16 lanes that read an operand's 16 rows at one
+        // piece of 8 columns then read 256 contiguous bytes of LDS. (Fetched piece by piece into the layout of
+        // rows contiguous along k, every four lanes would touch four cache lines: a fifth slower, measured.)
+        // The tile's rows are then packed rows first_packed .. + BN, and the epilogue finds the outputs they make.
+        const bool packed_b = is_packed(packing);
+        const long first_packed = MODE == MODE_GATED ? 2 * n0 : n0;
+        const long last_group = ((MODE == MODE_GATED ? 2L * N : (long)N) + 15) / 16 - 1;
 #pragma unroll
         for (int i = 0; i < LOADS_B; ++i) {
-            const int r = min(i * WAVES + wave, BLOCKS_B - 1) * ROWS + sub;
-            off_b[i] = (unsigned)(w_row(r) * K + chunk_of(r)) * 2u;
+            const int block = min(i * WAVES + wave, BLOCKS_B - 1);
+            if (packed_b) {
+                const long group = min(first_packed / 16 + block / 2, last_group);       // groups beyond the matrix: the last one again
+                off_b[i] = (unsigned)(((group * (K / 32) + block % 2) * 512 + lane * 8) * 2);
+            } else {
+                const int r = block * ROWS + sub;
+                off_b[i] = (unsigned)(w_row(r) * K + chunk_of(r)) * 2u;
+            }
         }
+        // a step of k0 columns along k moves a row contiguous along k by k0 elements, a packed one by k0 / 32 tiles
+        const unsigned w_step = packed_b ? 32u : 2u;                // bytes per column of k
         const int wave_uniform = __builtin_amdgcn_readfirstlane(wave);
         const unsigned lds_a0 = lds_address(stage_a), lds_b0 = lds_address(stage_b);
         auto issue = [&](int stage, int k0) {
@@ -165,16 +181,22 @@ __device__ __forceinline__ void gemm_tile(
 #pragma unroll
             for (int i = 0; i < LOADS_B; ++i) {
                 const int block = min(i * WAVES + wave_uniform, BLOCKS_B - 1);
-                load_to_lds(w, off_b[i] + (unsigned)k0 * 2u, lds_b0 + (unsigned)((stage * BN + block * ROWS) * DK * 2));
+                load_to_lds(w, off_b[i] + (unsigned)k0 * w_step, lds_b0 + (unsigned)((stage * BN + block * ROWS) * DK * 2));
             }
         };
         const int swizzle = swizzle_of(lane % 16);                 // of every row this lane reads: they differ by multiples of 32
+        // where this lane finds its piece of the w operand for each slice, from the start of its wavefront's rows
+        int b_place[SLICES];
+#pragma unroll
+        for (int slice = 0; slice < SLICES; ++slice)
+            b_place[slice] = packed_b ? (lane % 32 / 16 * 2 + slice / 2) * 512 + ((slice % 2 * 2 + lane / 32) * 16 + lane % 16) * 8
+                                      : (lane % 32) * DK + ((slice * 2 + lane / 32) ^ swizzle) * 8;
         // operands of one 16-wide slice of k: TM row blocks of a, TN row blocks of w
         struct Operands { bf16x8 a[TM], b[TN]; };
         auto read = [&](Operands& r, int stage, int slice) {
             const int place = ((slice * 2 + lane / 32) ^ swizzle) * 8;
             const bf16* tile_a = stage_a + ((long)stage * BM + wave_m * WAVE_M + lane % 32) * DK + place;
-            const bf16* tile_b = stage_b + ((long)stage * BN + wave_n * WAVE_N + lane % 32) * DK + place;
+            const bf16* tile_b = stage_b + ((long)stage * BN + wave_n * WAVE_N) * DK + b_place[slice];
 #pragma unroll
             for (int i = 0; i < TM; ++i) r.a[i] = *reinterpret_cast<const bf16x8*>(tile_a + i * 32 * DK);
 #pragma unroll
@@ -232,15 +254,16 @@ __device__ __forceinline__ void gemm_tile(
     #pragma unroll
         for (int i = 0; i < CHUNKS_B; ++i) {
             const int chunk = tid + i * THREADS;
-            off_b[i] = (unsigned)(w_row(chunk / 8) * K + (chunk % 8) * 8);
+            off_b[i] = (unsigned)weight_offset(packing, w_row(chunk / 8), (chunk % 8) * 8, K);
         }
+        const unsigned w_step = is_packed(packing) ? 16u : 1u;      // elements per column of k (tiles are 64 wide here: whole tiles of the packing)
 
         struct Stage { bf16x8 a[CHUNKS_A], b[CHUNKS_B]; };
         auto fetch = [&](Stage& stage, int k0) {                  // a whole tile of 64 along k, no guards
     #pragma unroll
             for (int i = 0; i < CHUNKS_A; ++i) stage.a[i] = *reinterpret_cast<const bf16x8*>(a + (off_a[i] + (unsigned)k0));
     #pragma unroll
-            for (int i = 0; i < CHUNKS_B; ++i) stage.b[i] = *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0));
+            for (int i = 0; i < CHUNKS_B; ++i) stage.b[i] = *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0 * w_step));
         };
         auto fetch_tail = [&](Stage& stage, int k0) {             // the last tile when K is no multiple of 64: zeros beyond K
     #pragma unroll
@@ -251,7 +274,7 @@ __device__ __forceinline__ void gemm_tile(
     #pragma unroll
             for (int i = 0; i < CHUNKS_B; ++i) {
                 const int k = k0 + ((tid + i * THREADS) % 8) * 8;
-                stage.b[i] = k + 8 <= K ? *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0)) : bf16x8{};
+                stage.b[i] = k + 8 <= K ? *reinterpret_cast<const bf16x8*>(w + (off_b[i] + (unsigned)k0 * w_step)) : bf16x8{};
             }
         };
         auto stash = [&](const Stage& stage, int buffer) {
@@ -361,7 +384,24 @@ __device__ __forceinline__ void gemm_tile(
                 }
         }
     }
-    if constexpr (MODE == MODE_GATED) {
+    // With a packed w that was copied as it lies (whole tiles along k), column q of the tile is packed row
+    // first_packed + q of w: the outputs are found through the packing.
+    const bool packed_columns = DK != 0 && is_packed(packing);
+    if (MODE == MODE_GATED && packed_columns) {
+        // a group of 16 packed rows: the gate rows of 8 outputs, then their up rows: a lane's partner is 8 lanes away
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float mine = acc[i][j][e], other = __shfl_xor(mine, 8, XRT_WAVE);
+                    const int q = lane % 32;
+                    const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
+                    const long n = n0 + (wave_n * WAVE_N + j * 32) / 2 + q / 16 * 8 + q % 8;
+                    if (q % 16 < 8 && m < M && n < N) out[m * (long)N + n] = from_float<TO>(silu(mine) * other);
+                }
+    } else if constexpr (MODE == MODE_GATED) {
         static_assert(TN % 2 == 0, "a wavefront holds as many gate blocks as up blocks");
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -374,6 +414,12 @@ __device__ __forceinline__ void gemm_tile(
                     if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(silu(acc[i][j][e]) * acc[i][j + TN / 2][e]);
                 }
     } else {
+        long column[TN];                                        // the output column of this lane in each block of 32
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            column[j] = n0 + wave_n * WAVE_N + j * 32 + lane % 32;
+            if (packed_columns) column[j] = column[j] < N ? logical_row(packing, column[j]) : (long)N;     // (packed rows beyond w make nothing)
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             // When accumulating, what the outputs of one row block hold is read in one go, from
@@ -386,7 +432,7 @@ __device__ __forceinline__ void gemm_tile(
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const long m = min(m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4, (long)M - 1);
-                        const long n = min(n0 + wave_n * WAVE_N + j * 32 + lane % 32, (long)N - 1);
+                        const long n = min(column[j], (long)N - 1);
                         before[j][e] = to_float(out[m * (long)N + n]);
                     }
             }
@@ -395,7 +441,7 @@ __device__ __forceinline__ void gemm_tile(
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
-                    const long n = n0 + wave_n * WAVE_N + j * 32 + lane % 32;
+                    const long n = column[j];
                     if (m < M && n < N) {
                         if constexpr (MODE == MODE_STORE) out[m * (long)N + n] = from_float<TO>(acc[i][j][e]);
                         else out[m * (long)N + n] = from_float<TO>(before[j][e] + acc[i][j][e]);
@@ -408,8 +454,8 @@ __device__ __forceinline__ void gemm_tile(
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int tiles_m, int tiles_n, int n_first, int k_per_split, const RowScale scale) {
-    gemm_tile<BM, BN, WM, WN, MODE, DK, STAGES, TO>(a, w, out, M, N, K, blockIdx.x, tiles_m, tiles_n, n_first, k_per_split, scale);
+    int tiles_m, int tiles_n, int n_first, int k_per_split, const Packing packing, const RowScale scale) {
+    gemm_tile<BM, BN, WM, WN, MODE, DK, STAGES, TO>(a, w, out, M, N, K, blockIdx.x, tiles_m, tiles_n, n_first, k_per_split, packing, scale);
 }
 
 // Two tile shapes in one launch: the first `large_blocks` workgroups take 256 x 256 tiles of the
@@ -420,18 +466,19 @@ __global__ void __launch_bounds__(WM * WN * XRT_WAVE) gemm_mfma_kernel(
 template <int MODE, typename TO>
 __global__ void __launch_bounds__(8 * XRT_WAVE) gemm_mfma_mixed_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int large_blocks, int large_tiles_m, int large_tiles_n, int split, int small_tiles_m, int small_tiles_n) {
+    int large_blocks, int large_tiles_m, int large_tiles_n, int split, int small_tiles_m, int small_tiles_n,
+    const Packing packing) {
     if ((int)blockIdx.x < large_blocks)
-        gemm_tile<256, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x, large_tiles_m, large_tiles_n, 0, K);
+        gemm_tile<256, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x, large_tiles_m, large_tiles_n, 0, K, packing);
     else
         gemm_tile<128, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x - large_blocks, small_tiles_m,
-                                                   small_tiles_n, split, K);
+                                                   small_tiles_n, split, K, packing);
 }
 
 // Launches the tiles of output columns [n_first, n_first + n_count).
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
-int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, hipStream_t s,
-                  int splits = 1, int k_per_split = 0, const RowScale scale = RowScale{}) {
+int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, const Packing& packing,
+                  hipStream_t s, int splits = 1, int k_per_split = 0, const RowScale scale = RowScale{}) {
     constexpr int BN_OUT = MODE == MODE_GATED ? BN / 2 : BN;
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr size_t staging = DK != 0 ? (size_t)STAGES * (BM + BN) * DK * sizeof(bf16) : (size_t)2 * (BM + BN) * PITCH * sizeof(bf16);
@@ -450,19 +497,19 @@ int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, in
     XRT_REQUIRE(splits == 1 || DK != 0, "linear (mfma): only whole tiles along k can be split");
     XRT_REQUIRE(scale.squares == nullptr || (BM <= 64 && splits == 1), "linear (mfma): rows are scaled by tiles of up to 64 rows that see all of k");
     kernel<<<dim3(grid, splits), THREADS, lds, s>>>(a, w, out, M, N, K, tiles_m, tiles_n, n_first,
-                                                    splits == 1 ? K : k_per_split, scale);
+                                                    splits == 1 ? K : k_per_split, packing, scale);
     XRT_LAUNCH_CHECK("linear (mfma)");
     return 0;
 }
 
 template <int BM, int BN, int WM, int WN, int MODE, typename TO>
-int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, hipStream_t s) {
+int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, const Packing& packing, hipStream_t s) {
     // Whole tiles along k go straight into LDS, in two stages of 64; a ragged last tile needs the
     // path through registers. (Four stages of 32 keep a load in flight for longer but meet at
     // twice as many barriers, and measured slower: 1.03 against 1.06 to 1.16 PFLOP/s on the large tiles.)
-    if (K % 64 == 0) return launch_kernel<BM, BN, WM, WN, MODE, 64, 2, TO>(a, w, out, M, N, K, n_first, n_count, s);
+    if (K % 64 == 0) return launch_kernel<BM, BN, WM, WN, MODE, 64, 2, TO>(a, w, out, M, N, K, n_first, n_count, packing, s);
     if constexpr (BM == 256 && BN == 256 || BM == 128 && BN == 128) {
-        return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, n_first, n_count, s);
+        return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, n_first, n_count, packing, s);
     } else {
         XRT_REQUIRE(false, "linear (mfma): this tile takes only K that is a multiple of 64 (K=%d)", K);
     }
@@ -478,7 +525,7 @@ long rounds_cost(long tiles, int tile_elements, int share, int penalty) {
 }
 
 template <int MODE, typename TO>
-int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, const Packing& packing, hipStream_t s) {
     // output columns per tile are half the tile's w rows in the gated mode
     constexpr int DIV = MODE == MODE_GATED ? 2 : 1;
     auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn / DIV - 1) / (bn / DIV)); };
@@ -509,21 +556,21 @@ int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, hipS
             configured = true;
         }
         kernel<<<large_blocks + small_blocks, 8 * XRT_WAVE, lds, s>>>(a, w, out, M, N, K, large_blocks, tiles_m, whole_columns,
-                                                                      split, small_tiles_m, small_tiles_n);
+                                                                      split, small_tiles_m, small_tiles_n, packing);
         XRT_LAUNCH_CHECK("linear (mfma, two tile shapes)");
         return 0;
     }
-    if (large <= medium && large <= small) return launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, 0, N, s);
+    if (large <= medium && large <= small) return launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, 0, N, packing, s);
     if constexpr (MODE != MODE_GATED)
-        if (medium <= small) return launch<256, 192, 4, 2, MODE, TO>(a, w, out, M, N, K, 0, N, s);
-    return launch<128, 128, 2, 2, MODE, TO>(a, w, out, M, N, K, 0, N, s);
+        if (medium <= small) return launch<256, 192, 4, 2, MODE, TO>(a, w, out, M, N, K, 0, N, packing, s);
+    return launch<128, 128, 2, 2, MODE, TO>(a, w, out, M, N, K, 0, N, packing, s);
 }
 
 template <typename TO>
-int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, hipStream_t s) {
-    if (mode == MODE_STORE) return launch_mode<MODE_STORE, TO>(a, w, out, M, N, K, s);
-    if (mode == MODE_ACCUMULATE) return launch_mode<MODE_ACCUMULATE, TO>(a, w, out, M, N, K, s);
-    return launch_mode<MODE_GATED, TO>(a, w, out, M, N, K, s);
+int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, const Packing& packing, hipStream_t s) {
+    if (mode == MODE_STORE) return launch_mode<MODE_STORE, TO>(a, w, out, M, N, K, packing, s);
+    if (mode == MODE_ACCUMULATE) return launch_mode<MODE_ACCUMULATE, TO>(a, w, out, M, N, K, packing, s);
+    return launch_mode<MODE_GATED, TO>(a, w, out, M, N, K, packing, s);
 }
 
 // ---- 17 to 64 rows of x: too many for the kernel that streams w through registers (it would read
@@ -694,7 +741,7 @@ __global__ void __launch_bounds__(256) split_reduce_qkv_kernel(const float* __re
 }
 
 template <typename TO>
-int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, float* workspace,
+int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, const Packing& packing, float* workspace,
                  const xrt_linear_norm* norm, const QkvAfter* after, hipStream_t s) {
     const SplitPlan plan = split_plan(M, N, K, mode);
     const bool scaled = norm && norm->squares_in, emits = norm && norm->squares_out;
@@ -704,19 +751,19 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
                 "linear (mfma): only a bfloat16 product split along k does what follows a q/k/v projection");
     if (M <= SPLIT_BM && plan.splits == 1) {                   // tiles enough: each applies the epilogue itself
         XRT_REQUIRE(!emits, "linear (mfma): only a product split along k writes what the norm after it needs");
-        if (mode == MODE_STORE) return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s, 1, 0, scale);
-        if (mode == MODE_GATED) return launch_kernel<SPLIT_BM, SPLIT_BN, 2, 2, MODE_GATED, 64, 3, TO>(a, w, out, M, N, K, 0, N, s, 1, 0, scale);
+        if (mode == MODE_STORE) return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, TO>(a, w, out, M, N, K, 0, N, packing, s, 1, 0, scale);
+        if (mode == MODE_GATED) return launch_kernel<SPLIT_BM, SPLIT_BN, 2, 2, MODE_GATED, 64, 3, TO>(a, w, out, M, N, K, 0, N, packing, s, 1, 0, scale);
         if constexpr (sizeof(TO) == 4)
-            return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_ACCUMULATE, 64, 3, TO>(a, w, out, M, N, K, 0, N, s, 1, 0, scale);
+            return launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_ACCUMULATE, 64, 3, TO>(a, w, out, M, N, K, 0, N, packing, s, 1, 0, scale);
         XRT_REQUIRE(false, "linear (mfma): accumulation needs a float32 output");
     }
     XRT_REQUIRE(workspace != nullptr, "linear (mfma): a product split along k needs its workspace");
     // the product of all rows of w, ungated, into the workspace: [splits][M][rows_w]
     const int status = M <= SPLIT_BM
         ? launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, float>(
-              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split)
+              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split)
         : launch_kernel<128, 128, 2, 2, MODE_STORE, 64, 2, float>(
-              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, s, plan.splits, plan.k_per_split);
+              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split);
     if (status != 0) return status;
     const unsigned blocks = (unsigned)(((long)M * N + 255) / 256);
     const xrt_linear_norm none = {};
@@ -748,13 +795,13 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
 
 bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, int mode) {
     const long rows_w = mode == MODE_GATED ? 2L * N : N;     // operands are addressed with 32-bit element offsets
-    return K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0 && (long)M * K < (1L << 31) && rows_w * K < (1L << 31);
+    return K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0 && (long)M * K < (1L << 31) && (rows_w + 15) * K < (1L << 31);
 }
 
 int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
-                    hipStream_t s) {
-    if (out_dtype == XRT_F32) return launch_shape<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, s);
-    return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, s);
+                    const Packing& packing, hipStream_t s) {
+    if (out_dtype == XRT_F32) return launch_shape<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, packing, s);
+    return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, packing, s);
 }
 
 // Whether a product runs through the tiles of this section (17 to 64 rows of x, or more rows and few
@@ -779,10 +826,10 @@ bool xrt_linear_split_takes_norm(const void* a, const void* w, int M, int N, int
     return split_plan(M, N, K, mode).splits > 1 && N % 64 == 0 && N >= 128;
 }
 
-int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, const Packing& packing,
                      float* workspace, const xrt_linear_norm* norm, hipStream_t s) {
-    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, workspace, norm, nullptr, s);
-    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, workspace, norm, nullptr, s);
+    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, packing, workspace, norm, nullptr, s);
+    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, packing, workspace, norm, nullptr, s);
 }
 
 // Whether the q/k/v projection of a step of 17 to 64 tokens can also do what follows it (rotation over the
@@ -794,7 +841,7 @@ bool xrt_linear_split_takes_qkv(const void* a, const void* w, int M, int N, int 
     return xrt_linear_split_takes(a, w, M, N, K, MODE_STORE, workspace_floats) && *workspace_floats > 0;
 }
 
-int xrt_linear_split_qkv(const void* a, const void* w, void* qkv, int M, int N, int K, float* workspace,
+int xrt_linear_split_qkv(const void* a, const void* w, void* qkv, int M, int N, int K, const Packing& packing, float* workspace,
                          const xrt_linear_norm* norm, const QkvAfter& after, hipStream_t s) {
-    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)qkv, M, N, K, MODE_STORE, workspace, norm, &after, s);
+    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)qkv, M, N, K, MODE_STORE, packing, workspace, norm, &after, s);
 }

@@ -9,9 +9,25 @@ extern "C" {
 
 const char* xrt_last_error(void);
 
+// How a bfloat16 weight matrix w[rows][K] is laid out. XRT_PACK_NONE (or a null pointer wherever a packing
+// is passed): rows contiguous along k. Otherwise tiles of 16 rows x 32 columns in the order in which the matrix
+// cores take them, rows padded to a multiple of 16 with zeros, K a multiple of 32; the rows may also be
+// regrouped so that outputs which an epilogue combines share a tile (csrc/packing.h says how):
+// XRT_PACK_GATED for [gate rows | up rows] (gated_n outputs, a multiple of 8), XRT_PACK_ROTARY for rows
+// [heads][head_dim] whose first rotated_heads heads are rotated over the whole head.
+// Products that are bound by reading w (few rows of a) stream a packed w faster; all others take either form.
+enum { XRT_PACK_NONE = 0, XRT_PACK_TILES = 1, XRT_PACK_GATED = 2, XRT_PACK_ROTARY = 3 };
+typedef struct xrt_packing { int kind; int gated_n; int head_dim; int rotated_heads; } xrt_packing;
+// packed[...] = w in the layout `packing` (rows padded to a multiple of 16: the packed matrix has
+// (rows + 15) / 16 * 16 * K elements); XRT_PACK_GATED needs rows = 2 * gated_n, XRT_PACK_ROTARY rows a
+// multiple of head_dim
+int xrt_pack_weight(const void* w, void* packed, int rows, int K, const xrt_packing* packing, void* stream);
+// whether packing pays for a matrix of these sizes (its tiles divide evenly among the compute units)
+int xrt_packing_suits(int rows, int K);
+
 // out[t, :] = table[ids[t], :] as float32
-int xrt_embed(const void* table, int table_dtype, const int* ids, float* out, int tokens, int hidden,
-              int vocab, void* stream);
+int xrt_embed(const void* table, int table_dtype, const xrt_packing* packing, const int* ids, float* out, int tokens,
+              int hidden, int vocab, void* stream);
 
 // out[i] = element i of the random-weights stream `key`: float(2 * (sum of twelve 10-bit fields of two
 // splitmix64 words) - 12 * 1023) * scale + offset, the same values as the host-side generator gives
@@ -43,6 +59,9 @@ int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype, float eps,
 int xrt_linear(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
                int mode, float* workspace, long workspace_floats, void* stream);
 long xrt_linear_workspace(const void* a, const void* w, int dtype, int M, int N, int K, int mode);
+// the same with w in the layout `packing` (null: rows contiguous along k)
+int xrt_linear_with(const void* a, const void* w, const xrt_packing* packing, int dtype, void* out, int out_dtype, int M, int N,
+                    int K, int mode, float* workspace, long workspace_floats, void* stream);
 
 // xrt_linear for callers that cannot allocate device memory: code under HIP graph capture, tight serving
 // loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. The partial sums of a
@@ -67,10 +86,10 @@ typedef struct xrt_linear_norm {
     const float* squares_in; int tiles_in; int width_in; float eps;
     void* scaled_out; const void* gain; int gain_dtype; float* squares_out;
 } xrt_linear_norm;
-int xrt_linear_takes_norm(const void* a, const void* w, int dtype, int M, int N, int K, int mode);
-int xrt_linear_norm_tiles(const void* a, const void* w, int dtype, int M, int N, int K);   // rows of the table at squares_out
-int xrt_linear_normed(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
-                      int mode, const xrt_linear_norm* norm, float* workspace, long workspace_floats, void* stream);
+int xrt_linear_takes_norm(const void* a, const void* w, const xrt_packing* packing, int dtype, int M, int N, int K, int mode);
+int xrt_linear_norm_tiles(const void* a, const void* w, const xrt_packing* packing, int dtype, int M, int N, int K);   // rows of the table at squares_out
+int xrt_linear_normed(const void* a, const void* w, const xrt_packing* packing, int dtype, void* out, int out_dtype, int M, int N,
+                      int K, int mode, const xrt_linear_norm* norm, float* workspace, long workspace_floats, void* stream);
 
 // per-head RMSNorm of q and k (optional), rotation of q and k (optional), write of k and v
 // into the cache (optional); qkv rows are [q heads | k heads | v heads]. longest_run: the most
@@ -87,7 +106,7 @@ int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, int n_kv_head
 // decode step allows it (bfloat16, at most 16 rows, no head norms), else in two. norm: null, or the
 // squares_in half of an RMSNorm before the projection (then a is what xrt_linear_normed would take).
 // workspace as for xrt_linear.
-int xrt_linear_qkv(const void* a, const void* w, int dtype, void* qkv, int M, int K, const xrt_linear_norm* norm,
+int xrt_linear_qkv(const void* a, const void* w, const xrt_packing* packing, int dtype, void* qkv, int M, int K, const xrt_linear_norm* norm,
                    int n_heads, int n_kv_heads, int head_dim, const int* positions, const int* slots,
                    const void* q_norm, const void* k_norm, int norm_dtype, float norm_eps,
                    const float* rope_theta, int rope_dim, float rope_scale,

@@ -44,14 +44,15 @@ class StepError(ValueError):
 class Engine:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype="bfloat16",
                  max_tokens: int = 4096, max_slots: Optional[int] = None,
-                 max_context: Optional[int] = None, device="cuda:0", ops=None, graphs: bool = True):
+                 max_context: Optional[int] = None, device="cuda:0", ops=None, graphs: bool = True,
+                 pack_weights="auto"):
         self.dtype = compute_dtype(dtype)
         self.device = torch.device(device)
         if ops is None:
             from ..ops import load_ops
             ops = load_ops()            # raises if the HIP library cannot be loaded: there is no other path
         self.ops = ops
-        self.runtime = Runtime(ops, self.dtype, self.device)
+        self.runtime = Runtime(ops, self.dtype, self.device, pack_weights)
         self.config = spec.config
         # by checkpoint name: a dict, or a source that reads or makes a tensor when a part asks for it and
         # keeps none, so that the device holds every weight once, in the form the parts bound it

@@ -50,6 +50,55 @@ class Prescaled:
         return self.values.shape
 
 
+class _Packing(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int), ("gated_n", ctypes.c_int), ("head_dim", ctypes.c_int),
+                ("rotated_heads", ctypes.c_int)]
+
+
+PACK_TILES, PACK_GATED, PACK_ROTARY = 1, 2, 3
+
+
+class PackedMatrix:
+    """A bfloat16 weight matrix [rows, k] kept in tiles of 16 rows x 32 columns in the order in which the matrix
+    cores take them (XRT_PACK_* of the library's header), so that products of few rows stream it faster.
+    `linear`, `linear_glu`, `linear_qkv` and `embed` take it in place of the plain matrix; nothing else reads it."""
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int, packing: _Packing):
+        self.data, self.packing = data, packing
+        self.shape = (rows, cols)
+        self.dtype, self.device = data.dtype, data.device
+
+    def dim(self) -> int:
+        return 2
+
+    def unpacked(self) -> torch.Tensor:
+        """The matrix [rows, k] with rows contiguous along k again (for inspection and tests; products never need it)."""
+        rows, cols = self.shape
+        groups = (rows + 15) // 16
+        by_packed_row = self.data.view(groups, cols // 32, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(groups * 16, cols)
+        logical = torch.arange(rows, device=self.data.device)
+        p = self.packing
+        if p.kind == PACK_GATED:
+            up = logical >= p.gated_n
+            j = torch.where(up, logical - p.gated_n, logical)
+            packed = j // 8 * 16 + up.long() * 8 + j % 8
+        elif p.kind == PACK_ROTARY:
+            head, d = logical // p.head_dim, logical % p.head_dim
+            half, within = d // (p.head_dim // 2), d % (p.head_dim // 2)
+            paired = head * p.head_dim + within // 8 * 16 + half * 8 + within % 8
+            packed = torch.where(head < p.rotated_heads, paired, logical)
+        else:
+            packed = logical
+        return by_packed_row[packed]
+
+
+def _matrix(w):
+    """(tensor that holds the data, packing argument) of a weight in either form."""
+    if isinstance(w, PackedMatrix):
+        return w.data, ctypes.byref(w.packing)
+    return w, None
+
+
 class _LinearNorm(ctypes.Structure):
     _fields_ = [("squares_in", ctypes.c_void_p), ("tiles_in", ctypes.c_int), ("width_in", ctypes.c_int),
                 ("eps", ctypes.c_float), ("scaled_out", ctypes.c_void_p), ("gain", ctypes.c_void_p),
@@ -82,7 +131,8 @@ class HipOps:
         self.path = path
         self.lib.xrt_last_error.restype = ctypes.c_char_p
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
-                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv", "xrt_random_normal"):
+                     "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv", "xrt_random_normal",
+                     "xrt_linear_with", "xrt_pack_weight", "xrt_packing_suits"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
         self.lib.xrt_attention_workspace.restype = ctypes.c_long
@@ -115,11 +165,32 @@ class HipOps:
     def embed(self, table, ids, out):
         vocab, hidden = table.shape
         tokens = ids.shape[0]
-        self._require(table, "embed table")
-        self._require(ids, "embed ids", torch.int32, (tokens,), table)
-        self._require(out, "embed out", torch.float32, (tokens, hidden), table)
-        self._check(self.lib.xrt_embed(_ptr(table), _code(table), _ptr(ids), _ptr(out), tokens, hidden, vocab,
+        data, packing = _matrix(table)
+        self._require(data, "embed table")
+        self._require(ids, "embed ids", torch.int32, (tokens,), data)
+        self._require(out, "embed out", torch.float32, (tokens, hidden), data)
+        self._check(self.lib.xrt_embed(_ptr(data), _code(data), packing, _ptr(ids), _ptr(out), tokens, hidden, vocab,
                                        self._stream(out)))
+
+    def packing_suits(self, rows: int, cols: int) -> bool:
+        """Whether a bfloat16 matrix of these sizes is better kept packed."""
+        return bool(self.lib.xrt_packing_suits(int(rows), int(cols)))
+
+    def pack(self, w: torch.Tensor, kind: str = "tiles", gated_n: int = 0, head_dim: int = 0, rotated_heads: int = 0):
+        """w [rows, k] (bfloat16, on the GPU) in the packed layout `kind`: "tiles", "gated" (w is gate rows then
+        up rows, gated_n each) or "rotary" (w is heads x head_dim rows, the first rotated_heads heads rotated over
+        the whole head)."""
+        self._require(w, "pack w", torch.bfloat16)
+        if w.dim() != 2:
+            raise KernelError("pack: w must be [rows, k]")
+        rows, cols = w.shape
+        code = {"tiles": PACK_TILES, "gated": PACK_GATED, "rotary": PACK_ROTARY}.get(kind)
+        if code is None:
+            raise KernelError(f"pack: unknown kind {kind!r}")
+        packing = _Packing(code, int(gated_n), int(head_dim), int(rotated_heads))
+        data = torch.empty(((rows + 15) // 16 * 16) * cols, dtype=torch.bfloat16, device=w.device)
+        self._check(self.lib.xrt_pack_weight(_ptr(w), _ptr(data), rows, cols, ctypes.byref(packing), self._stream(w)))
+        return PackedMatrix(data, rows, cols, packing)
 
     def random_normal(self, out, key: int, scale: float, offset: float = 0.0):
         """out[i] = element i of the random-weights stream `key` (weights/random_init.py), times scale, plus offset."""
@@ -169,20 +240,24 @@ class HipOps:
         if a.dim() != 2 or w.dim() != 2:
             raise KernelError("linear: operands must be [rows, k]")
         m, k = a.shape
+        data, packing = _matrix(w)
         self._require(a, "linear a")
-        self._require(w, "linear w", a.dtype, None, a)
+        self._require(data, "linear w", a.dtype, None, a)
         if w.shape[1] != k:
             raise KernelError(f"linear: a has {k} columns, w has {w.shape[1]}")
+        if w.shape[0] != (2 * n if mode == 2 else n):
+            raise KernelError(f"linear: w has {w.shape[0]} rows for {n} outputs")
         self._require(out, "linear out", None, (m, n), a)
-        sizes = (_ptr(a), _ptr(w), _code(a))
+        sizes = (_ptr(a), _ptr(data), _code(a))
+        packed = (_ptr(a), _ptr(data), packing, _code(a))
         # the norm after an accumulating product: only if that product, and one of the same rows
         # over the n columns it writes, can take it
         emit = None
-        if then_norm is not None and mode == 1 and n % 8 == 0 and self.lib.xrt_linear_takes_norm(*sizes, m, n, k, mode):
+        if then_norm is not None and mode == 1 and n % 8 == 0 and self.lib.xrt_linear_takes_norm(*packed, m, n, k, mode):
             gain, eps = then_norm
             self._require(gain, "norm gain", None, (n,), a)
             emit = Prescaled(torch.empty((m, n), dtype=torch.bfloat16, device=a.device),
-                             torch.empty((int(self.lib.xrt_linear_norm_tiles(*sizes, m, n, k)), SQUARES_STRIDE),
+                             torch.empty((int(self.lib.xrt_linear_norm_tiles(*packed, m, n, k)), SQUARES_STRIDE),
                                          dtype=torch.float32, device=a.device),
                              float(eps))
         if scaled is not None or emit is not None:
@@ -196,13 +271,13 @@ class HipOps:
                 norm.gain, norm.gain_dtype = then_norm[0].data_ptr(), _code(then_norm[0])
             need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
             workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
-            self._check(self.lib.xrt_linear_normed(*sizes, _ptr(out), _code(out), m, n, k, mode, ctypes.byref(norm),
+            self._check(self.lib.xrt_linear_normed(*packed, _ptr(out), _code(out), m, n, k, mode, ctypes.byref(norm),
                                                    _ptr(workspace), ctypes.c_long(need), self._stream(a)))
             return emit
         need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
-        self._check(self.lib.xrt_linear(*sizes, _ptr(out), _code(out), m, n, k, mode,
-                                        _ptr(workspace), ctypes.c_long(need), self._stream(a)))
+        self._check(self.lib.xrt_linear_with(*packed, _ptr(out), _code(out), m, n, k, mode,
+                                             _ptr(workspace), ctypes.c_long(need), self._stream(a)))
         return None
 
     def linear(self, a, w, out, accumulate=False, then_norm: Optional[Tuple[torch.Tensor, float]] = None):
@@ -257,8 +332,11 @@ class HipOps:
         if a.dim() != 2 or w.dim() != 2:
             raise KernelError("linear_qkv: operands must be [rows, k]")
         m, k = a.shape
+        data, packing = _matrix(w)
         self._require(a, "linear_qkv a")
-        self._require(w, "linear_qkv w", a.dtype, ((n_heads + 2 * n_kv_heads) * head_dim, k), a)
+        self._require(data, "linear_qkv w", a.dtype, None, a)
+        if tuple(w.shape) != ((n_heads + 2 * n_kv_heads) * head_dim, k):
+            raise KernelError(f"linear_qkv w: shape {tuple(w.shape)}, expected {((n_heads + 2 * n_kv_heads) * head_dim, k)}")
         self._require(qkv, "qkv", a.dtype, (m, w.shape[0]), a)
         prepare = self._prepare_arguments(qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm, k_norm,
                                           norm_eps, rope_theta, rope_dim, rope_scale, kv, longest_run)
@@ -268,9 +346,9 @@ class HipOps:
             self._require(scaled.squares, "sums of squares", torch.float32, (tiles, SQUARES_STRIDE), a)
             norm = _LinearNorm()
             norm.squares_in, norm.tiles_in, norm.width_in, norm.eps = scaled.squares.data_ptr(), tiles, k, scaled.eps
-        need = int(self.lib.xrt_linear_workspace(_ptr(a), _ptr(w), _code(a), m, w.shape[0], k, 0))
+        need = int(self.lib.xrt_linear_workspace(_ptr(a), _ptr(data), _code(a), m, w.shape[0], k, 0))
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
-        self._check(self.lib.xrt_linear_qkv(_ptr(a), _ptr(w), _code(a), _ptr(qkv), m, k,
+        self._check(self.lib.xrt_linear_qkv(_ptr(a), _ptr(data), packing, _code(a), _ptr(qkv), m, k,
                                             None if norm is None else ctypes.byref(norm), *prepare,
                                             _ptr(workspace), ctypes.c_long(need), self._stream(a)))
 

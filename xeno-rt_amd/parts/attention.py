@@ -74,8 +74,12 @@ class Attention(Mixer):
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         p = self.prefix
-        self.w_qkv = runtime.stacked(tensors[p + name] for name in ("q_proj.weight", "k_proj.weight", "v_proj.weight"))
-        self.w_o = runtime.matrix(tensors[p + "o_proj.weight"])
+        # q and k heads that a rotation over the whole head turns: their pairs are kept side by side
+        whole = isinstance(self.position, Rotary) and self.position.rope_dim == self.head_dim
+        self.w_qkv = runtime.weight([tensors[p + name] for name in ("q_proj.weight", "k_proj.weight", "v_proj.weight")],
+                                    "rotary", head_dim=self.head_dim,
+                                    rotated_heads=self.n_heads + self.n_kv_heads if whole else 0)
+        self.w_o = runtime.weight(tensors[p + "o_proj.weight"])
         if self.qk_norm:
             self.q_norm = runtime.vector(tensors[p + "q_norm.weight"])
             self.k_norm = runtime.vector(tensors[p + "k_norm.weight"])

@@ -62,12 +62,15 @@ class CacheNeeds:
 class Runtime:
     """What a part needs to run: the kernels, the compute dtype and the device."""
 
-    def __init__(self, ops, dtype: torch.dtype, device):
+    def __init__(self, ops, dtype: torch.dtype, device, pack_weights="auto"):
         if dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"compute dtype must be bfloat16 or float32, found {dtype}")
+        if pack_weights not in ("auto", "always", False):
+            raise ValueError(f"pack_weights must be 'auto', 'always' or False, found {pack_weights!r}")
         self.ops = ops
         self.dtype = dtype
         self.device = torch.device(device)
+        self.pack_weights = pack_weights        # "auto": where the kernels say it pays; "always": wherever it can be done
 
     def matrix(self, tensor: torch.Tensor) -> torch.Tensor:
         """A weight matrix in the compute dtype, contiguous, on the device. A tensor that comes from the
@@ -91,6 +94,25 @@ class Runtime:
             out[at:at + tensor.shape[0]].copy_(tensor)
             at += tensor.shape[0]
         return out
+
+    def weight(self, tensors, kind: str = "tiles", **details):
+        """What `ops.linear` (or `linear_glu`, `linear_qkv`, `embed`) takes as its w: the matrix (or the matrices
+        of equal width, one below the other) in the compute dtype on the device, and, where the kernels have a
+        faster layout for matrices of its sizes, in that layout. kind and details name what the product's
+        epilogue combines: "tiles" nothing, "gated" gate rows and up rows (gated_n of each), "rotary" the
+        pairs of a rotation over whole heads (head_dim, rotated_heads). Only products read the result."""
+        matrix = self.stacked(tensors) if isinstance(tensors, (list, tuple)) else self.matrix(tensors)
+        pack = getattr(self.ops, "pack", None)
+        if (pack is None or not self.pack_weights or self.dtype != torch.bfloat16 or matrix.device.type != "cuda"
+                or matrix.shape[1] % 32 != 0 or (matrix.shape[0] + 15) * matrix.shape[1] >= 2 ** 31):
+            return matrix
+        if kind == "gated" and details.get("gated_n", 0) % 8 != 0:
+            return matrix
+        if kind == "rotary" and details.get("head_dim", 0) % 16 != 0:
+            return matrix
+        if self.pack_weights != "always" and not self.ops.packing_suits(matrix.shape[0], matrix.shape[1]):
+            return matrix
+        return pack(matrix, kind, **details)
 
     def vector(self, tensor: torch.Tensor) -> torch.Tensor:
         """A small float vector: bfloat16 if the file stores it so and the model computes in bfloat16,

@@ -21,13 +21,16 @@ class Embedding(Part):
         self.vocab = vocab
         self.hidden = hidden
         self.table = None
+        self.shared_with_head = False       # set by an OutputHead that is tied to this table
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {self.prefix + "weight": WeightSpec((self.vocab, self.hidden))}
 
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        self.table = runtime.matrix(tensors[self.prefix + "weight"])
+        # a table that is also the head's weight is kept as products like it; one that is only looked up stays plain
+        tensor = tensors[self.prefix + "weight"]
+        self.table = runtime.weight(tensor) if self.shared_with_head else runtime.matrix(tensor)
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         """float32 residual stream [tokens, hidden] for int32 token ids."""
@@ -44,6 +47,8 @@ class OutputHead(Part):
         self.vocab = vocab
         self.hidden = hidden
         self.tied_to = tied_to
+        if tied_to is not None:
+            tied_to.shared_with_head = True
         self.weight = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
@@ -60,7 +65,7 @@ class OutputHead(Part):
         if self.tied_to is not None:
             self.weight = self.tied_to.table        # the same buffer, not a copy
         else:
-            self.weight = runtime.matrix(tensors[self.prefix + "weight"])
+            self.weight = runtime.weight(tensors[self.prefix + "weight"])
 
     def forward(self, y: torch.Tensor) -> torch.Tensor:
         logits = self.runtime.empty((y.shape[0], self.vocab), torch.float32)

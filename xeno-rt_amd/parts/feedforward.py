@@ -42,8 +42,9 @@ class GatedMLP(FeedForward):
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         p = self.prefix
-        self.w_gate_up = runtime.stacked(tensors[p + name] for name in ("gate_proj.weight", "up_proj.weight"))
-        self.w_down = runtime.matrix(tensors[p + "down_proj.weight"])
+        self.w_gate_up = runtime.weight([tensors[p + name] for name in ("gate_proj.weight", "up_proj.weight")],
+                                        "gated", gated_n=self.intermediate)
+        self.w_down = runtime.weight(tensors[p + "down_proj.weight"])
 
     def forward(self, h, batch, residual: torch.Tensor, then=None):
         rt = self.runtime
