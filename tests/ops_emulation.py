@@ -17,7 +17,7 @@ import math
 
 import torch
 
-BLOCK = 64
+from xeno_rt_amd.cache import BLOCK_TOKENS as BLOCK      # the cache's own constant: blocks are its unit
 
 
 class EmulatedOps:
@@ -66,7 +66,8 @@ class EmulatedOps:
             return self.Prescaled((fresh * gain.to(torch.float32)).to(w.dtype), (fresh * fresh).sum(-1), eps)
         return None
 
-    def linear_glu(self, a, w_gate_up, out):
+    def linear_glu(self, a, w_gate_up, out, activation="silu"):
+        assert activation == "silu"
         inter = w_gate_up.shape[0] // 2
         rows, inv = self._rows(a)
         both = (rows @ w_gate_up.to(torch.float32).t()) * inv

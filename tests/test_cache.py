@@ -123,6 +123,16 @@ def test_truncation_below_what_a_window_has_released_is_refused():
     assert ring.pool.n_held == 0
 
 
+def test_values_may_be_wider_or_narrower_than_keys():
+    needs = [CacheNeeds(kv=KVSpec(2, 16, value_dim=40)), CacheNeeds(kv=KVSpec(2, 16))]
+    cache = SequenceCache(needs, [0, 1], 256, 2, 256, torch.float32, "cpu")
+    assert len(cache.groups) == 2                           # another value width is another kind of storage
+    wide = cache.layer_cache(0).kv
+    assert tuple(wide.k.shape[1:]) == (2, 64, 16) and tuple(wide.v.shape[1:]) == (2, 40, 64)
+    assert tuple(cache.layer_cache(1).kv.v.shape[1:]) == (2, 16, 64)
+    assert KVSpec(2, 16).value_width == 16 and KVSpec(2, 16, value_dim=40).value_width == 40
+
+
 def test_state_is_zero_for_every_new_sequence():
     cache = make_cache(state=True)
     a = cache.alloc_slot()

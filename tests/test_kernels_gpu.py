@@ -254,6 +254,25 @@ def test_linear_refuses_what_it_cannot_do(ops):
         ops.linear(rand(8, 2).t(), w, torch.empty(2, 4, device=DEV))
     with pytest.raises(KernelError, match="GPU"):
         ops.linear(a.cpu(), w, torch.empty(2, 4, device=DEV))
+    # the gated product's activation: a name the package does not know, a code the library does not know
+    with pytest.raises(KernelError, match="activation"):
+        ops.linear_glu(a, w, torch.empty(2, 2, device=DEV), activation="gelu")
+    for operands in ((a, w), (rand(2, 64, dtype=torch.bfloat16), rand(32, 64, dtype=torch.bfloat16))):   # every kernel's entry
+        with pytest.raises(KernelError, match="unknown activation 3"):
+            ops._linear(*operands, torch.empty(2, operands[1].shape[0] // 2, dtype=operands[0].dtype, device=DEV),
+                        2 | (3 << 8), operands[1].shape[0] // 2)
+    with pytest.raises(KernelError, match="unknown activation"):
+        ops._linear(a, w, torch.empty(2, 4, device=DEV), 0 | (1 << 8), 4)        # only a gated product has one
+
+
+def test_attention_refuses_values_of_another_width_than_the_keys(ops):
+    from xeno_rt_amd.ops.hip import KernelError
+    kv = make_cache(4, 2, 32, torch.float32, 1, 4)
+    kv.v = torch.zeros(4, 2, 48, 64, device=DEV)
+    qkv = rand(3, (4 + 2 * 2) * 32)
+    batch = SimpleNamespace(positions=i32([0, 1, 2]), slots=i32([0, 0, 0]))
+    with pytest.raises(KernelError, match="as wide as the keys"):
+        ops.attention(qkv, 4, 2, 32, kv, batch, torch.empty(3, 4 * 32, device=DEV), scale=1.0)
 
 
 # ---- q/k/v preparation and attention ------------------------------------------------------
@@ -632,7 +651,24 @@ def test_sample_reference_cases(ops):
     assert sample(ops, logits, temperature=1.0, top_p=0.85, draws=[draw]) == [1]
 
 
-@pytest.mark.parametrize("vocab", [384, 1000, 128256])
+def distribution_by_sorting(logits, temperature, top_k, top_p):
+    """P.sampling_distribution with library sorting instead of a loop over the vocabulary, for large ones
+    (the test below holds it against the loop where that is affordable)."""
+    vocab = logits.numel()
+    order = torch.argsort(-logits.double(), stable=True)[:top_k if top_k > 0 else vocab]       # ties: the lower id first
+    kept = logits.double()[order]
+    probs = torch.exp((kept - kept[0]) / temperature)
+    probs = probs / probs.sum()
+    if top_p < 1.0:
+        reached = torch.nonzero(torch.cumsum(probs, 0) >= top_p)
+        keep = int(reached[0]) + 1 if reached.numel() else probs.numel()
+        order, probs = order[:keep], probs[:keep] / probs[:keep].sum()
+    dist = torch.zeros(vocab, dtype=torch.float64)
+    dist[order] = probs
+    return dist
+
+
+@pytest.mark.parametrize("vocab", [384, 1000, 128256, 300001, (1 << 19) - 7])      # the last two: beyond what goes through slices
 def test_sample_matches_the_plain_distribution(ops, vocab):
     g = torch.Generator().manual_seed(vocab)
     row = torch.randn(vocab, generator=g) * 2.0
@@ -640,16 +676,17 @@ def test_sample_matches_the_plain_distribution(ops, vocab):
     for temperature, top_k, top_p, penalty in [(1.0, 0, 1.0, 1.0), (0.7, 40, 0.95, 1.1), (1.5, 5, 1.0, 2.0),
                                                (1.0, 0, 0.5, 1.0)]:
         adjusted = P.apply_repetition_penalty(row, history, penalty)
-        dist = P.sampling_distribution(adjusted, temperature, top_k, top_p) if vocab <= 1000 else None
-        draws = 512
+        dist = distribution_by_sorting(adjusted, temperature, top_k, top_p)
+        if vocab <= 1000:
+            assert float((dist - P.sampling_distribution(adjusted, temperature, top_k, top_p)).abs().max()) < 1e-12
+        draws = 512 if vocab < 200000 else 128
         logits = row.to(DEV)[None, :].expand(draws, vocab).contiguous()
         u = ((torch.arange(draws) + 0.5) / draws).tolist()          # an even sweep of the unit interval
         picks = sample(ops, logits, temperature, top_k, top_p, penalty, history, draws=u)
         counts = torch.bincount(torch.tensor(picks), minlength=vocab).double() / draws
-        if dist is not None:
-            # an even sweep reproduces every probability to within 1/draws per token
-            assert float((counts - dist).abs().max()) <= 1.5 / draws + 1e-6
-            assert set(torch.nonzero(counts).flatten().tolist()) <= set(torch.nonzero(dist).flatten().tolist())
+        # an even sweep reproduces every probability to within 1/draws per token
+        assert float((counts - dist).abs().max()) <= 1.5 / draws + 1e-6
+        assert set(torch.nonzero(counts).flatten().tolist()) <= set(torch.nonzero(dist).flatten().tolist())
         if top_k:
             kept = set(torch.topk(adjusted, top_k).indices.tolist())
             assert set(picks) <= kept

@@ -10,7 +10,8 @@ from __future__ import annotations
 import heapq
 from typing import List
 
-BLOCK_TOKENS = 64   # tokens per block: the unit in which live requests hold cache
+BLOCK_TOKENS = 64   # tokens per block: the unit in which live requests hold cache (the kernel library is asked for its own
+                    # number when it is loaded, and refused if that differs)
 
 
 class CacheFull(RuntimeError):

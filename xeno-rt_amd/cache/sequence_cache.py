@@ -6,7 +6,7 @@ value rows have the same shape and window form a group; a group has storage of
 its own (one pool of blocks, one block table) and its own rule for which blocks
 a sequence of a given length holds: all of them, or those a window still sees.
 Storage of one call: keys [blocks, kv_heads, BLOCK_TOKENS, head_dim], values
-[blocks, kv_heads, head_dim, BLOCK_TOKENS] (values transposed inside a block, so
+[blocks, kv_heads, value_dim, BLOCK_TOKENS] (values transposed inside a block, so
 that the keys of one block are contiguous along head_dim and the values along
 tokens, which is how the attention kernels read them).
 
@@ -33,7 +33,7 @@ class KVView:
     """What an attention kernel needs of one layer call's keys and values."""
     spec: KVSpec
     k: torch.Tensor             # [blocks, kv_heads, BLOCK_TOKENS, head_dim]
-    v: torch.Tensor             # [blocks, kv_heads, head_dim, BLOCK_TOKENS]
+    v: torch.Tensor             # [blocks, kv_heads, value_dim, BLOCK_TOKENS]
     block_table: torch.Tensor   # int32 [slots, max_blocks]: logical block -> physical block, -1 = none
 
 
@@ -62,7 +62,7 @@ class KVGroup:
         self._end: Dict[int, int] = {}     # slot -> logical blocks [floor, end) may be held
         self._floor: Dict[int, int] = {}   # slot -> lowest logical block it may still hold
         shape_k = (len(calls), n_blocks, spec.n_kv_heads, BLOCK_TOKENS, spec.head_dim)
-        shape_v = (len(calls), n_blocks, spec.n_kv_heads, spec.head_dim, BLOCK_TOKENS)
+        shape_v = (len(calls), n_blocks, spec.n_kv_heads, spec.value_width, BLOCK_TOKENS)
         self.k = torch.zeros(shape_k, dtype=dtype, device=device)
         self.v = torch.zeros(shape_v, dtype=dtype, device=device)
 

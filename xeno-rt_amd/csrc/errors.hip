@@ -1,4 +1,4 @@
-// Last-error text of the calling thread.
+// Last-error text of the calling thread, and the constants that callers must share with the kernels.
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -12,3 +12,5 @@ void xrt_set_error(const char* format, ...) {
 }
 
 extern "C" const char* xrt_last_error(void) { return last_error_text; }
+
+extern "C" int xrt_block_tokens(void) { return XRT_BLOCK_TOKENS; }

@@ -20,6 +20,7 @@
 #include <cstdlib>
 #include "packing.h"
 #include "gemm_skinny.h"
+#include "activation.h"
 
 namespace {
 
@@ -30,14 +31,13 @@ constexpr int BK = 64;
 constexpr int PITCH = BK + 8;          // bf16 elements per LDS row
 enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
 
-__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 
 // One tile of the product, by one workgroup: `id` is the workgroup's number among those that work
 // on the output columns from n_first on, tiles_m x tiles_n of them.
 // The rows of a that come without their RMSNorm's division (see xrt_linear_norm in xrt_hip.h): the sums of
 // squares per tile of 16 columns, from which a tile of up to 64 rows works out 1 / rms of its rows and
 // multiplies its sums by it before the epilogue. squares null: nothing of the kind.
-struct RowScale { const float* squares; int tiles; int width; float eps; };
+struct RowScale { const float* squares; int tiles; int width; float eps; int activation; };     // (activation: of a gated epilogue)
 
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __device__ __forceinline__ void gemm_tile(
@@ -399,7 +399,7 @@ __device__ __forceinline__ void gemm_tile(
                     const int q = lane % 32;
                     const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
                     const long n = n0 + (wave_n * WAVE_N + j * 32) / 2 + q / 16 * 8 + q % 8;
-                    if (q % 16 < 8 && m < M && n < N) out[m * (long)N + n] = from_float<TO>(silu(mine) * other);
+                    if (q % 16 < 8 && m < M && n < N) out[m * (long)N + n] = from_float<TO>(gate_activation(mine, scale.activation) * other);
                 }
     } else if constexpr (MODE == MODE_GATED) {
         static_assert(TN % 2 == 0, "a wavefront holds as many gate blocks as up blocks");
@@ -411,7 +411,7 @@ __device__ __forceinline__ void gemm_tile(
                 for (int e = 0; e < 16; ++e) {
                     const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
                     const long n = n0 + wave_n * (WAVE_N / 2) + j * 32 + lane % 32;
-                    if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(silu(acc[i][j][e]) * acc[i][j + TN / 2][e]);
+                    if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(gate_activation(acc[i][j][e], scale.activation) * acc[i][j + TN / 2][e]);
                 }
     } else {
         long column[TN];                                        // the output column of this lane in each block of 32
@@ -467,12 +467,12 @@ template <int MODE, typename TO>
 __global__ void __launch_bounds__(8 * XRT_WAVE) gemm_mfma_mixed_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
     int large_blocks, int large_tiles_m, int large_tiles_n, int split, int small_tiles_m, int small_tiles_n,
-    const Packing packing) {
+    const Packing packing, const RowScale scale) {
     if ((int)blockIdx.x < large_blocks)
-        gemm_tile<256, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x, large_tiles_m, large_tiles_n, 0, K, packing);
+        gemm_tile<256, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x, large_tiles_m, large_tiles_n, 0, K, packing, scale);
     else
         gemm_tile<128, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x - large_blocks, small_tiles_m,
-                                                   small_tiles_n, split, K, packing);
+                                                   small_tiles_n, split, K, packing, scale);
 }
 
 // Launches the tiles of output columns [n_first, n_first + n_count).
@@ -503,13 +503,15 @@ int launch_kernel(const bf16* a, const bf16* w, TO* out, int M, int N, int K, in
 }
 
 template <int BM, int BN, int WM, int WN, int MODE, typename TO>
-int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, const Packing& packing, hipStream_t s) {
+int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_first, int n_count, const Packing& packing, int activation,
+           hipStream_t s) {
+    const RowScale plain = {nullptr, 0, 0, 0.f, activation};
     // Whole tiles along k go straight into LDS, in two stages of 64; a ragged last tile needs the
     // path through registers. (Four stages of 32 keep a load in flight for longer but meet at
     // twice as many barriers, and measured slower: 1.03 against 1.06 to 1.16 PFLOP/s on the large tiles.)
-    if (K % 64 == 0) return launch_kernel<BM, BN, WM, WN, MODE, 64, 2, TO>(a, w, out, M, N, K, n_first, n_count, packing, s);
+    if (K % 64 == 0) return launch_kernel<BM, BN, WM, WN, MODE, 64, 2, TO>(a, w, out, M, N, K, n_first, n_count, packing, s, 1, 0, plain);
     if constexpr (BM == 256 && BN == 256 || BM == 128 && BN == 128) {
-        return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, n_first, n_count, packing, s);
+        return launch_kernel<BM, BN, WM, WN, MODE, 0, 0, TO>(a, w, out, M, N, K, n_first, n_count, packing, s, 1, 0, plain);
     } else {
         XRT_REQUIRE(false, "linear (mfma): this tile takes only K that is a multiple of 64 (K=%d)", K);
     }
@@ -525,7 +527,7 @@ long rounds_cost(long tiles, int tile_elements, int share, int penalty) {
 }
 
 template <int MODE, typename TO>
-int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, const Packing& packing, hipStream_t s) {
+int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, const Packing& packing, int activation, hipStream_t s) {
     // output columns per tile are half the tile's w rows in the gated mode
     constexpr int DIV = MODE == MODE_GATED ? 2 : 1;
     auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn / DIV - 1) / (bn / DIV)); };
@@ -556,21 +558,21 @@ int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, cons
             configured = true;
         }
         kernel<<<large_blocks + small_blocks, 8 * XRT_WAVE, lds, s>>>(a, w, out, M, N, K, large_blocks, tiles_m, whole_columns,
-                                                                      split, small_tiles_m, small_tiles_n, packing);
+                                                                      split, small_tiles_m, small_tiles_n, packing, RowScale{nullptr, 0, 0, 0.f, activation});
         XRT_LAUNCH_CHECK("linear (mfma, two tile shapes)");
         return 0;
     }
-    if (large <= medium && large <= small) return launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, 0, N, packing, s);
+    if (large <= medium && large <= small) return launch<256, 256, 2, 4, MODE, TO>(a, w, out, M, N, K, 0, N, packing, activation, s);
     if constexpr (MODE != MODE_GATED)
-        if (medium <= small) return launch<256, 192, 4, 2, MODE, TO>(a, w, out, M, N, K, 0, N, packing, s);
-    return launch<128, 128, 2, 2, MODE, TO>(a, w, out, M, N, K, 0, N, packing, s);
+        if (medium <= small) return launch<256, 192, 4, 2, MODE, TO>(a, w, out, M, N, K, 0, N, packing, activation, s);
+    return launch<128, 128, 2, 2, MODE, TO>(a, w, out, M, N, K, 0, N, packing, activation, s);
 }
 
 template <typename TO>
-int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, const Packing& packing, hipStream_t s) {
-    if (mode == MODE_STORE) return launch_mode<MODE_STORE, TO>(a, w, out, M, N, K, packing, s);
-    if (mode == MODE_ACCUMULATE) return launch_mode<MODE_ACCUMULATE, TO>(a, w, out, M, N, K, packing, s);
-    return launch_mode<MODE_GATED, TO>(a, w, out, M, N, K, packing, s);
+int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, int activation, const Packing& packing, hipStream_t s) {
+    if (mode == MODE_STORE) return launch_mode<MODE_STORE, TO>(a, w, out, M, N, K, packing, activation, s);
+    if (mode == MODE_ACCUMULATE) return launch_mode<MODE_ACCUMULATE, TO>(a, w, out, M, N, K, packing, activation, s);
+    return launch_mode<MODE_GATED, TO>(a, w, out, M, N, K, packing, activation, s);
 }
 
 // ---- 17 to 64 rows of x: too many for the kernel that streams w through registers (it would read
@@ -611,7 +613,7 @@ SplitPlan split_plan(int M, int N, int K, int mode) {
 // tile of 16 columns are written as well (N a multiple of 16: the 16 lanes of a tile then share a row).
 template <int MODE, typename TO, int NORM = 0>
 __global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restrict__ parts, int splits, int M, int N,
-                                                            TO* __restrict__ out, const xrt_linear_norm norm) {
+                                                            TO* __restrict__ out, const xrt_linear_norm norm, int activation) {
     __shared__ float wave_sums[256 / XRT_WAVE];
     const long rows_w = MODE == MODE_GATED ? 2L * N : N;
     const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -653,7 +655,7 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restri
     if (inside) {
         if constexpr (MODE == MODE_STORE) out[index] = from_float<TO>(sum);
         else if constexpr (MODE == MODE_ACCUMULATE) { fresh = to_float(out[index]) + sum; out[index] = from_float<TO>(fresh); }
-        else out[index] = from_float<TO>(silu(sum) * up);
+        else out[index] = from_float<TO>(gate_activation(sum, activation) * up);
     }
     if constexpr (NORM == 2) {
         float squares = fresh * fresh;
@@ -741,12 +743,13 @@ __global__ void __launch_bounds__(256) split_reduce_qkv_kernel(const float* __re
 }
 
 template <typename TO>
-int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, const Packing& packing, float* workspace,
-                 const xrt_linear_norm* norm, const QkvAfter* after, hipStream_t s) {
+int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, int activation, const Packing& packing,
+                 float* workspace, const xrt_linear_norm* norm, const QkvAfter* after, hipStream_t s) {
     const SplitPlan plan = split_plan(M, N, K, mode);
     const bool scaled = norm && norm->squares_in, emits = norm && norm->squares_out;
     XRT_REQUIRE(!norm || M <= SPLIT_BM, "linear (mfma): the norm around a product takes at most %d rows here", SPLIT_BM);
-    const RowScale scale = scaled ? RowScale{norm->squares_in, norm->tiles_in, norm->width_in, norm->eps} : RowScale{};
+    const RowScale scale = scaled ? RowScale{norm->squares_in, norm->tiles_in, norm->width_in, norm->eps, activation}
+                                  : RowScale{nullptr, 0, 0, 0.f, activation};
     XRT_REQUIRE(!after || (plan.splits > 1 && mode == MODE_STORE && sizeof(TO) == 2),
                 "linear (mfma): only a bfloat16 product split along k does what follows a q/k/v projection");
     if (M <= SPLIT_BM && plan.splits == 1) {                   // tiles enough: each applies the epilogue itself
@@ -778,7 +781,7 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
         }
         return 0;
     }
-#define XRT_REDUCE(MODE_, NORM_) split_reduce_kernel<MODE_, TO, NORM_><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around)
+#define XRT_REDUCE(MODE_, NORM_) split_reduce_kernel<MODE_, TO, NORM_><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around, activation)
     if (mode == MODE_STORE) { if (scaled) XRT_REDUCE(MODE_STORE, 1); else XRT_REDUCE(MODE_STORE, 0); }
     else if (mode == MODE_GATED) { if (scaled) XRT_REDUCE(MODE_GATED, 1); else XRT_REDUCE(MODE_GATED, 0); }
     else if (scaled) XRT_REDUCE(MODE_ACCUMULATE, 1);
@@ -798,10 +801,10 @@ bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, 
     return K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0 && (long)M * K < (1L << 31) && (rows_w + 15) * K < (1L << 31);
 }
 
-int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, int activation,
                     const Packing& packing, hipStream_t s) {
-    if (out_dtype == XRT_F32) return launch_shape<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, packing, s);
-    return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, packing, s);
+    if (out_dtype == XRT_F32) return launch_shape<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, activation, packing, s);
+    return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, activation, packing, s);
 }
 
 // Whether a product runs through the tiles of this section (17 to 64 rows of x, or more rows and few
@@ -826,10 +829,10 @@ bool xrt_linear_split_takes_norm(const void* a, const void* w, int M, int N, int
     return split_plan(M, N, K, mode).splits > 1 && N % 64 == 0 && N >= 128;
 }
 
-int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, const Packing& packing,
-                     float* workspace, const xrt_linear_norm* norm, hipStream_t s) {
-    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, packing, workspace, norm, nullptr, s);
-    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, packing, workspace, norm, nullptr, s);
+int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, int activation,
+                     const Packing& packing, float* workspace, const xrt_linear_norm* norm, hipStream_t s) {
+    if (out_dtype == XRT_F32) return launch_split<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, activation, packing, workspace, norm, nullptr, s);
+    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, activation, packing, workspace, norm, nullptr, s);
 }
 
 // Whether the q/k/v projection of a step of 17 to 64 tokens can also do what follows it (rotation over the
@@ -843,5 +846,5 @@ bool xrt_linear_split_takes_qkv(const void* a, const void* w, int M, int N, int 
 
 int xrt_linear_split_qkv(const void* a, const void* w, void* qkv, int M, int N, int K, const Packing& packing, float* workspace,
                          const xrt_linear_norm* norm, const QkvAfter& after, hipStream_t s) {
-    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)qkv, M, N, K, MODE_STORE, packing, workspace, norm, &after, s);
+    return launch_split<bf16>((const bf16*)a, (const bf16*)w, (bf16*)qkv, M, N, K, MODE_STORE, XRT_ACT_SILU, packing, workspace, norm, &after, s);
 }

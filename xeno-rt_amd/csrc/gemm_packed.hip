@@ -19,6 +19,7 @@
 // rotated head's pairs into one tile).
 #include "packing.h"
 #include "gemm_skinny.h"
+#include "activation.h"
 
 namespace {
 
@@ -31,7 +32,6 @@ constexpr int WAVES = 8;
 constexpr int JL = 2;              // tiles of 32 along k per step of a wavefront
 enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
 
-__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 
 // MT: tiles of 16 rows of x. EXTRA 1: the kernel also does its share of an RMSNorm before or after the
 // product; 2: and what follows a q/k/v projection (both: one tile of x).
@@ -39,7 +39,7 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 template <int MT, int MODE, typename TO, int EXTRA = 0>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_packed_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    const Packing packing, const LinearNorm norm, const QkvAfter after) {
+    const Packing packing, const LinearNorm norm, const QkvAfter after, int activation) {
     constexpr bool AROUND = EXTRA != 0, QKV = EXTRA == 2;
     static_assert(!AROUND || MT == 1, "the norm around a product: one tile of x");
     static_assert(!QKV || (MODE == MODE_STORE && sizeof(TO) == 2), "after a q/k/v projection: a bfloat16 store");
@@ -320,7 +320,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
             if (c < 2 && mm < M) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (nn + i < N) out[(long)mm * N + nn + i] = from_float<TO>(silu(g[i]) * u[i]);
+                    if (nn + i < N) out[(long)mm * N + nn + i] = from_float<TO>(gate_activation(g[i], activation) * u[i]);
             }
             continue;
         }
@@ -372,7 +372,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
 }
 
 template <int MT, typename TO>
-int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const Packing& packing,
+int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, int activation, const Packing& packing,
                 const LinearNorm& norm, const QkvAfter* after, hipStream_t s) {
     const long rows_w = mode == MODE_GATED ? 2L * N : N;
     const unsigned grid = (unsigned)((rows_w + 15) / 16);
@@ -381,17 +381,17 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
     if constexpr (MT == 1) {
         if (after) {
             if constexpr (sizeof(TO) == 2) {
-                gemm_packed_kernel<1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, *after);
+                gemm_packed_kernel<1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, *after, activation);
                 XRT_LAUNCH_CHECK("linear (packed, q/k/v)");
                 return 0;
             }
         } else if (norm.squares_in || norm.squares_out) {
             if (mode == MODE_STORE)
-                gemm_packed_kernel<1, MODE_STORE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none);
+                gemm_packed_kernel<1, MODE_STORE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none, activation);
             else if (mode == MODE_ACCUMULATE)
-                gemm_packed_kernel<1, MODE_ACCUMULATE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none);
+                gemm_packed_kernel<1, MODE_ACCUMULATE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none, activation);
             else
-                gemm_packed_kernel<1, MODE_GATED, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none);
+                gemm_packed_kernel<1, MODE_GATED, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none, activation);
             XRT_LAUNCH_CHECK("linear (packed, with norm)");
             return 0;
         }
@@ -401,23 +401,23 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
         return 1;
     }
     if (mode == MODE_STORE)
-        gemm_packed_kernel<MT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none);
+        gemm_packed_kernel<MT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none, activation);
     else if (mode == MODE_ACCUMULATE)
-        gemm_packed_kernel<MT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none);
+        gemm_packed_kernel<MT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none, activation);
     else
-        gemm_packed_kernel<MT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none);
+        gemm_packed_kernel<MT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, none, activation);
     XRT_LAUNCH_CHECK("linear (packed)");
     return 0;
 }
 
 template <typename TO>
-int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const Packing& packing,
+int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, int activation, const Packing& packing,
                  const LinearNorm& norm, const QkvAfter* after, hipStream_t s) {
     switch ((M + 15) / 16) {
-        case 1: return launch_mode<1, TO>(x, w, out, M, N, K, mode, packing, norm, after, s);
-        case 2: return launch_mode<2, TO>(x, w, out, M, N, K, mode, packing, norm, after, s);
-        case 3: return launch_mode<3, TO>(x, w, out, M, N, K, mode, packing, norm, after, s);
-        default: return launch_mode<4, TO>(x, w, out, M, N, K, mode, packing, norm, after, s);
+        case 1: return launch_mode<1, TO>(x, w, out, M, N, K, mode, activation, packing, norm, after, s);
+        case 2: return launch_mode<2, TO>(x, w, out, M, N, K, mode, activation, packing, norm, after, s);
+        case 3: return launch_mode<3, TO>(x, w, out, M, N, K, mode, activation, packing, norm, after, s);
+        default: return launch_mode<4, TO>(x, w, out, M, N, K, mode, activation, packing, norm, after, s);
     }
 }
 
@@ -442,7 +442,7 @@ bool xrt_linear_packed_takes_qkv(int M, int N, const Packing& packing, const Qkv
     return packing.kind == XRT_PACK_ROTARY && packing.head_dim == after.head_dim && packing.rotated_heads == rotated;
 }
 
-int xrt_linear_packed(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+int xrt_linear_packed(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, int activation,
                       const Packing* packing, const LinearNorm* norm, const QkvAfter* after, hipStream_t s) {
     const LinearNorm none = {};
     if (norm && !xrt_linear_packed_takes_norm(M)) {
@@ -462,6 +462,6 @@ int xrt_linear_packed(const void* a, const void* w, void* out, int out_dtype, in
         return 1;
     }
     const LinearNorm& around = norm ? *norm : none;
-    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, *packing, around, after, s);
-    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, *packing, around, after, s);
+    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, activation, *packing, around, after, s);
+    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, activation, *packing, around, after, s);
 }

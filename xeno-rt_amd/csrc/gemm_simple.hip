@@ -9,6 +9,7 @@
 // [out][in], no bias.
 #include "common.h"
 #include "xrt_hip.h"
+#include "activation.h"
 
 namespace {
 
@@ -36,14 +37,12 @@ __device__ __forceinline__ void load4(const T* __restrict__ base, long row, int 
     }
 }
 
-__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }   // silu.rs:1-3
-
 // RM rows of the output per thread: a tile is 16 RM x 64. With few rows of a (a decode step) the
 // small tile does a quarter of the arithmetic; an element's sum is the same either way.
 template <typename TI, typename TO, int MODE, int RM>
 __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__ a, const TI* __restrict__ w,
                                                           TO* __restrict__ out, int M, int N, int K,
-                                                          int vector_ok) {
+                                                          int vector_ok, int activation) {
     constexpr int BM = 16 * RM;
     __shared__ __attribute__((aligned(16))) float As[BK][BM + PAD];
     __shared__ __attribute__((aligned(16))) float Ws[BK][BN + PAD];
@@ -116,28 +115,28 @@ __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__
             TO* dst = out + m * (long)N + n;
             if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(acc[i][j]);
             if constexpr (MODE == MODE_ACCUMULATE) *dst = from_float<TO>(before[i][j] + acc[i][j]);
-            if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(silu(acc[i][j]) * acc_up[i][j]);
+            if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(gate_activation(acc[i][j], activation) * acc_up[i][j]);
         }
     }
 }
 
 template <typename TI, typename TO, int RM>
-void launch_rows(const void* a, const void* w, void* out, int M, int N, int K, int mode, hipStream_t s) {
+void launch_rows(const void* a, const void* w, void* out, int M, int N, int K, int mode, int activation, hipStream_t s) {
     constexpr int BM = 16 * RM;
     const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
     const int vector_ok = (K % 4 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
     if (mode == MODE_STORE)
-        gemm_simple_kernel<TI, TO, MODE_STORE, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+        gemm_simple_kernel<TI, TO, MODE_STORE, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok, activation);
     else if (mode == MODE_ACCUMULATE)
-        gemm_simple_kernel<TI, TO, MODE_ACCUMULATE, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+        gemm_simple_kernel<TI, TO, MODE_ACCUMULATE, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok, activation);
     else
-        gemm_simple_kernel<TI, TO, MODE_GATED, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok);
+        gemm_simple_kernel<TI, TO, MODE_GATED, RM><<<grid, 256, 0, s>>>((const TI*)a, (const TI*)w, (TO*)out, M, N, K, vector_ok, activation);
 }
 
 template <typename TI, typename TO>
-int launch(const void* a, const void* w, void* out, int M, int N, int K, int mode, hipStream_t s) {
-    if (M <= 16) launch_rows<TI, TO, 1>(a, w, out, M, N, K, mode, s);
-    else launch_rows<TI, TO, 4>(a, w, out, M, N, K, mode, s);
+int launch(const void* a, const void* w, void* out, int M, int N, int K, int mode, int activation, hipStream_t s) {
+    if (M <= 16) launch_rows<TI, TO, 1>(a, w, out, M, N, K, mode, activation, s);
+    else launch_rows<TI, TO, 4>(a, w, out, M, N, K, mode, activation, s);
     XRT_LAUNCH_CHECK("linear (plain)");
     return 0;
 }
@@ -145,10 +144,10 @@ int launch(const void* a, const void* w, void* out, int M, int N, int K, int mod
 }  // namespace
 
 int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
-                     int mode, hipStream_t s) {
-    if (dtype == XRT_F32 && out_dtype == XRT_F32) return launch<float, float>(a, w, out, M, N, K, mode, s);
-    if (dtype == XRT_BF16 && out_dtype == XRT_F32) return launch<bf16, float>(a, w, out, M, N, K, mode, s);
-    if (dtype == XRT_BF16 && out_dtype == XRT_BF16) return launch<bf16, bf16>(a, w, out, M, N, K, mode, s);
+                     int mode, int activation, hipStream_t s) {
+    if (dtype == XRT_F32 && out_dtype == XRT_F32) return launch<float, float>(a, w, out, M, N, K, mode, activation, s);
+    if (dtype == XRT_BF16 && out_dtype == XRT_F32) return launch<bf16, float>(a, w, out, M, N, K, mode, activation, s);
+    if (dtype == XRT_BF16 && out_dtype == XRT_BF16) return launch<bf16, bf16>(a, w, out, M, N, K, mode, activation, s);
     xrt_set_error("linear: unsupported dtypes in=%d out=%d", dtype, out_dtype);
     return 1;
 }

@@ -18,5 +18,6 @@ bool xrt_linear_skinny_takes_norm(int M);
 int xrt_linear_skinny_norm_tiles(int N);
 bool xrt_linear_skinny_takes_qkv(int M, int N, const QkvAfter& after);
 // norm and after may be null; with `after`, out is the bfloat16 q/k/v buffer and mode is 0
-int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+// activation: the XRT_ACT_* code of a gated product (mode 2), unused otherwise
+int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, int activation,
                       const xrt_linear_norm* norm, const QkvAfter* after, hipStream_t s);

@@ -29,6 +29,7 @@
 #include "common.h"
 #include "xrt_hip.h"
 #include "gemm_skinny.h"
+#include "activation.h"
 
 namespace {
 
@@ -42,7 +43,6 @@ constexpr int KSTEP = 64;         // K covered by one step of a wavefront
 constexpr int JL = KSTEP / 32;   // load instructions per operand tile and step: 4 lane groups x 8 elements each
 enum { MODE_STORE = 0, MODE_ACCUMULATE = 1, MODE_GATED = 2 };
 
-__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 
 // MT: tiles of 16 rows of x; RT: tiles of 16 rows of w per wavefront; GATED doubles the w tiles.
 // With one tile of x (the common decode case) the kernel is held to 128 registers at most (it takes
@@ -54,7 +54,7 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 template <int MT, int RT, int MODE, typename TO, int EXTRA = 0>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skinny_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K, int given_rows,
-    const LinearNorm norm, const QkvAfter after) {
+    const LinearNorm norm, const QkvAfter after, int activation) {
     // given_rows: rows of w that a workgroup's tile holds, 16 or fewer (with RT == 1): the host picks them so
     // that the workgroups divide evenly among the compute units. Lanes beyond read the tile's last row again.
     // After a q/k/v projection the tiles of the query heads have 16 rows and come first; those of the key
@@ -413,7 +413,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                         fresh[i] = to_float(*dst) + g[i];
                         *dst = from_float<TO>(fresh[i]);
                     }
-                    if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(silu(g[i]) * u[i]);
+                    if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(gate_activation(g[i], activation) * u[i]);
                 }
             }
             if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
@@ -457,7 +457,7 @@ int balanced_rows(int N, int mode) {
 }
 
 template <int MT, int RT, typename TO>
-int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
+int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, int activation, const LinearNorm& norm,
                 const QkvAfter* after, hipStream_t s) {
     const int rows = RT == 1 && !after ? balanced_rows(N, mode) : 16;
     unsigned grid = (unsigned)(RT == 1 ? (N + rows - 1) / rows : (N + 16 * RT - 1) / (16 * RT));
@@ -480,17 +480,17 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
     if constexpr (MT == 1 && RT == 1) {
         if (after) {
             if constexpr (sizeof(TO) == 2) {
-                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, then);
+                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, then, activation);
                 XRT_LAUNCH_CHECK("linear (skinny, q/k/v)");
                 return 0;
             }
         } else if (norm.squares_in || norm.squares_out) {
             if (mode == MODE_STORE)
-                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
+                gemm_skinny_kernel<1, 1, MODE_STORE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none, activation);
             else if (mode == MODE_ACCUMULATE)
-                gemm_skinny_kernel<1, 1, MODE_ACCUMULATE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
+                gemm_skinny_kernel<1, 1, MODE_ACCUMULATE, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none, activation);
             else
-                gemm_skinny_kernel<1, 1, MODE_GATED, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
+                gemm_skinny_kernel<1, 1, MODE_GATED, TO, 1><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none, activation);
             XRT_LAUNCH_CHECK("linear (skinny, with norm)");
             return 0;
         }
@@ -500,11 +500,11 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
         return 1;
     }
     if (mode == MODE_STORE)
-        gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
+        gemm_skinny_kernel<MT, RT, MODE_STORE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none, activation);
     else if (mode == MODE_ACCUMULATE)
-        gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
+        gemm_skinny_kernel<MT, RT, MODE_ACCUMULATE, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none, activation);
     else if constexpr (RT == 1)
-        gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none);
+        gemm_skinny_kernel<MT, RT, MODE_GATED, TO><<<grid, block, 0, s>>>(x, w, out, M, N, K, rows, norm, none, activation);
     else {
         xrt_set_error("linear (skinny): a gated product takes one row tile per wavefront");
         return 1;
@@ -514,7 +514,7 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
 }
 
 template <typename TO>
-int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, const LinearNorm& norm,
+int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, int activation, const LinearNorm& norm,
                  const QkvAfter* after, hipStream_t s) {
     const int mt = (M + 15) / 16;
     // two row tiles per wavefront keep more loads in flight and halve the reads of x, if enough
@@ -523,7 +523,7 @@ int launch_tiles(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int
     // the wider tile pays as soon as it leaves most compute units a workgroup)
     const bool around = norm.squares_in || norm.squares_out || after;
     const bool wide = !around && mode != MODE_GATED && (N / 32) >= (mt >= 3 ? 160 : 1024);
-#define XRT_SKINNY(MT_) (wide ? launch_mode<MT_, 2, TO>(x, w, out, M, N, K, mode, norm, after, s) : launch_mode<MT_, 1, TO>(x, w, out, M, N, K, mode, norm, after, s))
+#define XRT_SKINNY(MT_) (wide ? launch_mode<MT_, 2, TO>(x, w, out, M, N, K, mode, activation, norm, after, s) : launch_mode<MT_, 1, TO>(x, w, out, M, N, K, mode, activation, norm, after, s))
     switch (mt) {
         case 1: return XRT_SKINNY(1);
         case 2: return XRT_SKINNY(2);
@@ -552,7 +552,7 @@ bool xrt_linear_skinny_takes_qkv(int M, int N, const QkvAfter& after) {
            (after.rope_theta == nullptr || (after.rope_dim % 16 == 0 && after.rope_dim <= after.head_dim));
 }
 
-int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, int activation,
                       const LinearNorm* norm, const QkvAfter* after, hipStream_t s) {
     const LinearNorm none = {};
     if (norm && !xrt_linear_skinny_takes_norm(M)) {
@@ -564,6 +564,6 @@ int xrt_linear_skinny(const void* a, const void* w, void* out, int out_dtype, in
         return 1;
     }
     const LinearNorm& around = norm ? *norm : none;
-    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, around, after, s);
-    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, around, after, s);
+    if (out_dtype == XRT_F32) return launch_tiles<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, activation, around, after, s);
+    return launch_tiles<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, activation, around, after, s);
 }

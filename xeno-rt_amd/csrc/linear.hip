@@ -1,11 +1,12 @@
 // Entry point of all matrix products: checks the operands and picks the kernel.
 #include "packing.h"
 #include "gemm_skinny.h"
+#include "activation.h"
 
 int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
-                     int mode, hipStream_t s);
+                     int mode, int activation, hipStream_t s);
 bool xrt_linear_mfma_accepts(const void* a, const void* w, int M, int N, int K, int mode);
-int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, int activation,
                     const Packing& packing, hipStream_t s);
 
 bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats);
@@ -13,13 +14,13 @@ bool xrt_linear_split_takes_norm(const void* a, const void* w, int M, int N, int
 bool xrt_linear_split_takes_qkv(const void* a, const void* w, int M, int N, int K, const QkvAfter& after, long* workspace_floats);
 int xrt_linear_split_qkv(const void* a, const void* w, void* qkv, int M, int N, int K, const Packing& packing, float* workspace,
                          const xrt_linear_norm* norm, const QkvAfter& after, hipStream_t s);
-int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, const Packing& packing,
-                     float* workspace, const xrt_linear_norm* norm, hipStream_t s);
+int xrt_linear_split(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, int activation,
+                     const Packing& packing, float* workspace, const xrt_linear_norm* norm, hipStream_t s);
 
 bool xrt_linear_packed_accepts(const void* a, const void* w, int M, int K, int mode, const Packing* packing);
 bool xrt_linear_packed_takes_norm(int M);
 bool xrt_linear_packed_takes_qkv(int M, int N, const Packing& packing, const QkvAfter& after);
-int xrt_linear_packed(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode,
+int xrt_linear_packed(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int mode, int activation,
                       const Packing* packing, const xrt_linear_norm* norm, const QkvAfter* after, hipStream_t s);
 
 static const Packing ROWS_ALONG_K = {XRT_PACK_NONE, 0, 0, 0};
@@ -52,6 +53,11 @@ extern "C" int xrt_linear(const void* a, const void* w, int dtype, void* out, in
 
 extern "C" int xrt_linear_with(const void* a, const void* w, const xrt_packing* packing, int dtype, void* out, int out_dtype,
                                int M, int N, int K, int mode, float* workspace, long workspace_floats, void* stream) {
+    // a gated product carries its activation's code above the mode's low byte
+    const int activation = mode >= 0 ? activation_of(mode) : 0;
+    XRT_REQUIRE(activation >= 0 && activation < XRT_ACT_COUNT && (activation == 0 || mode_of(mode) == 2),
+                "linear: unknown activation %d in mode %d", activation, mode);
+    if (mode >= 0) mode = mode_of(mode);
     XRT_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
     XRT_REQUIRE(mode >= 0 && mode <= 2, "linear: unknown mode %d", mode);
     XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "linear: unknown dtype %d", dtype);
@@ -69,7 +75,7 @@ extern "C" int xrt_linear_with(const void* a, const void* w, const xrt_packing* 
         const long out_row = (long)N * (out_dtype == XRT_F32 ? 4 : 2);
         for (int m0 = 0; m0 < M; m0 += run) {
             const int status = xrt_linear_with((const char*)a + (long)m0 * K * 2, w, packing, dtype, (char*)out + m0 * out_row, out_dtype,
-                                               M - m0 < run ? M - m0 : run, N, K, mode, workspace, workspace_floats, stream);
+                                               M - m0 < run ? M - m0 : run, N, K, mode | (activation << 8), workspace, workspace_floats, stream);
             if (status != 0) return status;
         }
         return 0;
@@ -78,16 +84,16 @@ extern "C" int xrt_linear_with(const void* a, const void* w, const xrt_packing* 
     if (dtype == XRT_BF16) {
         long need = 0;
         if (xrt_linear_split_takes(a, w, M, N, K, mode, &need) && (need == 0 || (workspace != nullptr && workspace_floats >= need)))
-            return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, layout, workspace, nullptr, (hipStream_t)stream);
+            return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, activation, layout, workspace, nullptr, (hipStream_t)stream);
     }
     if (xrt_linear_packed_accepts(a, w, M, K, mode, packing))
-        return xrt_linear_packed(a, w, out, out_dtype, M, N, K, mode, packing, nullptr, nullptr, (hipStream_t)stream);
+        return xrt_linear_packed(a, w, out, out_dtype, M, N, K, mode, activation, packing, nullptr, nullptr, (hipStream_t)stream);
     if (dtype == XRT_BF16 && !is_packed(layout) && xrt_linear_skinny_accepts(a, w, M, K))
-        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, nullptr, nullptr, (hipStream_t)stream);
+        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, activation, nullptr, nullptr, (hipStream_t)stream);
     if (dtype == XRT_BF16 && xrt_linear_mfma_accepts(a, w, M, N, K, mode))
-        return xrt_linear_mfma(a, w, out, out_dtype, M, N, K, mode, layout, (hipStream_t)stream);
+        return xrt_linear_mfma(a, w, out, out_dtype, M, N, K, mode, activation, layout, (hipStream_t)stream);
     XRT_REQUIRE(!is_packed(layout), "linear: M=%d N=%d K=%d is beyond what the kernels for a packed w take", M, N, K);
-    return xrt_linear_plain(a, w, dtype, out, out_dtype, M, N, K, mode, (hipStream_t)stream);
+    return xrt_linear_plain(a, w, dtype, out, out_dtype, M, N, K, mode, activation, (hipStream_t)stream);
 }
 
 extern "C" int xrt_linear_takes_norm(const void* a, const void* w, const xrt_packing* packing, int dtype, int M, int N, int K, int mode) {
@@ -114,6 +120,10 @@ extern "C" int xrt_linear_normed(const void* a, const void* w, const xrt_packing
                                  int M, int N, int K, int mode, const xrt_linear_norm* norm, float* workspace,
                                  long workspace_floats, void* stream) {
     XRT_REQUIRE(a && w && out && norm, "linear with norm: null operand");
+    const int activation = mode >= 0 ? activation_of(mode) : 0;
+    XRT_REQUIRE(activation >= 0 && activation < XRT_ACT_COUNT && (activation == 0 || mode_of(mode) == 2),
+                "linear with norm: unknown activation %d in mode %d", activation, mode);
+    if (mode >= 0) mode = mode_of(mode);
     if (check_packing(packing, dtype, N, K, mode) != 0) return 1;
     const Packing& layout = packing_of(packing);
     XRT_REQUIRE(dtype == XRT_BF16 && M >= 1 && N > 0 && K > 0 && mode >= 0 && mode <= 2,
@@ -133,15 +143,15 @@ extern "C" int xrt_linear_normed(const void* a, const void* w, const xrt_packing
     }
     if (is_packed(layout) && xrt_linear_packed_accepts(a, w, M, K, mode, packing) && xrt_linear_packed_takes_norm(M)) {
         XRT_REQUIRE(mode != 1 || layout.kind == XRT_PACK_TILES, "linear with norm: an accumulating product takes a w packed in plain tiles");
-        return xrt_linear_packed(a, w, out, out_dtype, M, N, K, mode, packing, norm, nullptr, (hipStream_t)stream);
+        return xrt_linear_packed(a, w, out, out_dtype, M, N, K, mode, activation, packing, norm, nullptr, (hipStream_t)stream);
     }
     if (!is_packed(layout) && xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_norm(M))
-        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, norm, nullptr, (hipStream_t)stream);
+        return xrt_linear_skinny(a, w, out, out_dtype, M, N, K, mode, activation, norm, nullptr, (hipStream_t)stream);
     long need = 0;
     XRT_REQUIRE(M <= 64 && xrt_linear_split_takes(a, w, M, N, K, mode, &need),
                 "linear with norm: M=%d N=%d K=%d is not a product that takes it", M, N, K);
     XRT_REQUIRE(need == 0 || (workspace != nullptr && workspace_floats >= need), "linear with norm: the workspace needs %ld floats", need);
-    return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, layout, workspace, norm, (hipStream_t)stream);
+    return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, activation, layout, workspace, norm, (hipStream_t)stream);
 }
 
 extern "C" int xrt_linear_qkv(const void* a, const void* w, const xrt_packing* packing, int dtype, void* qkv, int M, int K,
@@ -164,9 +174,9 @@ extern "C" int xrt_linear_qkv(const void* a, const void* w, const xrt_packing* p
         (k_cache == nullptr || (block_table && slots && table_stride > 0 && n_blocks > 0)) &&
         (rope_theta == nullptr || rope_dim > 0);
     if (one_kernel && is_packed(layout) && xrt_linear_packed_accepts(a, w, M, K, 0, packing) && xrt_linear_packed_takes_qkv(M, N, layout, after))
-        return xrt_linear_packed(a, w, qkv, XRT_BF16, M, N, K, 0, packing, norm, &after, (hipStream_t)stream);
+        return xrt_linear_packed(a, w, qkv, XRT_BF16, M, N, K, 0, XRT_ACT_SILU, packing, norm, &after, (hipStream_t)stream);
     if (one_kernel && !is_packed(layout) && xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_qkv(M, N, after))
-        return xrt_linear_skinny(a, w, qkv, XRT_BF16, M, N, K, 0, norm, &after, (hipStream_t)stream);
+        return xrt_linear_skinny(a, w, qkv, XRT_BF16, M, N, K, 0, XRT_ACT_SILU, norm, &after, (hipStream_t)stream);
     // 17 to 64 tokens, the product split along k: the kernel that adds the partial sums does the rest
     long need = 0;
     if (dtype == XRT_BF16 && a && w && qkv && M > 0 && K > 0 && !q_norm && !k_norm && positions &&

@@ -28,7 +28,9 @@ namespace {
 constexpr int THREADS = 1024;
 constexpr int BLOCK_WAVES = THREADS / XRT_WAVE;
 constexpr int IN_FLIGHT = 16;          // loads of a thread that a pass keeps in flight
-constexpr int MAX_VOCAB = 255 * THREADS;   // a thread sees at most 255 tokens (8-bit counters below); the seen-bitmap takes vocab/8 bytes of LDS
+constexpr int MAX_VOCAB = 255 * THREADS;   // the largest vocabulary that goes through slices (one lane per slice below)
+constexpr int LARGEST_VOCAB = 1 << 19;     // the largest vocabulary at all: its seen-bitmap, vocab / 8 bytes, fits the LDS of a compute unit beside the rest
+constexpr int COUNTED_AT_ONCE = 240;       // keys that a thread counts in 8-bit counters before it empties them
 constexpr int SEGMENT = 128;           // survivors of top-k that one wavefront's run of ids may hold in LDS
 constexpr int CANDIDATES = 15;         // thresholds tried per pass: the non-zero values of four bits
 
@@ -175,7 +177,7 @@ __device__ void sample_row(
     // ---- top-k: the largest key T with count(key >= T) >= k ---------------------
     // Found four bits at a time from the top. With the bits above already fixed in `low`, a pass
     // counts, among the keys that share those bits, how many have each value of the next four
-    // (sixteen 8-bit counters packed into two registers: a thread sees at most 255 keys), and
+    // (sixteen 8-bit counters packed into two registers, emptied before any of them can reach 256), and
     // how many keys lie above altogether. The largest value whose keys, with everything above
     // them, number at least k fixes the next four bits.
     unsigned k_threshold = 0u;
@@ -186,6 +188,16 @@ __device__ void sample_row(
             unsigned long long packed_low = 0ull, packed_high = 0ull;
             unsigned above = 0u;
             const unsigned fixed_bits = shift == 28 ? 0u : low >> (shift + 4);
+            unsigned count[SUMS] = {};
+            auto empty_counters = [&]() {
+#pragma unroll
+                for (int d = 0; d < 8; ++d) {
+                    count[d] += (unsigned)(packed_low >> (d * 8)) & 255u;
+                    count[8 + d] += (unsigned)(packed_high >> (d * 8)) & 255u;
+                }
+                packed_low = packed_high = 0ull;
+            };
+            int counted = 0;
             row.each([&](int, float v) {
                 const unsigned key = order_key(v);
                 const unsigned upper = shift == 28 ? 0u : key >> (shift + 4);
@@ -196,13 +208,12 @@ __device__ void sample_row(
                 } else if (upper > fixed_bits) {
                     above += 1u;
                 }
+                if (++counted == COUNTED_AT_ONCE) {             // (only vocabularies beyond 245 760 get here)
+                    empty_counters();
+                    counted = 0;
+                }
             });
-            unsigned count[SUMS];
-#pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                count[d] = (unsigned)(packed_low >> (d * 8)) & 255u;
-                count[8 + d] = (unsigned)(packed_high >> (d * 8)) & 255u;
-            }
+            empty_counters();
             count[16] = above;
             block_sums(count, scratch_u);
             unsigned at_or_above = count[16], digit = 0u;
@@ -844,13 +855,24 @@ extern "C" int xrt_sample(const float* logits, int rows, int vocab, int* out, co
                           long workspace_bytes, void* stream) {
     XRT_REQUIRE(rows >= 0, "sample: negative row count");
     XRT_REQUIRE(vocab > 0, "sample: cannot sample from an empty logits vector");          // sampler.rs:56-60
-    XRT_REQUIRE(vocab <= MAX_VOCAB, "sample: vocabulary %d exceeds %d", vocab, MAX_VOCAB);
+    XRT_REQUIRE(vocab <= LARGEST_VOCAB, "sample: vocabulary %d exceeds %d", vocab, LARGEST_VOCAB);
     XRT_REQUIRE(logits && out && temperature && top_k && top_p && penalty && history_spans && uniforms,
                 "sample: null operand");
     XRT_REQUIRE(append_at == nullptr || history != nullptr, "sample: tokens to append and no history to append them to");
     if (rows == 0) return 0;
     const Chosen chosen{out, history, append_at};
     const size_t lds = (size_t)((vocab + 31) / 32) * sizeof(unsigned);
+    if (lds > 32 * 1024) {
+        // a bitmap of seen tokens beyond what a kernel may take of LDS without asking
+        static bool configured = false;
+        if (!configured) {
+            for (const void* kernel : {reinterpret_cast<const void*>(sample_kernel), reinterpret_cast<const void*>(sample_candidates_kernel)}) {
+                hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LARGEST_VOCAB / 8);
+                XRT_REQUIRE(e == hipSuccess, "sample: cannot reserve %d bytes of LDS: %s", LARGEST_VOCAB / 8, hipGetErrorString(e));
+            }
+            configured = true;
+        }
+    }
     const long need = xrt_sample_workspace(rows, vocab);
     if (workspace != nullptr && need > 0 && workspace_bytes >= need) {
         const int slices = (vocab + SLICE - 1) / SLICE;

@@ -9,6 +9,10 @@ extern "C" {
 
 const char* xrt_last_error(void);
 
+// tokens in one block of the cache: keys [kv_head][token][dim], values [kv_head][dim][token] inside a block.
+// Whoever keeps the block tables must count in the same blocks.
+int xrt_block_tokens(void);
+
 // How a bfloat16 weight matrix w[rows][K] is laid out. XRT_PACK_NONE (or a null pointer wherever a packing
 // is passed): rows contiguous along k. Otherwise tiles of 16 rows x 32 columns in the order in which the matrix
 // cores take them, rows padded to a multiple of 16 with zeros, K a multiple of 32; the rows may also be
@@ -52,7 +56,10 @@ int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype, float eps,
                 const int* rows, int n_rows, int hidden, void* stream);
 
 // out[m, n] (+)= sum_k a[m, k] * w[n, k]   (mode 0 store, 1 accumulate into float32 out,
-// 2 gated: out[m, n] = silu(a.w[n]) * (a.w[n + N]) with w of 2N rows)
+// 2 gated: out[m, n] = act(a.w[n]) * (a.w[n + N]) with w of 2N rows; the activation's code rides above the
+// mode's low byte, XRT_GATED(XRT_ACT_SILU) == 2: silu(z) = z / (1 + exp(-z)) is the one that exists)
+#define XRT_ACT_SILU 0
+#define XRT_GATED(activation) (2 | ((activation) << 8))
 // Some products (17 to 64 rows of a, or more rows and a narrow w) run faster split along k, through a workspace of float32
 // sums: xrt_linear_workspace says how many floats that takes (0: none); without it the product
 // takes another kernel.

@@ -31,6 +31,7 @@ def _ptr(tensor: Optional[torch.Tensor]):
     return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
 
 
+ACTIVATIONS = {"silu": 0}   # gate activations of the gated product: name -> XRT_ACT_* code of the library
 SQUARES_STRIDE = 64         # rows of a table of sums of squares (XRT_SQUARES_STRIDE of the library)
 
 
@@ -132,8 +133,12 @@ class HipOps:
         self.lib.xrt_last_error.restype = ctypes.c_char_p
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
                      "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv", "xrt_random_normal",
-                     "xrt_linear_with", "xrt_pack_weight", "xrt_packing_suits"):
+                     "xrt_linear_with", "xrt_pack_weight", "xrt_packing_suits", "xrt_block_tokens"):
             getattr(self.lib, name).restype = ctypes.c_int
+        from ..cache.allocator import BLOCK_TOKENS
+        if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
+            raise KernelError(f"{path} keeps {int(self.lib.xrt_block_tokens())} tokens in a cache block, "
+                              f"the cache's bookkeeping {BLOCK_TOKENS}: library and package do not belong together")
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
         self.lib.xrt_attention_workspace.restype = ctypes.c_long
         self.lib.xrt_probe_read_bytes.restype = ctypes.c_long
@@ -233,7 +238,8 @@ class HipOps:
         self._check(self.lib.xrt_rmsnorm(_ptr(x), _ptr(weight), _code(weight), ctypes.c_float(eps), _ptr(out),
                                          _code(out), _ptr(rows), n_rows, hidden, self._stream(x)))
 
-    def _linear(self, a, w, out, mode, n, then_norm=None):
+    def _linear(self, a, w, out, coded_mode, n, then_norm=None):
+        mode = coded_mode & 255                 # what rides above is a gated product's activation
         scaled = a if isinstance(a, Prescaled) else None
         if scaled is not None:
             a = scaled.values
@@ -271,12 +277,12 @@ class HipOps:
                 norm.gain, norm.gain_dtype = then_norm[0].data_ptr(), _code(then_norm[0])
             need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
             workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
-            self._check(self.lib.xrt_linear_normed(*packed, _ptr(out), _code(out), m, n, k, mode, ctypes.byref(norm),
+            self._check(self.lib.xrt_linear_normed(*packed, _ptr(out), _code(out), m, n, k, coded_mode, ctypes.byref(norm),
                                                    _ptr(workspace), ctypes.c_long(need), self._stream(a)))
             return emit
         need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
-        self._check(self.lib.xrt_linear_with(*packed, _ptr(out), _code(out), m, n, k, mode,
+        self._check(self.lib.xrt_linear_with(*packed, _ptr(out), _code(out), m, n, k, coded_mode,
                                              _ptr(workspace), ctypes.c_long(need), self._stream(a)))
         return None
 
@@ -286,10 +292,13 @@ class HipOps:
         product after the norm; None means that the caller runs the norm."""
         return self._linear(a, w, out, 1 if accumulate else 0, w.shape[0], then_norm)
 
-    def linear_glu(self, a, w_gate_up, out):
+    def linear_glu(self, a, w_gate_up, out, activation: str = "silu"):
+        """out = act(a w_gate^T) * (a w_up^T) with w_gate_up = [gate rows | up rows]."""
         if w_gate_up.shape[0] % 2 != 0:
             raise KernelError("linear_glu: the weight needs gate rows followed by as many up rows")
-        self._linear(a, w_gate_up, out, 2, w_gate_up.shape[0] // 2)
+        if activation not in ACTIVATIONS:
+            raise KernelError(f"linear_glu: activation must be one of {sorted(ACTIVATIONS)}, found {activation!r}")
+        self._linear(a, w_gate_up, out, 2 | (ACTIVATIONS[activation] << 8), w_gate_up.shape[0] // 2)
 
     def _prepare_arguments(self, qkv, n_heads, n_kv_heads, head_dim, positions, slots, q_norm, k_norm, norm_eps,
                            rope_theta, rope_dim, rope_scale, kv, longest_run):
@@ -356,6 +365,10 @@ class HipOps:
         from ..cache import BLOCK_TOKENS
         n_blocks = kv.k.shape[0]
         self._require(kv.k, "key cache", like.dtype, (n_blocks, n_kv_heads, BLOCK_TOKENS, head_dim), like)
+        if kv.v.dim() == 4 and kv.v.shape[2] != head_dim:
+            raise KernelError(f"value cache: values of width {kv.v.shape[2]} beside keys of width {head_dim}: the attention "
+                              "kernels of this library take values as wide as the keys (a mixer whose values differ "
+                              "brings its own kernel and reads the cache's tensors itself)")
         self._require(kv.v, "value cache", like.dtype, (n_blocks, n_kv_heads, head_dim, BLOCK_TOKENS), like)
         self._require(kv.block_table, "block table", torch.int32, None, like)
         if kv.block_table.dim() != 2:

@@ -36,7 +36,8 @@ class WeightSpec:
 
 @dataclass(frozen=True)
 class KVSpec:
-    """Keys and values for every token: rows of n_kv_heads x head_dim.
+    """Keys and values for every token: n_kv_heads rows of head_dim (keys) and of value_dim (values;
+    as wide as the keys unless given).
 
     window = None keeps all tokens; window = W keeps what a query can still see
     when it looks at the W most recent tokens (itself included).
@@ -44,6 +45,11 @@ class KVSpec:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)

@@ -50,7 +50,7 @@ class GatedMLP(FeedForward):
         rt = self.runtime
         tokens = h.shape[0]
         act = rt.empty((tokens, self.intermediate))
-        rt.ops.linear_glu(h, self.w_gate_up, act)
+        rt.ops.linear_glu(h, self.w_gate_up, act, activation=self.activation)
         return rt.ops.linear(act, self.w_down, residual, accumulate=True,
                              then_norm=None if then is None else then.row_scale())
 
