@@ -815,3 +815,87 @@ def test_sample_rows_are_independent(ops):
     alone = [sample(ops, logits[r:r + 1].contiguous(), 0.9, 50, 0.9, 1.0, draws=[u[r]])[0] for r in range(5)]
     assert together == alone
 
+
+
+# ---- every kernel once more, against the plain C++ references -------------------------------------
+
+@pytest.fixture(scope="module")
+def cpp():
+    from reference_cpp import CppReference
+    return CppReference()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_elementwise_and_products_against_the_cpp_references(ops, cpp, dtype):
+    table, ids = rand(333, 96, dtype=DT[dtype], seed=1), i32([0, 332, 7, 7])
+    out = torch.empty(4, 96, device=DEV)
+    ops.embed(table, ids, out)
+    assert torch.equal(out.cpu(), cpp.embed(table, ids))
+    x, gain = rand(6, 1000, seed=2, scale=3.0), (rand(1000, seed=3) + 1.0).to(DT[dtype])
+    normed = torch.empty(6, 1000, dtype=DT[dtype], device=DEV)
+    ops.rmsnorm(x, gain, 1e-4, normed)
+    assert rel(normed.float().cpu(), cpp.rmsnorm(x, gain, 1e-4)) < ULP[dtype]
+    for m, n, k in ((3, 40, 96), (16, 176, 64), (40, 520, 256), (300, 130, 192)):
+        a, w = rand(m, k, dtype=DT[dtype], seed=m), rand(2 * n, k, dtype=DT[dtype], seed=n, scale=0.2)
+        stored = torch.empty(m, 2 * n, device=DEV)
+        ops.linear(a, w, stored)
+        assert rel(stored.cpu(), cpp.linear(a, w)) < 2e-5
+        base = rand(m, 2 * n, seed=9)
+        summed = base.clone()
+        ops.linear(a, w, summed, accumulate=True)
+        assert rel(summed.cpu(), cpp.linear(a, w, base=base)) < 2e-5
+        gated = torch.empty(m, n, dtype=DT[dtype], device=DEV)
+        ops.linear_glu(a, w, gated)
+        assert rel(gated.float().cpu(), cpp.linear_glu(a, w)) < ULP[dtype] * 2
+        if dtype == "bfloat16" and k % 32 == 0 and n % 8 == 0:          # the same from packed weights; and the packing itself
+            ops.linear_glu(a, ops.pack(w, "gated", gated_n=n), gated)
+            assert rel(gated.float().cpu(), cpp.linear_glu(a, w)) < ULP[dtype] * 2
+            assert torch.equal(ops.pack(w, "gated", gated_n=n).data.float().cpu(), cpp.pack(w, kind=2, gated_n=n))
+            assert torch.equal(ops.pack(w, "rotary", head_dim=16, rotated_heads=n // 16).data.float().cpu(),
+                               cpp.pack(w, kind=3, head_dim=16, rotated_heads=n // 16))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 32), (8, 2, 128), (6, 3, 64)])
+def test_preparation_and_attention_against_the_cpp_references(ops, cpp, dtype, nh, nkv, hd):
+    """A prompt of 150 tokens, then one token more (the matrix-core kernels in bfloat16 at head sizes 64 and 128,
+    the general kernel otherwise): the rows and the cache after the preparation, and the attention's output."""
+    width, eps = (nh + 2 * nkv) * hd, 1e-4
+    theta = (torch.tensor(10000.0) ** (torch.arange(hd // 2) * 2.0 / hd))
+    qn, kn = rand(hd, seed=1).cpu() + 1.0, rand(hd, seed=2).cpu() + 1.0
+    kv = make_cache(5, nkv, hd, DT[dtype], 1, 4)
+    kv.block_table[0, :3] = i32([4, 1, 2])
+    host_k, host_v = torch.zeros(5, nkv, 64, hd), torch.zeros(5, nkv, hd, 64)
+    tol = 3e-5 if dtype == "float32" else ULP[dtype]
+    for count, start in ((150, 0), (1, 150)):
+        batch = described([0], [count], [start])
+        qkv = rand(count, width, dtype=DT[dtype], seed=count)
+        want = cpp.qkv_prepare(qkv, nh, nkv, hd, batch.positions, batch.slots, qn, kn, eps, theta, hd, 1.0,
+                               kv=(host_k, host_v, kv.block_table.cpu()))
+        ops.qkv_prepare(qkv, nh, nkv, hd, batch.positions, batch.slots, q_norm=qn.to(DEV), k_norm=kn.to(DEV), norm_eps=eps,
+                        rope_theta=theta.to(DEV), rope_dim=hd, kv=kv, longest_run=count)
+        assert rel(qkv.float().cpu(), want) < tol
+        assert rel(kv.k.float().cpu(), host_k) < tol and rel(kv.v.float().cpu(), host_v) < tol
+        out = torch.empty(count, nh * hd, dtype=DT[dtype], device=DEV)
+        ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=1.0 / math.sqrt(hd))
+        # the reference on exactly what the kernel read: the prepared rows and the cache as the device holds them
+        expected = cpp.attention(qkv, nh, nkv, hd, kv.k, kv.v, kv.block_table, batch.positions, batch.slots, 1.0 / math.sqrt(hd))
+        assert rel(out.float().cpu(), expected) < (2e-5 if dtype == "float32" else 2e-2)
+
+
+def test_sampling_and_random_weights_against_the_cpp_references(ops, cpp):
+    from xeno_rt_amd.weights import random_init
+    vocab, rows = 5000, 64
+    logits = rand(rows, vocab, seed=5, scale=2.0)
+    history = [3, 7, 7, vocab - 1]
+    u = ((torch.arange(rows) + 0.5) / rows).tolist()
+    for temperature, top_k, top_p, penalty in [(0.0, 0, 1.0, 1.0), (1.0, 0, 1.0, 1.0), (0.7, 40, 0.95, 1.1), (1.5, 5, 1.0, 2.0)]:
+        got = sample(ops, logits, temperature, top_k, top_p, penalty, history, draws=u)
+        want = cpp.sample(logits, [temperature] * rows, [top_k] * rows, [top_p] * rows, [penalty] * rows,
+                          history * rows, [len(history) * (r + e) for r in range(rows) for e in (0, 1)], u)
+        # weights are summed in another order: a draw that falls on the edge between two tokens may take the neighbour
+        assert sum(a != b for a, b in zip(got, want)) <= 1, (temperature, top_k, top_p, penalty)
+    key = random_init.tensor_key(3, "w")
+    out = torch.empty(100000, device=DEV)
+    ops.random_normal(out, key, random_init.normal_scale(0.02), 0.0)
+    assert torch.equal(out.cpu(), cpp.random_normal(100000, key, random_init.normal_scale(0.02)))

@@ -128,5 +128,74 @@ def build(verbose: bool = True) -> str:
     return library
 
 
+# ---- the plain C++ references of the kernels (csrc/reference/): host code, built with the host compiler ----------
+
+REFERENCE = os.path.join(CSRC, "reference")
+REFERENCE_LIBRARY = "libxrt_ref.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-Wall", "-Wextra"]
+SANITIZE_FLAGS = ["-O1", "-g", "-std=c++17", "-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-static-libasan"]
+
+
+def _host_compiler() -> str:
+    for name in ("g++", "c++", "clang++"):
+        found = shutil.which(name)
+        if found:
+            return found
+    raise BuildError("no host C++ compiler found: the plain C++ references cannot be compiled")
+
+
+def reference_hash() -> str:
+    digest = hashlib.sha256()
+    for name in sorted(os.listdir(REFERENCE)):
+        with open(os.path.join(REFERENCE, name), "rb") as handle:
+            digest.update(name.encode())
+            digest.update(handle.read())
+    return digest.hexdigest()[:16]
+
+
+def find_reference_library():
+    wanted = reference_hash()
+    for folder in library_folders():
+        path = os.path.join(folder, REFERENCE_LIBRARY)
+        stamp = path + ".hash"
+        if os.path.isfile(path) and os.path.isfile(stamp) and open(stamp).read().strip() == wanted:
+            return path
+    return None
+
+
+def build_reference(verbose: bool = True) -> str:
+    """Compile csrc/reference/reference.cpp for the CPU into a shared library of its own; returns its path."""
+    folder = next((f for f in library_folders() if _writable(f)), None)
+    if folder is None:
+        raise BuildError("no writable folder for the reference library")
+    library = os.path.join(folder, REFERENCE_LIBRARY)
+    partial = library + f".{os.getpid()}.tmp"
+    done = subprocess.run([_host_compiler(), *HOST_FLAGS, "-fPIC", "-shared", "-o", partial,
+                           os.path.join(REFERENCE, "reference.cpp")], capture_output=True, text=True)
+    if done.returncode != 0:
+        raise BuildError(f"compiling the C++ references failed:\n{done.stderr}")
+    os.replace(partial, library)
+    with open(library + ".hash", "w") as handle:
+        handle.write(reference_hash() + "\n")
+    if verbose:
+        print(f"[xrt build] built {library}", file=sys.stderr, flush=True)
+    return library
+
+
+def build_reference_selftest(sanitize: bool = True) -> str:
+    """Compile the references with their self-test (csrc/reference/selftest.cpp) into a program, under the host's
+    address and undefined-behaviour sanitizers unless told otherwise; returns its path."""
+    folder = os.path.join(next((f for f in library_folders() if _writable(f)), tempfile.gettempdir()), "_build")
+    os.makedirs(folder, exist_ok=True)
+    program = os.path.join(folder, "reference_selftest" + ("_sanitized" if sanitize else ""))
+    flags = SANITIZE_FLAGS if sanitize else HOST_FLAGS
+    done = subprocess.run([_host_compiler(), *flags, "-o", program, os.path.join(REFERENCE, "selftest.cpp"),
+                           os.path.join(REFERENCE, "reference.cpp")], capture_output=True, text=True)
+    if done.returncode != 0:
+        raise BuildError(f"compiling the references' self-test failed:\n{done.stderr}")
+    return program
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_reference())
