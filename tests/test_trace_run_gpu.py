@@ -113,6 +113,38 @@ def test_replay_schedules(name, dtype, tmp_path):
             assert torch.equal(got_whole[n], got_tail[n]) and torch.equal(got_whole[n], got_batched[n])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("head_dim", [64, 128])
+def test_replay_in_portions(head_dim, dtype, tmp_path):
+    """A request fed in portions of several tokens (the matrix-core attention at head sizes 64 and 128 continues
+    a sequence in the middle of its cache): a portion that ends at a block's end, so that the next starts on a
+    block's boundary; a portion of two tokens; one that ends at a block's end again; then token by token, while
+    a second request of the same steps starts later and runs beside it."""
+    raw = dict(TINY["qwen3" if head_dim == 128 else "llama"], hidden_size=128, num_attention_heads=2, num_key_value_heads=1,
+               head_dim=head_dim, max_position_embeddings=512)
+    # (weights of std 0.1: at this width std 0.2 makes scores so large that their rounding to bfloat16 alone moves
+    # logits by 5 % of the largest, in the kernels as in the stand-in that only rounds where they round)
+    folder = make_folder(raw, tmp_path / "model", seed=head_dim, std=0.1)
+    plain = P.PlainModel(folder)
+    vocab = plain.config.vocab_size
+    ids, other = token_ids(vocab, 230, seed=1), token_ids(vocab, 150, seed=2)
+    cuts = [0, 64, 66, 192, 225, 226, 227, 228, 229, 230]
+    steps = []
+    for index, (begin, end) in enumerate(zip(cuts, cuts[1:])):
+        entries = [{"id": "a", "tokens": ids[begin:end], "want": list(range(end - begin))}]
+        if index >= 2:                   # the second request: one portion a step, of other sizes
+            first, last = (index - 2) * 21, min(150, (index - 1) * 21)
+            entries.append({"id": "b", "tokens": other[first:last], "want": list(range(last - first))})
+        steps.append({"step": index, "entries": entries, "end": ["a", "b"] if end == 230 else []})
+    assert (len(cuts) - 3) * 21 >= 147
+    got = collect(steps, replay(folder, dtype, tmp_path / "portions", steps, 512))
+    assert_logits(got["a"], plain.logits(ids), dtype, f"head {head_dim}: a request in portions")
+    assert_logits(got["b"], plain.logits(other)[:got["b"].shape[0]], dtype, f"head {head_dim}: a request in portions beside it")
+    if dtype == "float32":
+        whole = trace_whole({"a": ids})
+        assert torch.equal(collect(whole, replay(folder, dtype, tmp_path / "whole", whole, 512))["a"], got["a"])
+
+
 def test_replay_without_wanted_logits_writes_no_file(tmp_path):
     folder = make_folder(TINY["llama"], tmp_path / "model", seed=1)
     steps = [{"step": 0, "entries": [{"id": "x", "tokens": [1, 2, 3], "want": []}], "end": []},
