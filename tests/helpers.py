@@ -106,3 +106,19 @@ def run_batched(engine, requests, prompts):
         for i, slot in enumerate(slots):
             if not done[i]:
                 engine.free_slot(slot)
+
+
+def assert_greedy_tokens(logits_of, prompt, tokens, dtype, penalty=1.0, what=""):
+    """`tokens` are what greedy generation from `prompt` gives, by the plain logits `logits_of(ids) -> [len, vocab]`:
+    in 32-bit every token is the plain loop's choice; in bfloat16 every token is, given the tokens before it, within
+    twice the logits' tolerance of the plain model's best (two near-equal logits may change places)."""
+    import plain_llama as P
+    history = list(prompt)
+    for index, token in enumerate(tokens):
+        row = P.apply_repetition_penalty(logits_of(history)[-1].float(), history, penalty)
+        if dtype == "float32":
+            assert token == P.greedy(row), f"{what}: token {index} is {token}, the plain loop chooses {P.greedy(row)}"
+        else:
+            assert float(row.max() - row[token]) <= 2 * TOLERANCE[dtype]["max"] * float(row.abs().max()), \
+                f"{what}: token {index} ({token}) is not among the plain model's best"
+        history.append(token)

@@ -356,6 +356,11 @@ def test_toy_architecture_with_parts_of_its_own(dtype, tmp_path):
     # slots are used again: the state of the next sequence starts from zero
     for got, logits in zip(run_batched(engine, requests[::-1], [1, 20, 60]), want[::-1]):
         assert_logits(got, logits, dtype, "toy batch in used slots")
-    out = generate(engine, [GenerateRequest(requests[1][:5], max_tokens=4, temperature=0.0, repetition_penalty=1.0)])
-    assert len(out[0].tokens) == 4
+    out = generate(engine, [GenerateRequest(requests[1][:5], max_tokens=4, temperature=0.0, repetition_penalty=1.0),
+                            GenerateRequest(requests[2][:3], max_tokens=6, temperature=0.0, repetition_penalty=1.3)])
+    assert [len(o.tokens) for o in out] == [4, 6]
+    from helpers import assert_greedy_tokens
+    logits_of = lambda ids: plain_toy(w, config, ids)
+    assert_greedy_tokens(logits_of, requests[1][:5], out[0].tokens, dtype, 1.0, "toy generation")
+    assert_greedy_tokens(logits_of, requests[2][:3], out[1].tokens, dtype, 1.3, "toy generation with a penalty")
     engine.cache.check()

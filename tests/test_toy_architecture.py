@@ -4,7 +4,7 @@ stepped and generated from on the CPU, with the test stand-in for the kernels: n
 or a change to the framework's files."""
 import torch
 
-from helpers import assert_logits, run_batched, run_tail_decoded, run_whole, token_ids
+from helpers import assert_greedy_tokens, assert_logits, run_batched, run_tail_decoded, run_whole, token_ids
 from ops_emulation import EmulatedOps
 from test_parts_gpu import define_toy, plain_toy
 
@@ -32,5 +32,8 @@ def test_toy_architecture_on_the_cpu_stand_in(tmp_path):
     out = generate(engine, [GenerateRequest(requests[1][:5], max_tokens=4, temperature=0.0, repetition_penalty=1.0),
                             GenerateRequest(requests[2][:3], max_tokens=6, temperature=0.0, repetition_penalty=1.3)])
     assert [len(o.tokens) for o in out] == [4, 6]
+    logits_of = lambda ids: plain_toy(w, config, ids)
+    assert_greedy_tokens(logits_of, requests[1][:5], out[0].tokens, "float32", 1.0, "toy generation")
+    assert_greedy_tokens(logits_of, requests[2][:3], out[1].tokens, "float32", 1.3, "toy generation with a penalty")
     engine.cache.check()
     assert engine.cache.slots.n_held == 0
