@@ -32,7 +32,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 __device__ __forceinline__ int key_of_row(int tile, int r) { return (r / 4) * 8 + tile * 4 + (r % 4); }
 
 template <int HD>
-__global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
+__global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) attention_decode_kernel(
     const bf16* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads,
     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
     __shared__ floatx4 merge_o[WAVES][DT][XRT_WAVE];
     __shared__ float merge_ml[WAVES][2][16];
 
-    const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
+    const int lane = threadIdx.x % XRT_WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / XRT_WAVE);   // in a scalar register, and with it the blocks' numbers
     const int r = lane % 16, c = lane / 16;
     const int part = blockIdx.x;                   // this workgroup's four chunks become one partial result
     const int chunk = part * WAVES + wave;
@@ -80,15 +80,13 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
         for (int ks = 0; ks < KS; ++ks)
             q[ks] = *reinterpret_cast<const bf16x8*>(qkv + (long)token * row_width + (long)head * HD + ks * 32 + c * 8);
 
-        for (int b = first_block; b <= last_block; ++b) {
-            int block = block_table[(long)slot * table_stride + b];
-            block = min(max(block, 0), n_blocks - 1);          // the host never hands out anything else
+        // Loads are always on their way: a block's values are asked for before its scores are computed, and the
+        // next block's keys right after, before the softmax and the value product of this one.
+        const int* table = block_table + (long)slot * table_stride;
+        auto block_of = [&](int b) { return min(max(table[min(b, last_block)], 0), n_blocks - 1); };   // the host never hands out anything else
+        bf16x8 kreg[2][2][KS], vreg[2][DT];
+        auto ask_keys = [&](int block) {
             const bf16* kb = k_cache + ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * HD;
-            const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * XRT_BLOCK_TOKENS;
-            const int valid = min(XRT_BLOCK_TOKENS, n_keys - b * XRT_BLOCK_TOKENS);   // keys of this block that exist
-
-            // all loads of the block go out together: the values do not wait for the scores
-            bf16x8 kreg[2][2][KS], vreg[2][DT];
 #pragma unroll
             for (int g = 0; g < 2; ++g)
 #pragma unroll
@@ -96,6 +94,12 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
                         kreg[g][t][ks] = *reinterpret_cast<const bf16x8*>(kb + (long)(g * 32 + key_of_row(t, r)) * HD + c * 8 + ks * 32);
+        };
+        int block = block_of(first_block), next_block = block_of(first_block + 1);
+        ask_keys(block);
+        for (int b = first_block; b <= last_block; ++b) {
+            const bf16* vb = v_cache + ((long)block * n_kv_heads + kv_head) * HD * XRT_BLOCK_TOKENS;
+            const int valid = min(XRT_BLOCK_TOKENS, n_keys - b * XRT_BLOCK_TOKENS);   // keys of this block that exist
 #pragma unroll
             for (int g = 0; g < 2; ++g)
 #pragma unroll
@@ -113,6 +117,9 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_decode_kernel(
                     for (int ks = 0; ks < KS; ++ks)
                         s[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[g][t][ks], q[ks], s[g][t], 0, 0, 0);
                 }
+            block = next_block;
+            next_block = block_of(b + 2);
+            if (b < last_block) ask_keys(block);
             // register i of s[g][t] is key g*32 + c*8 + t*4 + i, for query head r
             float block_max = -INFINITY;
 #pragma unroll
