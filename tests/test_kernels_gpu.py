@@ -91,7 +91,8 @@ def test_rmsnorm_reference_vector(ops):
 SHAPES = [(1, 64, 64), (3, 200, 96), (8, 1000, 176), (17, 96, 192), (64, 333, 520), (130, 257, 72),
           (300, 520, 1032), (1, 3, 5), (5, 7, 13), (33, 4100, 264), (64, 40, 4096), (65, 40, 4096),
           (2048, 6144, 128), (2000, 6200, 136), (70, 300, 64), (300, 520, 1024), (2100, 6100, 320),
-          (2100, 8300, 128), (40, 4100, 1024), (64, 333, 640), (33, 130, 128), (17, 700, 192)]
+          (2100, 8300, 128), (40, 4100, 1024), (64, 333, 640), (33, 130, 128), (17, 700, 192),
+          (600, 520, 8192), (520, 1030, 8320)]         # the last two: many rows, few columns, a very long k (large tiles that split k)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16 packed"])

@@ -586,26 +586,37 @@ int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
 // few to fill the chip: such products are still bound by reading w.
 constexpr int SPLIT_BM = 64, SPLIT_BN = 128;
 
-struct SplitPlan { int splits, k_per_split; long rows_w; };
+struct SplitPlan { int splits, k_per_split; long rows_w; int tile; };      // tile: rows of x per tile (64, 128 or 256)
 
 SplitPlan split_plan(int M, int N, int K, int mode) {
     const long rows_w = mode == MODE_GATED ? 2L * N : N;
     const long tiles_n = (rows_w + SPLIT_BN - 1) / SPLIT_BN;
     const int units = K / 64;                                  // k is dealt out in pieces of 64
-    int splits, least;                                         // least: pieces of k that a part should have
+    int splits, least, tile = SPLIT_BM;                        // least: pieces of k that a part should have
+    const long large_tiles = (long)((M + 255) / 256) * ((rows_w + 255) / 256);
     if (M <= SPLIT_BM) {
         splits = (int)(256 / tiles_n);                         // one workgroup per compute unit, or fewer
         least = 1;
+    } else if (large_tiles <= 128 && M >= 512 && mode != MODE_GATED && units >= 128) {
+        // Many rows and a very long k, but so few columns that the largest tiles would leave half of the compute
+        // units idle (the projection back from the feed-forward's width): the large tiles split k between them.
+        // The tiles of 128 x 128, which fill the chip without a second kernel, read their operands from LDS
+        // more often for the same products and take longer here.
+        splits = (int)(256 / large_tiles);
+        splits = splits > 4 ? 4 : splits;
+        least = 32;
+        tile = 256;
     } else {
         const long tiles = (long)((M + 127) / 128) * tiles_n;  // two of these workgroups share a compute unit
         splits = tiles >= 384 ? 1 : (int)((512 + tiles - 1) / tiles);
         least = 4;
+        tile = 128;
     }
     splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
     splits = splits > units / least ? (units / least < 1 ? 1 : units / least) : splits;
     const int per = (units + splits - 1) / splits;
     splits = (units + per - 1) / per;                          // no empty part
-    return SplitPlan{splits, per * 64, rows_w};
+    return SplitPlan{splits, per * 64, rows_w, tile};
 }
 
 // NORM 1: the rows of a came without their RMSNorm's division (norm.squares_in): the sums are multiplied by
@@ -668,6 +679,32 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restri
             const float gain = norm.gain_dtype == XRT_F32 ? ((const float*)norm.gain)[n] : to_float(((const bf16*)norm.gain)[n]);
             ((bf16*)norm.scaled_out)[index] = from_float<bf16>(fresh * gain);
         }
+    }
+}
+
+// The same for store and accumulate without a norm, four neighbouring columns a thread (N a multiple of 4):
+// what products of many rows use, whose partial sums are tens of megabytes.
+template <int MODE, typename TO>
+__global__ void __launch_bounds__(256) split_reduce_wide_kernel(const float* __restrict__ parts, int splits, long count, TO* __restrict__ out) {
+    const long index = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (index >= count) return;
+    float4 sum = *reinterpret_cast<const float4*>(parts + index);
+    for (int p = 1; p < splits; ++p) {
+        const float4 part = *reinterpret_cast<const float4*>(parts + p * count + index);
+        sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+    }
+    if constexpr (MODE == MODE_ACCUMULATE) {
+        static_assert(sizeof(TO) == 4, "accumulation needs a float32 output");
+        const float4 before = *reinterpret_cast<const float4*>(out + index);
+        // the order of the one-column kernel: the parts first, in order, then onto what was there
+        sum.x = before.x + sum.x; sum.y = before.y + sum.y; sum.z = before.z + sum.z; sum.w = before.w + sum.w;
+    }
+    if constexpr (sizeof(TO) == 4) {
+        *reinterpret_cast<float4*>(out + index) = sum;
+    } else {
+        struct alignas(8) Four { TO e[4]; } four;
+        four.e[0] = from_float<TO>(sum.x); four.e[1] = from_float<TO>(sum.y); four.e[2] = from_float<TO>(sum.z); four.e[3] = from_float<TO>(sum.w);
+        *reinterpret_cast<Four*>(out + index) = four;
     }
 }
 
@@ -765,6 +802,9 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
     const int status = M <= SPLIT_BM
         ? launch_kernel<SPLIT_BM, SPLIT_BN, 1, 4, MODE_STORE, 64, 3, float>(
               a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split)
+        : plan.tile == 256
+        ? launch_kernel<256, 256, 2, 4, MODE_STORE, 64, 2, float>(
+              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split)
         : launch_kernel<128, 128, 2, 2, MODE_STORE, 64, 2, float>(
               a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split);
     if (status != 0) return status;
@@ -779,6 +819,15 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
             else split_reduce_qkv_kernel<0><<<pair_blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around, *after);
             XRT_LAUNCH_CHECK("linear (split reduce, q/k/v)");
         }
+        return 0;
+    }
+    if (!scaled && !emits && mode != MODE_GATED && N % 4 == 0 && M > SPLIT_BM && (uintptr_t)out % 16 == 0) {
+        const long count = (long)M * N;
+        const unsigned wide_blocks = (unsigned)((count / 4 + 255) / 256);
+        if (mode == MODE_STORE) split_reduce_wide_kernel<MODE_STORE, TO><<<wide_blocks, 256, 0, s>>>(workspace, plan.splits, count, out);
+        else if constexpr (sizeof(TO) == 4) split_reduce_wide_kernel<MODE_ACCUMULATE, TO><<<wide_blocks, 256, 0, s>>>(workspace, plan.splits, count, out);
+        else XRT_REQUIRE(false, "linear (mfma): accumulation needs a float32 output");
+        XRT_LAUNCH_CHECK("linear (split reduce, four columns a thread)");
         return 0;
     }
 #define XRT_REDUCE(MODE_, NORM_) split_reduce_kernel<MODE_, TO, NORM_><<<blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around, activation)
