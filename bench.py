@@ -45,6 +45,7 @@ OTHER_BATCHES = {"llama3-8b": (1, 64), "qwen3-8b": (1, 64), "qwen3-32b": (1,)}
 CONTEXT = 4096
 SHORT_CONTEXT = 128
 PREFILL_TOKENS = 2048
+LONG_PREFILL = 8192                # a second prefill point, where attention weighs more
 UNEQUAL_PROMPTS = (8, 64, 2048)     # the Qwen3-8B shape's batch of prompts: count, shortest, longest
 
 
@@ -235,7 +236,7 @@ def main() -> int:
     others = () if args.skip_points else tuple(b for b in OTHER_BATCHES[args.shape] if b != batch)
     largest_batch = max((batch,) + others)
     engine = Engine.random(config, seed=args.seed, dtype=args.dtype, max_tokens=largest_batch * CONTEXT,
-                           max_slots=largest_batch, max_context=CONTEXT)
+                           max_slots=largest_batch, max_context=CONTEXT if args.skip_points else max(CONTEXT, LONG_PREFILL))
     bench = Bench(engine, args.seed)
 
     def priced(ms, mean_length, sequences):
@@ -275,6 +276,11 @@ def main() -> int:
         points[f"decode_b{batch}_ctx{SHORT_CONTEXT}"] = round(value, 1)
         points[f"decode_b{batch}_ctx{SHORT_CONTEXT}_ms"] = round(ms, 4)
         points[f"decode_b{batch}_ctx{SHORT_CONTEXT}_frac"] = round(priced(ms, length, batch) / PEAK_HBM_GBS, 4)
+        if largest_batch * CONTEXT >= LONG_PREFILL:
+            seconds = bench.prefill([LONG_PREFILL], repeats=2)
+            points[f"prefill_{LONG_PREFILL}"] = round(LONG_PREFILL / seconds, 1)
+            points[f"prefill_{LONG_PREFILL}_ms"] = round(seconds * 1e3, 3)
+            points[f"prefill_{LONG_PREFILL}_frac"] = round(prefill_flops(config, [LONG_PREFILL]) / seconds / PEAK_FLOPS[short], 4)
         if args.shape == "qwen3-8b":
             count, low, high = UNEQUAL_PROMPTS
             lengths = torch.randint(low, high + 1, (count,), generator=torch.Generator().manual_seed(args.seed)).tolist()
