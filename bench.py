@@ -76,7 +76,8 @@ def sync():
 
 
 def measured_ceilings(ops, device):
-    """(GB/s of a kernel that only reads 2 GiB, TFLOP/s of bfloat16 matrix-core products on resident tiles)."""
+    """(GB/s of a kernel that only reads 2 GiB, TFLOP/s of bfloat16 matrix-core products on resident tiles of small
+    whole numbers, the same on tiles of random numbers: the chip holds a lower clock on those)."""
     buffer = torch.ones(1 << 29, dtype=torch.int32, device=device)          # 2 GiB: beyond every cache
     best_read = 0.0
     for nontemporal in (False, True):
@@ -88,13 +89,16 @@ def measured_ceilings(ops, device):
         sync()
         best_read = max(best_read, count / (begin.elapsed_time(end) * 1e-3) / 1e9)
     del buffer
-    ops.probe_mfma(1000, device)
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    begin.record()
-    flops = ops.probe_mfma(200000, device)
-    end.record()
-    sync()
-    return best_read, flops / (begin.elapsed_time(end) * 1e-3) / 1e12
+    rates = []
+    for random_operands in (False, True):
+        ops.probe_mfma(1000, device, random_operands)
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        flops = ops.probe_mfma(200000, device, random_operands)
+        end.record()
+        sync()
+        rates.append(flops / (begin.elapsed_time(end) * 1e-3) / 1e12)
+    return best_read, rates[0], rates[1]
 
 
 class Bench:
@@ -254,7 +258,7 @@ def main() -> int:
                           "tokens_per_s": round(tokens_per_s, 1)}), flush=True)
         return 0
     achieved = priced(ms_per_step, mean_length, batch)
-    read_gbs, mfma_tflops = measured_ceilings(engine.ops, engine.device)
+    read_gbs, mfma_tflops, mfma_random_tflops = measured_ceilings(engine.ops, engine.device)
 
     seconds = bench.prefill([PREFILL_TOKENS])
     flops = prefill_flops(config, [PREFILL_TOKENS])
@@ -263,6 +267,7 @@ def main() -> int:
     if short == "bf16":
         prefill["measured_peak_tflops"] = round(mfma_tflops, 1)
         prefill["frac_of_measured"] = round(flops / seconds / (mfma_tflops * 1e12), 4)
+        prefill["measured_peak_random_operands_tflops"] = round(mfma_random_tflops, 1)
 
     points = {}
     if not args.skip_points:

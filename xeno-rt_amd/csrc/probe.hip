@@ -28,10 +28,21 @@ __global__ void __launch_bounds__(256) probe_read_kernel(const uint4v* __restric
 }
 
 // Four independent chains of 32x32x16 products per wavefront, operands and sums in registers.
-__global__ void __launch_bounds__(256) probe_mfma_kernel(long iterations, float* sink) {
+// The operands are small whole numbers, or (random_operands) numbers of either sign in [1, 2) with random mantissas:
+// the matrix cores draw more power on those, and the clock that the chip then holds is lower.
+__global__ void __launch_bounds__(256) probe_mfma_kernel(long iterations, int random_operands, float* sink) {
     bf16x8 a, b;
+    unsigned state = (threadIdx.x * 2654435761u) ^ (blockIdx.x * 40503u);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) { a[e] = (bf16)(float)((threadIdx.x + e) % 3); b[e] = (bf16)(float)((threadIdx.x + 2 * e) % 5); }
+    for (int e = 0; e < 8; ++e) {
+        a[e] = (bf16)(float)((threadIdx.x + e) % 3);
+        b[e] = (bf16)(float)((threadIdx.x + 2 * e) % 5);
+        if (random_operands) {
+            state = state * 1664525u + 1013904223u;
+            a[e] = __builtin_bit_cast(bf16, (unsigned short)(((state >> 16) & 0x807fu) | 0x3f80u));
+            b[e] = __builtin_bit_cast(bf16, (unsigned short)((state & 0x807fu) | 0x3f80u));
+        }
+    }
     floatx16 acc[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c)
@@ -44,7 +55,7 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(long iterations, float*
     float total = 0.f;
 #pragma unroll
     for (int c = 0; c < 4; ++c) total += acc[c][0] + acc[c][15];
-    if (total == -1.f) sink[0] = total;             // sums of non-negative products: never true
+    if (total == -1.5f && iterations < 0) sink[0] = total;             // never true
 }
 
 }  // namespace
@@ -66,9 +77,9 @@ extern "C" long xrt_probe_read_bytes(long bytes) {
     return per_group * 16 * 2048;
 }
 
-extern "C" int xrt_probe_mfma(long iterations, void* sink, void* stream) {
+extern "C" int xrt_probe_mfma(long iterations, int random_operands, void* sink, void* stream) {
     XRT_REQUIRE(sink && iterations > 0, "probe_mfma: bad operands");
-    probe_mfma_kernel<<<XRT_PROBE_MFMA_GROUPS, 256, 0, (hipStream_t)stream>>>(iterations, (float*)sink);
+    probe_mfma_kernel<<<XRT_PROBE_MFMA_GROUPS, 256, 0, (hipStream_t)stream>>>(iterations, random_operands, (float*)sink);
     XRT_LAUNCH_CHECK("probe_mfma");
     return 0;
 }

@@ -42,11 +42,13 @@ int xrt_random_normal(void* out, int dtype, long count, unsigned long long key, 
 // xrt_probe_read reads xrt_probe_read_bytes(bytes) bytes of `buffer` once (plain or non-temporal loads) and
 // writes nothing (sink: 4 bytes that stay as they are). xrt_probe_mfma runs `iterations` rounds of four
 // 32x32x16 bfloat16 matrix-core products per wavefront on tiles held in registers, in XRT_PROBE_MFMA_GROUPS
-// workgroups of four wavefronts: XRT_PROBE_MFMA_GROUPS * 4 * iterations * 4 * 2 * 32 * 32 * 16 flops.
+// workgroups of four wavefronts: XRT_PROBE_MFMA_GROUPS * 4 * iterations * 4 * 2 * 32 * 32 * 16 flops. Its operands
+// are small whole numbers, or with random_operands numbers of either sign with random mantissas, on which
+// the chip holds a lower clock.
 #define XRT_PROBE_MFMA_GROUPS 512
 int xrt_probe_read(const void* buffer, long bytes, int nontemporal, void* sink, void* stream);
 long xrt_probe_read_bytes(long bytes);
-int xrt_probe_mfma(long iterations, void* sink, void* stream);
+int xrt_probe_mfma(long iterations, int random_operands, void* sink, void* stream);
 
 // residual[i] += delta[i]
 int xrt_add(float* residual, const void* delta, int delta_dtype, long count, void* stream);

@@ -213,10 +213,10 @@ class HipOps:
                                             self._stream(buffer)))
         return int(self.lib.xrt_probe_read_bytes(ctypes.c_long(size)))
 
-    def probe_mfma(self, iterations: int, device) -> int:
+    def probe_mfma(self, iterations: int, device, random_operands: bool = False) -> int:
         """Matrix-core products on tiles held in registers; returns the flops done."""
         sink = torch.zeros(1, dtype=torch.float32, device=device)
-        self._check(self.lib.xrt_probe_mfma(ctypes.c_long(iterations), _ptr(sink), self._stream(sink)))
+        self._check(self.lib.xrt_probe_mfma(ctypes.c_long(iterations), int(random_operands), _ptr(sink), self._stream(sink)))
         return 512 * 4 * iterations * 4 * 2 * 32 * 32 * 16
 
     def add(self, residual, delta):
