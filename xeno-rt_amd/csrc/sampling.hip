@@ -447,7 +447,8 @@ constexpr int LEAST_SLICES = 8;        // with fewer slices their tops are too f
 
 struct SliceCandidates {
     int count;                         // -1: this row does not go this way; more than SLICE_HOLDS: they did not fit;
-                                       // -2: a row that takes the largest logit: `largest` is the slice's, `unused` its first index (0x7fffffff: none)
+                                       // -2: a row that takes the largest logit: `largest` is the slice's, `unused` its first index (0x7fffffff: none);
+                                       // -3: a row that draws from all tokens (no top-k, no top-p): `largest` and `mass` only
     float largest, mass;               // for a row without top-k: the slice's largest value, and the sum of exp((value - largest) / temperature)
     int unused;
     unsigned top[SLICE_TOPS];          // keys of SLICE_TOPS different tokens of the slice, the largest first (0: none)
@@ -498,7 +499,10 @@ __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
     SliceCandidates& mine = candidates[(long)r * slices + slice];
     const bool greedy = temperature[r] <= 1e-5f;                // the largest logit, first index: the slices' largest, then the first of those
     const int k = top_k_by_slices(temperature[r], top_k[r], top_p[r], vocab);
-    if (k == 0 && !greedy) {
+    // a temperature alone: the draw runs over all tokens; a slice hands on its mass and largest value, the row's
+    // workgroup finds the slice in which the drawn number falls and walks that slice alone
+    const bool whole = !greedy && top_k[r] == 0 && !(top_p[r] < 1.0f);
+    if (k == 0 && !greedy && !whole) {
         if (tid == 0) mine.count = -1;
         return;
     }
@@ -576,7 +580,7 @@ __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
         const float inv_temp = 1.0f / temperature[r], top = slice_largest;
         float sum = 0.f;
 #pragma unroll
-        for (int e = 0; e < SLICE_EACH; ++e) sum += key[e] != 0u ? expf((value[e] - top) * inv_temp) : 0.f;
+        for (int e = 0; e < SLICE_EACH; ++e) sum += key[e] != 0u && top > -INFINITY ? expf((value[e] - top) * inv_temp) : 0.f;   // (a slice of -inf alone has no mass)
         sum = wave_sum(sum);
         if (tid % XRT_WAVE == 0) wave_mass[tid / XRT_WAVE] = sum;
         __syncthreads();
@@ -585,8 +589,10 @@ __global__ void __launch_bounds__(SLICE_THREADS) sample_slices_kernel(
             for (int w = 0; w < SLICE_WAVES; ++w) total += wave_mass[w];
             mine.mass = total;
             mine.largest = top;
+            if (whole) mine.count = -3;
         }
     }
+    if (whole) return;
 #pragma unroll
     for (int e = 0; e < SLICE_EACH; ++e) {
         if (key[e] != 0u && key[e] >= threshold) {
@@ -632,6 +638,83 @@ __global__ void __launch_bounds__(THREADS) sample_candidates_kernel(
                 if (other > best || (other == best && other_index < best_index)) { best = other; best_index = other_index; }
             }
             if (tid == 0) out.put(r, best_index == 0x7fffffff ? 0 : best_index);   // nothing compared greater (all NaN or -inf): index 0
+        }
+        return;
+    }
+    if (mine[0].count == -3) {
+        // A temperature alone: the inverse CDF over all tokens, in the order of ids (sampler.rs:147-164, :185-195). The
+        // slices' masses say in which slice the drawn number falls; that slice's weights are worked out again, relative
+        // to the row's largest value, and one wavefront walks them.
+        __shared__ float whole_weight[SLICE];
+        __shared__ unsigned whole_seen[SLICE / 32];
+        __shared__ int whole_slice;
+        __shared__ float whole_target, whole_best;
+        const float inv_temp = 1.0f / temperature[r];
+        if (tid < XRT_WAVE) {
+            float best = tid < slices ? mine[tid].largest : -INFINITY;
+#pragma unroll
+            for (int offset = XRT_WAVE / 2; offset > 0; offset >>= 1) best = fmaxf(best, __shfl_xor(best, offset, XRT_WAVE));
+            const float share = tid < slices ? mine[tid].mass * expf((mine[tid].largest - best) * inv_temp) : 0.f;
+            float total = 0.f;
+            for (int j = 0; j < slices; ++j) total += __shfl(share, j, XRT_WAVE);
+            const float target = uniforms[r] * total;
+            float before = 0.f;
+            int pick = -1, last = -1;
+            for (int j = 0; j < slices && pick < 0; ++j) {      // every lane walks the same list
+                const float x = __shfl(share, j, XRT_WAVE);
+                if (x > 0.f) {
+                    last = j;
+                    if (target < before + x) pick = j; else before += x;
+                }
+            }
+            if (pick < 0 && last >= 0) { pick = last; before -= __shfl(share, last, XRT_WAVE); }     // rounding at the very end: the last slice with mass
+            if (tid == 0) { whole_slice = pick; whole_target = target - before; whole_best = best; }
+        }
+        if (tid < SLICE / 32) whole_seen[tid] = 0u;
+        __syncthreads();
+        const int slice = whole_slice;
+        if (slice < 0) {                                        // no token has a weight (all -inf or NaN): the reference's fallback
+            if (tid == 0) out.put(r, 0);
+            return;
+        }
+        const int first = slice * SLICE;
+        const float factor = penalty[r], best = whole_best;
+        const int h_begin = history_spans[2 * r], h_end = history_spans[2 * r + 1];
+        if (factor > 1.0f && h_end > h_begin) {
+            for (int i = h_begin + tid; i < h_end; i += THREADS) {
+                const int token = history[i] - first;
+                if (token >= 0 && token < SLICE && token + first < vocab) atomicOr(&whole_seen[token >> 5], 1u << (token & 31));
+            }
+            __syncthreads();
+        }
+        const float* row = logits + (long)r * vocab;
+        for (int local = tid; local < SLICE; local += THREADS) {
+            const float v = row[min(first + local, vocab - 1)];
+            const float changed = v > 0.f ? v / factor : v * factor;
+            const float adjusted = (whole_seen[local >> 5] >> (local & 31)) & 1u ? changed : v;
+            whole_weight[local] = first + local < vocab ? expf((adjusted - best) * inv_temp) : 0.f;
+        }
+        __syncthreads();
+        if (tid < XRT_WAVE) {
+            const float target = whole_target;
+            float running = 0.f;
+            int pick = -1, last_kept = -1;
+            for (int base = 0; base < SLICE && pick < 0; base += XRT_WAVE) {
+                const float w = whole_weight[base + tid];
+                float through = w;                              // inclusive sum over the lanes, in lane order
+#pragma unroll
+                for (int offset = 1; offset < XRT_WAVE; offset <<= 1) {
+                    const float below = __shfl_up(through, offset, XRT_WAVE);
+                    if (tid >= offset) through += below;
+                }
+                const unsigned long long hits = __ballot(w > 0.f && running + through > target);
+                const unsigned long long kepts = __ballot(w > 0.f);
+                if (hits != 0ull) pick = base + __builtin_ctzll(hits);
+                if (kepts != 0ull) last_kept = base + 63 - __builtin_clzll(kepts);
+                running += __shfl(through, XRT_WAVE - 1, XRT_WAVE);
+            }
+            if (pick < 0) pick = last_kept;                     // rounding at the slice's end: its last token with a weight
+            if (tid == 0) out.put(r, pick >= 0 ? first + pick : 0);
         }
         return;
     }

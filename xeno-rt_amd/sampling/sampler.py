@@ -135,7 +135,7 @@ class Sampler:
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
         # rows that the kernels can sample from a few candidates instead of passes over the whole row, and rows
         # that take the largest logit (many workgroups look for it slice by slice, instead of one over the row)
-        small_top_k = any(c.is_greedy() or 0 < c.top_k <= 64 or (c.top_k == 0 and c.top_p < 1.0) for c in configs)
+        small_top_k = any(c.is_greedy() or c.top_k <= 64 for c in configs)       # (no top-k is top_k 0: a top-p alone, or a draw from all tokens)
         if log is not None:
             self.ops.sample(logits, out, floats[0], ints[:rows], floats[1], floats[2], log[0].tokens,
                             ints[rows:3 * rows], floats[3], small_top_k=small_top_k, append_at=ints[3 * rows:])
