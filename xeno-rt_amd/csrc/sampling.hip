@@ -19,7 +19,8 @@
 // into slices of 4096 tokens, a workgroup per slice holds its slice in registers and finds the
 // slice's own k largest (ties included), and the row's workgroup then works on those few
 // candidates only: the row's k largest are among them. Slices whose ties overflow their list send the
-// row back to the path above.
+// row back to the path above. A temperature alone (no top-k, no top-p) goes through the slices too: each
+// hands on its mass, the row's workgroup finds the slice in which the drawn number falls and walks it.
 #include "common.h"
 #include "xrt_hip.h"
 
