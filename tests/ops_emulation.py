@@ -114,7 +114,7 @@ class EmulatedOps:
                 kv.k[block, :, pos % BLOCK, :] = qkv[t, qw:qw + kw].reshape(n_kv_heads, head_dim).to(kv.k.dtype)
                 kv.v[block, :, :, pos % BLOCK] = v[t].to(kv.v.dtype)
 
-    def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None):
+    def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None):
         tokens = qkv.shape[0]
         group = n_heads // n_kv_heads
         q = qkv[:, :n_heads * head_dim].to(torch.float32).reshape(tokens, n_heads, head_dim)
@@ -135,6 +135,8 @@ class EmulatedOps:
             for head in range(n_heads):
                 kvh = head // group
                 scores = (keys[:, kvh, :] @ q[t, head]) * scale
+                if distance_slopes is not None:
+                    scores = scores + float(distance_slopes[head]) * (index - pos).to(torch.float32)
                 probs = torch.softmax(scores, dim=0)
                 out[t, head * head_dim:(head + 1) * head_dim] = (probs @ values[:, kvh, :]).to(out.dtype)
 

@@ -71,12 +71,13 @@ class CppReference:
                                      ctypes.c_float(rope_scale), _p(k), _p(v), _p(table), stride, blocks)
         return out
 
-    def attention(self, qkv, n_heads, n_kv_heads, head_dim, k, v, block_table, positions, slots, scale, window=0):
+    def attention(self, qkv, n_heads, n_kv_heads, head_dim, k, v, block_table, positions, slots, scale, window=0, distance_slopes=None):
         qkv, k, v = _f32(qkv), _f32(k), _f32(v)
         table, positions, slots = _i32(block_table), _i32(positions), _i32(slots)
         out = torch.empty(qkv.shape[0], n_heads * head_dim)
         self.lib.xrt_ref_attention(_p(qkv), qkv.shape[0], n_heads, n_kv_heads, head_dim, _p(k), _p(v), _p(table),
-                                   table.shape[1], _p(positions), _p(slots), _p(out), ctypes.c_float(scale), int(window or 0))
+                                   table.shape[1], _p(positions), _p(slots), _p(out), ctypes.c_float(scale), int(window or 0),
+                                   _p(_f32(distance_slopes)) if distance_slopes is not None else None)
         return out
 
     def sample(self, logits, temperature, top_k, top_p, penalty, history, history_spans, uniforms):

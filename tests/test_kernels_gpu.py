@@ -495,6 +495,46 @@ def test_attention_finds_a_far_key(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd", [(6, 3, 32), (8, 2, 128)])
+def test_attention_with_scores_biased_by_distance(ops, cpp, dtype, nh, nkv, hd):
+    """distance_slopes: a key at position j adds slope * (j - P) to the scaled score of the query at P, one slope per
+    query head (also where the matrix-core kernels would run without it: a described decode step and a prefill).
+    Against float64 on the host and against the plain C++ reference."""
+    lengths = [200, 65]
+    kv, keys, values = filled_cache(nkv, hd, DT[dtype], lengths, seed=hd + 1)
+    slopes = torch.tensor([0.5 ** (h + 1) for h in range(nh)], dtype=torch.float32, device=DEV)
+    scale = 1.0 / math.sqrt(hd)
+    for batch, slots, positions in (
+            (SimpleNamespace(slots=i32([0, 0, 1, -1]), positions=i32([199, 64, 64, 0])), [0, 0, 1, -1], [199, 64, 64, 0]),
+            (described([0, 1], [1, 1], [199, 64]), [0, 1], [199, 64]),
+            (described([0], [40], [160]), [0] * 40, list(range(160, 200)))):
+        qkv = rand(len(slots), (nh + 2 * nkv) * hd, dtype=DT[dtype], seed=9)
+        out = torch.full((len(slots), nh * hd), 7.0, dtype=DT[dtype], device=DEV)
+        ops.attention(qkv, nh, nkv, hd, kv, batch, out, scale=scale, distance_slopes=slopes)
+        plain = torch.empty_like(out)
+        ops.attention(qkv, nh, nkv, hd, kv, batch, plain, scale=scale)
+        from_cpp = cpp.attention(qkv.cpu(), nh, nkv, hd, kv.k.cpu(), kv.v.cpu(), kv.block_table.cpu(), torch.tensor(positions), torch.tensor(slots), scale,
+                                 distance_slopes=slopes.cpu())
+        for t, (slot, pos) in enumerate(zip(slots, positions)):
+            if slot < 0:
+                assert float(out[t].abs().max()) == 0.0
+                continue
+            k = keys[slot][:pos + 1].double().cpu()                 # [keys, kv heads, dim]
+            v = values[slot][:pos + 1].double().cpu()
+            distance = torch.arange(pos + 1, dtype=torch.float64) - pos
+            want = torch.empty(nh * hd, dtype=torch.float64)
+            for head in range(nh):
+                q = qkv[t, head * hd:(head + 1) * hd].double().cpu()
+                scores = (k[:, head // (nh // nkv)] @ q) * scale + float(slopes[head]) * distance
+                want[head * hd:(head + 1) * hd] = torch.softmax(scores, 0) @ v[:, head // (nh // nkv)]
+            limit = 2e-5 if dtype == "float32" else 1e-2
+            assert rel(out[t].cpu(), want) < limit, (t, slot, pos)
+            assert rel(from_cpp[t], want) < 2e-5, (t, slot, pos)
+            if pos > 8:
+                assert rel(plain[t].cpu(), want) > 10 * limit        # the slopes do change the result
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_attention_window_edge(ops, dtype):
     """With a window of W a query at P sees keys P-W+1..P: a loud key just outside must be
     ignored, the same key just inside must win."""

@@ -132,6 +132,62 @@ def test_attention_part_prompt_then_decode(dtype, nh, nkv, hd, qk_norm):
     assert part.scale == 1.0 / math.sqrt(hd)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_part_with_a_position_encoding_on_the_scores(dtype):
+    """A position encoding defined here, which leaves q and k alone and lowers the scores of far keys instead
+    (one slope per head): the attention part hands its slopes to the kernel. A prompt, then single tokens."""
+    from xeno_rt_amd.cache import SequenceCache
+    from xeno_rt_amd.parts import Attention
+    from xeno_rt_amd.parts.base import PositionEncoding
+
+    class DistanceBias(PositionEncoding):
+        capturable = True
+
+        def __init__(self, n_heads):
+            self.values = [2.0 ** -(h + 2) for h in range(n_heads)]
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.slopes = torch.tensor(self.values, dtype=torch.float32, device=runtime.device)
+
+        def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch):
+            return None
+
+        def score_slopes(self):
+            return self.slopes
+
+    hidden, nh, nkv, hd, length, prompt = 80, 4, 2, 128, 100, 70
+    part = Attention("a.", hidden, nh, nkv, hd, position=DistanceBias(nh))
+    w = weights_for(part, 5, std=0.15)
+    part.bind(w, runtime(dtype))
+    cache = SequenceCache([part.cache_needs()], [0], 256, 1, 128, DT[dtype], DEV)
+    h = torch.randn(length, hidden, generator=torch.Generator().manual_seed(4)).to(DT[dtype])
+    x = h.double()
+    q, k, v = (P.linear(x, w[f"a.{n}_proj.weight"].double()) for n in "qkv")
+    distance = torch.arange(length, dtype=torch.float64)[None, :] - torch.arange(length, dtype=torch.float64)[:, None]
+    mixed = torch.empty(length, nh * hd, dtype=torch.float64)
+    for head in range(nh):
+        kv_head = head // (nh // nkv)
+        scores = q[:, head * hd:(head + 1) * hd] @ k[:, kv_head * hd:(kv_head + 1) * hd].T / math.sqrt(hd)
+        scores = scores + part.position.values[head] * distance
+        scores = scores.masked_fill(distance > 0, -float("inf"))
+        mixed[:, head * hd:(head + 1) * hd] = torch.softmax(scores, dim=1) @ v[:, kv_head * hd:(kv_head + 1) * hd]
+    want = P.linear(mixed, w["a.o_proj.weight"].double())
+    unbiased = P.linear(P.causal_attention(q, k, v, nh, nkv, hd), w["a.o_proj.weight"].double())
+    slot = cache.alloc_slot()
+    got = []
+    at = 0
+    for count in [prompt] + [1] * (length - prompt):
+        batch, _ = batch_for(cache, [slot], [count])
+        residual = torch.zeros(count, hidden, device=DEV)
+        part.forward(h[at:at + count].to(DEV), batch, cache.layer_cache(0), residual)
+        got.append(residual.clone())
+        at += count
+        cache.commit(slot, at)
+    assert rel(torch.cat(got), want) < TOL[dtype]
+    assert rel(unbiased, want) > 10 * TOL[dtype]                # the slopes do change the result
+
+
 def test_parts_are_found_by_kind_and_name():
     from xeno_rt_amd.parts import create_part, registered_parts, RMSNorm, Rotary
     assert "attention" in registered_parts("mixer") and "gated_mlp" in registered_parts("feed_forward")

@@ -1,14 +1,14 @@
 // Entry point of attention: checks the operands and picks the kernel.
 //   bfloat16, head size 64 or 128, no window: the matrix-core kernels: decode (every sequence
 //   brings one token) or prefill (any token counts);
-//   everything else (float32, other head sizes, windows): the general kernel.
+//   everything else (float32, other head sizes, windows, scores biased by distance): the general kernel.
 #include "common.h"
 #include "xrt_hip.h"
 
 int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
-                          int window, hipStream_t s);
+                          int window, const float* distance_slopes, hipStream_t s);
 bool xrt_attention_decode_accepts(int head_dim);
 long xrt_attention_decode_workspace(int tokens, int n_heads, int n_kv_heads, int head_dim, int max_context);
 int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
@@ -35,7 +35,7 @@ extern "C" long xrt_attention_workspace(int dtype, int tokens, int n_heads, int 
 extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                              const void* k_cache, const void* v_cache, const int* block_table,
                              int table_stride, int n_blocks, const int* positions, const int* slots, void* out,
-                             float scale, int window, const int* seq_offsets, const int* seq_slots,
+                             float scale, int window, const float* distance_slopes, const int* seq_offsets, const int* seq_slots,
                              const int* seq_starts, int n_seqs, int max_count, int max_context,
                              float* workspace, long workspace_floats, void* stream) {
     XRT_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
@@ -48,7 +48,7 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
     if (tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const bool described = seq_offsets && seq_slots && seq_starts && n_seqs > 0 && max_count > 0 && max_context > 0;
-    if (dtype == XRT_BF16 && window == 0 && described) {
+    if (dtype == XRT_BF16 && window == 0 && distance_slopes == nullptr && described) {
         const long need = xrt_attention_workspace(dtype, tokens, n_heads, n_kv_heads, head_dim, window, max_count, max_context);
         if (takes_decode_kernel(dtype, n_heads, n_kv_heads, head_dim, window, max_count, max_context) &&
             (need == 0 || (workspace != nullptr && workspace_floats >= need)))
@@ -65,5 +65,5 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
         }
     }
     return xrt_attention_generic(qkv, dtype, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
-                                 table_stride, n_blocks, positions, slots, out, scale, window, s);
+                                 table_stride, n_blocks, positions, slots, out, scale, window, distance_slopes, s);
 }

@@ -9,6 +9,10 @@
 // One wavefront per (token, head). Keys are visited block by block (64 keys, lane j takes
 // key j) in the order of their positions, whatever the step looks like, so the result of a
 // token does not depend on how its request was cut into steps or batched.
+//
+// A position encoding that acts on the scores instead of on q and k is served here too: with
+// distance_slopes (one float per query head) a key at position j adds slope * (j - P) to the
+// score of the query at position P, after the scale. Not in the reference's model.
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -22,7 +26,7 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
     const T* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads, int head_dim,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
-    T* __restrict__ out, float scale, int window) {
+    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes) {
     __shared__ float qs[MAX_HEAD_DIM];
     __shared__ float ps[XRT_WAVE];
     const int lane = threadIdx.x;
@@ -36,6 +40,7 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
     }
     const int pos = positions[token];
     const int first = window > 0 ? max(0, pos - window + 1) : 0;
+    const float slope = distance_slopes ? distance_slopes[head] : 0.f;
     const T* q = qkv + (long)token * row_width + (long)head * head_dim;
     for (int e = lane; e < head_dim; e += XRT_WAVE) qs[e] = to_float(q[e]);
     wave_sync();
@@ -56,6 +61,7 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
             float dot = 0.f;
             for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(key[d]), dot);
             s = dot * scale;
+            if (distance_slopes) s += slope * (float)(j - pos);
         }
         const float m_new = fmaxf(m, wave_max(s));
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -91,7 +97,7 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
 int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
-                          int window, hipStream_t s) {
+                          int window, const float* distance_slopes, hipStream_t s) {
     XRT_REQUIRE(head_dim <= MAX_HEAD_DIM, "attention: head_dim %d exceeds %d", head_dim, MAX_HEAD_DIM);
     const long items = (long)tokens * n_heads;
     XRT_REQUIRE(items < (1L << 31), "attention: too many (token, head) pairs");
@@ -99,11 +105,11 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
     if (dtype == XRT_F32)
         attention_generic_kernel<float><<<(unsigned)items, XRT_WAVE, 0, s>>>(
             (const float*)qkv, row_width, n_heads, n_kv_heads, head_dim, (const float*)k_cache,
-            (const float*)v_cache, block_table, table_stride, n_blocks, positions, slots, (float*)out, scale, window);
+            (const float*)v_cache, block_table, table_stride, n_blocks, positions, slots, (float*)out, scale, window, distance_slopes);
     else
         attention_generic_kernel<bf16><<<(unsigned)items, XRT_WAVE, 0, s>>>(
             (const bf16*)qkv, row_width, n_heads, n_kv_heads, head_dim, (const bf16*)k_cache,
-            (const bf16*)v_cache, block_table, table_stride, n_blocks, positions, slots, (bf16*)out, scale, window);
+            (const bf16*)v_cache, block_table, table_stride, n_blocks, positions, slots, (bf16*)out, scale, window, distance_slopes);
     XRT_LAUNCH_CHECK("attention (generic)");
     return 0;
 }

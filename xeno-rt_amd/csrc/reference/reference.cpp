@@ -112,7 +112,7 @@ void xrt_ref_qkv_prepare(float* qkv, int tokens, int n_heads, int n_kv_heads, in
 
 void xrt_ref_attention(const float* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const float* k_cache,
                        const float* v_cache, const int* block_table, int table_stride, const int* positions,
-                       const int* slots, float* out, float scale, int window) {
+                       const int* slots, float* out, float scale, int window, const float* distance_slopes) {
     const int width = (n_heads + 2 * n_kv_heads) * head_dim, group = n_heads / n_kv_heads;
     for (int t = 0; t < tokens; ++t)
         for (int head = 0; head < n_heads; ++head) {
@@ -128,7 +128,7 @@ void xrt_ref_attention(const float* qkv, int tokens, int n_heads, int n_kv_heads
                 const float* k = k_cache + (((long)block * n_kv_heads + kv) * BLOCK + key % BLOCK) * head_dim;
                 float dot = 0.f;
                 for (int d = 0; d < head_dim; ++d) dot += q[d] * k[d];
-                scores[key - first] = dot * scale;
+                scores[key - first] = dot * scale + (distance_slopes ? distance_slopes[head] * (float)(key - pos) : 0.f);
             }
             const float largest = *std::max_element(scores.begin(), scores.end());
             float total = 0.f;

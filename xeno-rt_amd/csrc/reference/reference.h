@@ -17,7 +17,7 @@ void xrt_ref_qkv_prepare(float* qkv, int tokens, int n_heads, int n_kv_heads, in
                          const int* block_table, int table_stride, int n_blocks);
 void xrt_ref_attention(const float* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const float* k_cache,
                        const float* v_cache, const int* block_table, int table_stride, const int* positions,
-                       const int* slots, float* out, float scale, int window);
+                       const int* slots, float* out, float scale, int window, const float* distance_slopes);
 void xrt_ref_sample(const float* logits, int rows, int vocab, int* out, const float* temperature, const int* top_k,
                     const float* top_p, const float* penalty, int* history, const int* history_spans,
                     const int* append_at, const float* uniforms);

@@ -62,14 +62,19 @@ int main() {
         check(close_to(r1[0], q1[0] * std::cos(1.0f) - q1[2] * std::sin(1.0f)) && close_to(r1[2], q1[0] * std::sin(1.0f) + q1[2] * std::cos(1.0f)), "rotation pairs (i, i + d/2)");
         check(k_cache[1 * hd + 0] == qkv[width + nh * hd] && v_cache[0 * 64 + 1] == before[width + (nh + nkv) * hd], "cache holds rotated keys and raw values");
         std::vector<float> out(tokens * nh * hd);
-        xrt_ref_attention(qkv.data(), tokens, nh, nkv, hd, k_cache.data(), v_cache.data(), table, 1, positions, slots, out.data(), 0.5f, 0);
+        xrt_ref_attention(qkv.data(), tokens, nh, nkv, hd, k_cache.data(), v_cache.data(), table, 1, positions, slots, out.data(), 0.5f, 0, nullptr);
         bool first_is_value = true;                             // one key: the output is its value
         for (int d = 0; d < hd; ++d) first_is_value = first_is_value && close_to(out[d], before[(nh + nkv) * hd + d]);
         check(first_is_value, "attention over one key");
-        xrt_ref_attention(qkv.data(), tokens, nh, nkv, hd, k_cache.data(), v_cache.data(), table, 1, positions, slots, out.data(), 0.5f, 1);
+        xrt_ref_attention(qkv.data(), tokens, nh, nkv, hd, k_cache.data(), v_cache.data(), table, 1, positions, slots, out.data(), 0.5f, 1, nullptr);
         bool windowed = true;                                   // a window of one: every token sees itself alone
         for (int d = 0; d < hd; ++d) windowed = windowed && close_to(out[nh * hd + d], before[width + (nh + nkv) * hd + d]);
         check(windowed, "attention window");
+        const std::vector<float> steep(nh, 200.0f);              // scores fall by 200 per position of distance: again itself alone
+        xrt_ref_attention(qkv.data(), tokens, nh, nkv, hd, k_cache.data(), v_cache.data(), table, 1, positions, slots, out.data(), 0.5f, 0, steep.data());
+        bool biased = true;
+        for (int d = 0; d < hd; ++d) biased = biased && close_to(out[nh * hd + d], before[width + (nh + nkv) * hd + d]);
+        check(biased, "attention scores biased by distance");
         const float gain[4] = {1, 1, 1, 1};
         xrt_ref_qkv_prepare(qkv.data(), tokens, nh, nkv, hd, positions, slots, gain, gain, 0.f, nullptr, 0, 1.0f, nullptr, nullptr, table, 1, 1);
         float squares = 0.f;

@@ -126,13 +126,15 @@ int xrt_linear_qkv(const void* a, const void* w, const xrt_packing* packing, int
 // step may be described (seq_* arrays, n_seqs, the largest token count of a sequence and the
 // longest sequence after the step): then the matrix-core kernels can be used; a decode step (max_count 1)
 // then needs a workspace of xrt_attention_workspace(...) floats for the partial results of the parts that
-// its keys are cut into (0: none), and takes the general kernel without it.
+// its keys are cut into (0: none), and takes the general kernel without it. distance_slopes (null: none): one
+// float per query head; a key at position j then adds slope * (j - P) to the scaled score of the query at
+// position P, for position encodings that act on the scores (the general kernel serves them).
 long xrt_attention_workspace(int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int window,
                              int max_count, int max_context);
 int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                   const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                   int n_blocks, const int* positions, const int* slots, void* out, float scale, int window,
-                  const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs,
+                  const float* distance_slopes, const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs,
                   int max_count, int max_context, float* workspace, long workspace_floats, void* stream);
 
 // one token per row of float32 logits. With a workspace of xrt_sample_workspace(rows, vocab) bytes (0: this

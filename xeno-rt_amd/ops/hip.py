@@ -375,7 +375,9 @@ class HipOps:
             raise KernelError("block table: expected [slots, blocks]")
         return kv.k, kv.v, kv.block_table, kv.block_table.shape[1], n_blocks
 
-    def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None):
+    def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None):
+        """Causal attention of the step's tokens over the cache. distance_slopes: float32 [n_heads], or None; a key at
+        position j adds slope * (j - P) to the scaled score of the query at position P."""
         from ..cache import BLOCK_TOKENS
         tokens = qkv.shape[0]
         width = (n_heads + 2 * n_kv_heads) * head_dim
@@ -384,6 +386,8 @@ class HipOps:
         self._require(batch.positions, "positions", torch.int32, (tokens,), qkv)
         self._require(batch.slots, "slots", torch.int32, (tokens,), qkv)
         k_cache, v_cache, table, stride, n_blocks = self._kv(kv, qkv, n_kv_heads, head_dim)
+        if distance_slopes is not None:
+            self._require(distance_slopes, "attention distance_slopes", torch.float32, (n_heads,), qkv)
         # the step's sequences, if the batch describes them: lets the matrix-core kernels run
         offsets = getattr(batch, "sequence_offsets", None)
         seq_slots = getattr(batch, "sequence_slots", None)
@@ -405,7 +409,7 @@ class HipOps:
         self._check(self.lib.xrt_attention(
             _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(k_cache), _ptr(v_cache),
             _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out),
-            ctypes.c_float(scale), int(window or 0), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
+            ctypes.c_float(scale), int(window or 0), _ptr(distance_slopes), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
 
     def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms,

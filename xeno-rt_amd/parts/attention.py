@@ -116,7 +116,9 @@ class Attention(Mixer):
                 ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots, kv=write_to, longest_run=longest_run)
 
         out = rt.empty((tokens, self.q_width))
-        ops.attention(qkv, *dims, kv, batch, out, scale=self.scale, window=self.window)
+        slopes = None if self.position is None else self.position.score_slopes()
+        ops.attention(qkv, *dims, kv, batch, out, scale=self.scale, window=self.window,
+                      **({} if slopes is None else {"distance_slopes": slopes}))
         return ops.linear(out, self.w_o, residual, accumulate=True,
                           then_norm=None if then is None else then.row_scale())
 

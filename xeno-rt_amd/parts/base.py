@@ -175,6 +175,11 @@ class PositionEncoding(Part):
         """
         raise NotImplementedError
 
+    def score_slopes(self) -> Optional[torch.Tensor]:
+        """For an encoding that acts on the attention scores: float32 [n_heads] on the device; a key at position j
+        then adds slope * (j - P) to the scaled score of the query at position P. None: the scores stay as they are."""
+        return None
+
 
 # A mixer, a feed-forward or a block may set `passes_norms = True`. It then promises two things.
 # Its `forward` takes a keyword `then`: the norm that follows it on the residual stream, or None. If
