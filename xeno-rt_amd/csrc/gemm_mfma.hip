@@ -603,8 +603,8 @@ SplitPlan split_plan(int M, int N, int K, int mode) {
         // The tiles of 128 x 128, which fill the chip without a second kernel, read their operands from LDS
         // more often for the same products and take longer here.
         splits = (int)(256 / large_tiles);
-        splits = splits > 4 ? 4 : splits;
-        least = 32;
+        splits = splits > 8 ? 8 : splits;
+        least = 24;
         tile = 256;
     } else {
         const long tiles = (long)((M + 127) / 128) * tiles_n;  // two of these workgroups share a compute unit
