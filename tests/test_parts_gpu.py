@@ -132,10 +132,10 @@ def test_attention_part_prompt_then_decode(dtype, nh, nkv, hd, qk_norm):
     assert part.scale == 1.0 / math.sqrt(hd)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_attention_part_with_a_position_encoding_on_the_scores(dtype):
+def attention_with_scores_biased_by_distance(rt, dtype, device):
     """A position encoding defined here, which leaves q and k alone and lowers the scores of far keys instead
-    (one slope per head): the attention part hands its slopes to the kernel. A prompt, then single tokens."""
+    (one slope per head): the attention part hands its slopes to the kernel. A prompt, then single tokens.
+    Returns (what the part added to the residual, the same by plain arithmetic, the same without the slopes)."""
     from xeno_rt_amd.cache import SequenceCache
     from xeno_rt_amd.parts import Attention
     from xeno_rt_amd.parts.base import PositionEncoding
@@ -159,8 +159,8 @@ def test_attention_part_with_a_position_encoding_on_the_scores(dtype):
     hidden, nh, nkv, hd, length, prompt = 80, 4, 2, 128, 100, 70
     part = Attention("a.", hidden, nh, nkv, hd, position=DistanceBias(nh))
     w = weights_for(part, 5, std=0.15)
-    part.bind(w, runtime(dtype))
-    cache = SequenceCache([part.cache_needs()], [0], 256, 1, 128, DT[dtype], DEV)
+    part.bind(w, rt)
+    cache = SequenceCache([part.cache_needs()], [0], 256, 1, 128, DT[dtype], device)
     h = torch.randn(length, hidden, generator=torch.Generator().manual_seed(4)).to(DT[dtype])
     x = h.double()
     q, k, v = (P.linear(x, w[f"a.{n}_proj.weight"].double()) for n in "qkv")
@@ -178,13 +178,22 @@ def test_attention_part_with_a_position_encoding_on_the_scores(dtype):
     got = []
     at = 0
     for count in [prompt] + [1] * (length - prompt):
-        batch, _ = batch_for(cache, [slot], [count])
-        residual = torch.zeros(count, hidden, device=DEV)
-        part.forward(h[at:at + count].to(DEV), batch, cache.layer_cache(0), residual)
+        from xeno_rt_amd.engine.batch import build_batch
+        cache.reserve(slot, at + count)
+        cache.sync()
+        batch = build_batch([slot], [[0] * count], [at], [[]], device)
+        residual = torch.zeros(count, hidden, device=device)
+        part.forward(h[at:at + count].to(device), batch, cache.layer_cache(0), residual)
         got.append(residual.clone())
         at += count
         cache.commit(slot, at)
-    assert rel(torch.cat(got), want) < TOL[dtype]
+    return torch.cat(got), want, unbiased
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_part_with_a_position_encoding_on_the_scores(dtype):
+    got, want, unbiased = attention_with_scores_biased_by_distance(runtime(dtype), dtype, DEV)
+    assert rel(got, want) < TOL[dtype]
     assert rel(unbiased, want) > 10 * TOL[dtype]                # the slopes do change the result
 
 

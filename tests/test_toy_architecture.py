@@ -6,7 +6,7 @@ import torch
 
 from helpers import assert_greedy_tokens, assert_logits, run_batched, run_tail_decoded, run_whole, token_ids
 from ops_emulation import EmulatedOps
-from test_parts_gpu import define_toy, plain_toy
+from test_parts_gpu import attention_with_scores_biased_by_distance, define_toy, plain_toy
 
 
 def test_toy_architecture_on_the_cpu_stand_in(tmp_path):
@@ -37,3 +37,11 @@ def test_toy_architecture_on_the_cpu_stand_in(tmp_path):
     assert_greedy_tokens(logits_of, requests[2][:3], out[1].tokens, "float32", 1.3, "toy generation with a penalty")
     engine.cache.check()
     assert engine.cache.slots.n_held == 0
+
+
+def test_a_position_encoding_on_the_scores_on_the_cpu_stand_in():
+    from xeno_rt_amd.parts import Runtime
+    got, want, unbiased = attention_with_scores_biased_by_distance(Runtime(EmulatedOps(), torch.float32, "cpu"), "float32", "cpu")
+    error = float((got.double() - want).abs().max()) / float(want.abs().max())
+    assert error < 2e-5
+    assert float((unbiased - want).abs().max()) / float(want.abs().max()) > 1e-3
