@@ -43,8 +43,8 @@ __device__ __forceinline__ int key_of_row(int r) { return (r / 16) * 16 + ((r % 
 // Wavefronts 4..7 first take the early tile's; when its last block of keys is done they write its result and
 // turn to the late tile as well: from then on the blocks of a stage are dealt out in turn, one to wavefront w
 // and one to wavefront w + 4, which hold the same 32 queries, and in the end the two merge what they have
-// (maximum, sum, weighted values) through LDS. Every workgroup of a sequence thus has the same work, about half
-// of what the last tile of 256 queries had on its own.
+// (maximum, sum, weighted values) through LDS. Every workgroup of a sequence thus has the same work: with tiles
+// that stand alone the last one of a causal sequence has twice the mean, and the step ends when it does.
 constexpr int GROUPS = 4;              // groups of 32 queries in a tile
 constexpr int WAVES = 2 * GROUPS;
 constexpr int QW = GROUPS * QT;        // queries of a tile
