@@ -217,6 +217,8 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None,
                         help="run fewer layers of the same sizes (both numbers are reported)")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--context", type=int, default=CONTEXT,
+                        help="tokens every sequence holds when the timed decode steps end (the headline: 4096)")
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
     parser.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
@@ -232,15 +234,17 @@ def main() -> int:
     shape = SHAPES[args.shape]
     layers = args.layers if args.layers is not None else shape["num_hidden_layers"]
     batch = args.batch if args.batch is not None else HEADLINE_BATCH[args.shape]
-    config = parse_config(dict(shape, num_hidden_layers=layers))
+    config = parse_config(dict(shape, num_hidden_layers=layers,
+                               max_position_embeddings=max(shape["max_position_embeddings"], args.context, LONG_PREFILL)))
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     element = 2 if short == "bf16" else 4
     if args.phase != "all":
         args.skip_points = True
     others = () if args.skip_points else tuple(b for b in OTHER_BATCHES[args.shape] if b != batch)
     largest_batch = max((batch,) + others)
-    engine = Engine.random(config, seed=args.seed, dtype=args.dtype, max_tokens=largest_batch * CONTEXT,
-                           max_slots=largest_batch, max_context=CONTEXT if args.skip_points else max(CONTEXT, LONG_PREFILL))
+    context = args.context
+    engine = Engine.random(config, seed=args.seed, dtype=args.dtype, max_tokens=largest_batch * context,
+                           max_slots=largest_batch, max_context=context if args.skip_points else max(context, LONG_PREFILL))
     bench = Bench(engine, args.seed)
 
     def priced(ms, mean_length, sequences):
@@ -252,10 +256,10 @@ def main() -> int:
         print(json.dumps({"phase": "prefill", "tokens": PREFILL_TOKENS, "ms": round(seconds * 1e3, 3),
                           "frac": round(prefill_flops(config, [PREFILL_TOKENS]) / seconds / PEAK_FLOPS[short], 4)}), flush=True)
         return 0
-    tokens_per_s, ms_per_step, mean_length = bench.decode(batch, args.steps, args.warmup, CONTEXT, check=args.phase == "all")
+    tokens_per_s, ms_per_step, mean_length = bench.decode(batch, args.steps, args.warmup, context, check=args.phase == "all")
     if args.phase == "decode":
-        print(json.dumps({"phase": "decode", "batch": batch, "ms_per_step": round(ms_per_step, 4),
-                          "tokens_per_s": round(tokens_per_s, 1)}), flush=True)
+        print(json.dumps({"phase": "decode", "batch": batch, "context": context, "ms_per_step": round(ms_per_step, 4),
+                          "tokens_per_s": round(tokens_per_s, 1), "frac": round(priced(ms_per_step, mean_length, batch) / PEAK_HBM_GBS, 4)}), flush=True)
         return 0
     achieved = priced(ms_per_step, mean_length, batch)
     read_gbs, mfma_tflops, mfma_random_tflops = measured_ceilings(engine.ops, engine.device)
@@ -272,7 +276,7 @@ def main() -> int:
     points = {}
     if not args.skip_points:
         for other in others:
-            value, ms, length = bench.decode(other, args.steps, args.warmup, CONTEXT)
+            value, ms, length = bench.decode(other, args.steps, args.warmup, context)
             points[f"decode_b{other}"] = round(value, 1)
             points[f"decode_b{other}_ms"] = round(ms, 4)
             points[f"decode_b{other}_frac"] = round(priced(ms, length, other) / PEAK_HBM_GBS, 4)
@@ -281,7 +285,7 @@ def main() -> int:
         points[f"decode_b{batch}_ctx{SHORT_CONTEXT}"] = round(value, 1)
         points[f"decode_b{batch}_ctx{SHORT_CONTEXT}_ms"] = round(ms, 4)
         points[f"decode_b{batch}_ctx{SHORT_CONTEXT}_frac"] = round(priced(ms, length, batch) / PEAK_HBM_GBS, 4)
-        if largest_batch * CONTEXT >= LONG_PREFILL:
+        if largest_batch * context >= LONG_PREFILL:
             seconds = bench.prefill([LONG_PREFILL], repeats=2)
             points[f"prefill_{LONG_PREFILL}"] = round(LONG_PREFILL / seconds, 1)
             points[f"prefill_{LONG_PREFILL}_ms"] = round(seconds * 1e3, 3)
@@ -304,7 +308,7 @@ def main() -> int:
                    "hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size,
                    "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
                    "head_dim": config.head_dim, "vocab_size": config.vocab_size, "rope_theta": config.rope_theta,
-                   "rms_norm_eps": config.rms_norm_eps, "qk_norm": config.qk_norm, "global_batch": batch, "seq_len": CONTEXT,
+                   "rms_norm_eps": config.rms_norm_eps, "qk_norm": config.qk_norm, "global_batch": batch, "seq_len": context,
                    "prefill_tokens": PREFILL_TOKENS, "sampling": "greedy on device", "parallelism": "single GPU"},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
