@@ -230,6 +230,32 @@ def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n, packed):
     assert (again is not None) == (m <= 16)                     # 64 to 127 columns: only the kernel for up to 16 rows writes them
 
 
+@pytest.mark.parametrize("m,hidden,k", [(520, 1032, 4160), (2048, 4096, 4096), (600, 520, 8192), (1024, 8192, 4096)])
+@pytest.mark.parametrize("gain_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("packed", [False, True])
+def test_rmsnorm_done_by_the_second_kernel_of_a_product_of_many_rows(ops, m, hidden, k, gain_dtype, packed):
+    # x += a w^T; y = rmsnorm(x) * gain: with many rows, few columns and a long k the product runs as large tiles that split
+    # k, and the kernel that adds the parts writes y as well: the norm kernel's result to the bit
+    a = rand(m, k, dtype=torch.bfloat16, seed=1)
+    w = rand(hidden, k, dtype=torch.bfloat16, seed=2, scale=0.1)
+    x = rand(m, hidden, seed=3, scale=2.0)
+    x[m // 2] *= 50.0
+    gain = (rand(hidden, seed=4) + 1.0).to(gain_dtype)
+    eps = 1e-3
+    fresh = x.double().cpu() + a.double().cpu() @ w.double().cpu().t()
+    alone = x.clone()
+    w = packed_or_not(ops, w, packed)
+    normed = ops.linear(a, w, x, accumulate=True, then_norm=(gain, eps))
+    assert isinstance(normed, torch.Tensor) and normed.dtype == torch.bfloat16 and normed.shape == (m, hidden)
+    assert rel(x.cpu(), fresh) < 1e-5
+    assert ops.linear(a, w, alone, accumulate=True) is None
+    assert rel(alone.cpu(), fresh) < 1e-5
+    by_the_norm_kernel = torch.empty(m, hidden, dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(x, gain, eps, by_the_norm_kernel)
+    assert torch.equal(normed, by_the_norm_kernel)
+    assert rel(normed.cpu(), P.rmsnorm(fresh, gain.double().cpu(), eps)) < ULP["bfloat16"]
+
+
 def test_rmsnorm_is_left_to_its_own_kernel_where_the_products_cannot_do_it(ops):
     gain = rand(200, seed=4).to(torch.bfloat16)
     for m, dtype in ((17, torch.bfloat16), (300, torch.bfloat16), (4, torch.float32)):

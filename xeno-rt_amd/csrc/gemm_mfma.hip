@@ -588,7 +588,9 @@ constexpr int SPLIT_BM = 64, SPLIT_BN = 128;
 
 struct SplitPlan { int splits, k_per_split; long rows_w; int tile; };      // tile: rows of x per tile (64, 128 or 256)
 
-SplitPlan split_plan(int M, int N, int K, int mode) {
+// whole_norm: an RMSNorm follows that the second kernel can do outright, which is worth a split in two where the product alone
+// would do as well without (k from 4096 on instead of from 8192 on).
+SplitPlan split_plan(int M, int N, int K, int mode, bool whole_norm = false) {
     const long rows_w = mode == MODE_GATED ? 2L * N : N;
     const long tiles_n = (rows_w + SPLIT_BN - 1) / SPLIT_BN;
     const int units = K / 64;                                  // k is dealt out in pieces of 64
@@ -597,7 +599,7 @@ SplitPlan split_plan(int M, int N, int K, int mode) {
     if (M <= SPLIT_BM) {
         splits = (int)(256 / tiles_n);                         // one workgroup per compute unit, or fewer
         least = 1;
-    } else if (large_tiles <= 128 && M >= 512 && mode != MODE_GATED && units >= 128) {
+    } else if (large_tiles <= 128 && M >= 512 && mode != MODE_GATED && units >= (whole_norm ? 64 : 128)) {
         // Many rows and a very long k, but so few columns that the largest tiles would leave half of the compute
         // units idle (the projection back from the feed-forward's width): the large tiles split k between them.
         // The tiles of 128 x 128, which fill the chip without a second kernel, read their operands from LDS
@@ -708,6 +710,58 @@ __global__ void __launch_bounds__(256) split_reduce_wide_kernel(const float* __r
     }
 }
 
+// The second kernel of an accumulating product of many rows that an RMSNorm follows: a workgroup takes a whole row, adds the
+// parts onto the residual and writes the row's norm as well. The norm is the norm kernel's (elementwise.hip) to the bit: the same
+// four columns a thread, the same order of the sum of squares, (x * 1/rms) * gain.
+constexpr int NORM_QUADS = 8;                      // four-column pieces a thread holds: rows of up to 8 * 256 * 4 columns
+template <typename T> struct alignas(sizeof(T) * 4) Four { T e[4]; };
+template <typename TW>
+__global__ void __launch_bounds__(256) split_reduce_rmsnorm_kernel(const float* __restrict__ parts, int splits, long count, int N,
+                                                                    float* __restrict__ out, const TW* __restrict__ gain, float eps,
+                                                                    bf16* __restrict__ normed) {
+    __shared__ float scratch[32];
+    const long row = (long)blockIdx.x * N;
+    const int quads = N / 4;
+    float4 kept[NORM_QUADS];
+    Four<TW> weight[NORM_QUADS];
+#pragma unroll
+    for (int i = 0; i < NORM_QUADS; ++i) {
+        const int q = threadIdx.x + i * 256;
+        kept[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        weight[i] = Four<TW>{};
+        if (q < quads) {
+            const long index = row + 4L * q;
+            float4 sum = *reinterpret_cast<const float4*>(parts + index);
+            for (int p = 1; p < splits; ++p) {
+                const float4 part = *reinterpret_cast<const float4*>(parts + p * count + index);
+                sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+            }
+            const float4 before = *reinterpret_cast<const float4*>(out + index);
+            kept[i] = make_float4(before.x + sum.x, before.y + sum.y, before.z + sum.z, before.w + sum.w);
+            *reinterpret_cast<float4*>(out + index) = kept[i];
+            weight[i] = *reinterpret_cast<const Four<TW>*>(gain + 4 * q);
+        }
+    }
+    float squares = 0.f;
+#pragma unroll
+    for (int i = 0; i < NORM_QUADS; ++i)
+        squares = fmaf(kept[i].x, kept[i].x, fmaf(kept[i].y, kept[i].y, fmaf(kept[i].z, kept[i].z, fmaf(kept[i].w, kept[i].w, squares))));
+    squares = block_sum(squares, scratch);
+    const float inv_rms = 1.0f / sqrtf(squares / (float)N + eps);
+#pragma unroll
+    for (int i = 0; i < NORM_QUADS; ++i) {
+        const int q = threadIdx.x + i * 256;
+        if (q < quads) {
+            Four<bf16> r;
+            r.e[0] = from_float<bf16>((kept[i].x * inv_rms) * to_float(weight[i].e[0]));
+            r.e[1] = from_float<bf16>((kept[i].y * inv_rms) * to_float(weight[i].e[1]));
+            r.e[2] = from_float<bf16>((kept[i].z * inv_rms) * to_float(weight[i].e[2]));
+            r.e[3] = from_float<bf16>((kept[i].w * inv_rms) * to_float(weight[i].e[3]));
+            *reinterpret_cast<Four<bf16>*>(normed + row + 4L * q) = r;
+        }
+    }
+}
+
 // The second kernel of a q/k/v projection split along k (no head norms, the rotation over the whole head):
 // a thread adds up the two outputs that the rotation pairs (dims d and d + head_dim / 2 of one head), for
 // NORM 1 scales them by the row's 1 / rms, rotates q and k by the token's position, writes bfloat16 q/k/v and
@@ -782,9 +836,15 @@ __global__ void __launch_bounds__(256) split_reduce_qkv_kernel(const float* __re
 template <typename TO>
 int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int mode, int activation, const Packing& packing,
                  float* workspace, const xrt_linear_norm* norm, const QkvAfter* after, hipStream_t s) {
-    const SplitPlan plan = split_plan(M, N, K, mode);
+    // the whole norm after an accumulating product of many rows: normed rows asked for, and no sums of squares
+    const bool whole_norm = norm && norm->scaled_out && !norm->squares_out && !norm->squares_in;
+    const SplitPlan plan = split_plan(M, N, K, mode, whole_norm);
     const bool scaled = norm && norm->squares_in, emits = norm && norm->squares_out;
-    XRT_REQUIRE(!norm || M <= SPLIT_BM, "linear (mfma): the norm around a product takes at most %d rows here", SPLIT_BM);
+    XRT_REQUIRE(!norm || M <= SPLIT_BM || whole_norm, "linear (mfma): the halves of a norm around a product take at most %d rows here", SPLIT_BM);
+    if (whole_norm)
+        XRT_REQUIRE(M > SPLIT_BM && mode == MODE_ACCUMULATE && sizeof(TO) == 4 && plan.tile == 256 && plan.splits > 1 && N % 4 == 0 &&
+                    N <= NORM_QUADS * 256 * 4 && norm->gain && (uintptr_t)out % 16 == 0 && (uintptr_t)norm->scaled_out % 8 == 0,
+                    "linear (mfma): M=%d N=%d K=%d is not a product whose second kernel does the norm after it", M, N, K);
     const RowScale scale = scaled ? RowScale{norm->squares_in, norm->tiles_in, norm->width_in, norm->eps, activation}
                                   : RowScale{nullptr, 0, 0, 0.f, activation};
     XRT_REQUIRE(!after || (plan.splits > 1 && mode == MODE_STORE && sizeof(TO) == 2),
@@ -818,6 +878,17 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
             if (scaled) split_reduce_qkv_kernel<1><<<pair_blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around, *after);
             else split_reduce_qkv_kernel<0><<<pair_blocks, 256, 0, s>>>(workspace, plan.splits, M, N, out, around, *after);
             XRT_LAUNCH_CHECK("linear (split reduce, q/k/v)");
+        }
+        return 0;
+    }
+    if (whole_norm) {
+        if constexpr (sizeof(TO) == 4) {
+            const long count = (long)M * N;
+            if (norm->gain_dtype == XRT_F32)
+                split_reduce_rmsnorm_kernel<float><<<M, 256, 0, s>>>(workspace, plan.splits, count, N, out, (const float*)norm->gain, norm->eps, (bf16*)norm->scaled_out);
+            else
+                split_reduce_rmsnorm_kernel<bf16><<<M, 256, 0, s>>>(workspace, plan.splits, count, N, out, (const bf16*)norm->gain, norm->eps, (bf16*)norm->scaled_out);
+            XRT_LAUNCH_CHECK("linear (split reduce with the norm after it)");
         }
         return 0;
     }
@@ -865,6 +936,19 @@ bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, i
     if (plan.splits == 1) return M <= SPLIT_BM;               // more rows and enough tiles without a split: the kernels above
     if (plan.rows_w * (long)M >= (1L << 31)) return false;
     *workspace_floats = (long)plan.splits * M * plan.rows_w;
+    return true;
+}
+
+// Whether an accumulating product of many rows runs as large tiles that split k, so that its second kernel can do the
+// RMSNorm that follows it outright; and the floats of workspace it then needs.
+bool xrt_linear_split_takes_whole_norm(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats) {
+    *workspace_floats = 0;
+    if (mode != MODE_ACCUMULATE || M <= SPLIT_BM || K % 64 != 0 || N % 4 != 0 || N > NORM_QUADS * 256 * 4 ||
+        !xrt_linear_mfma_accepts(a, w, M, N, K, mode))
+        return false;
+    const SplitPlan plan = split_plan(M, N, K, mode, true);
+    if (plan.tile != 256 || plan.splits < 2 || (long)M * N >= (1L << 31)) return false;
+    *workspace_floats = (long)plan.splits * M * N;
     return true;
 }
 

@@ -11,6 +11,7 @@ int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int 
 
 bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats);
 bool xrt_linear_split_takes_norm(const void* a, const void* w, int M, int N, int K, int mode);
+bool xrt_linear_split_takes_whole_norm(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats);
 bool xrt_linear_split_takes_qkv(const void* a, const void* w, int M, int N, int K, const QkvAfter& after, long* workspace_floats);
 int xrt_linear_split_qkv(const void* a, const void* w, void* qkv, int M, int N, int K, const Packing& packing, float* workspace,
                          const xrt_linear_norm* norm, const QkvAfter& after, hipStream_t s);
@@ -104,7 +105,16 @@ extern "C" int xrt_linear_takes_norm(const void* a, const void* w, const xrt_pac
     } else if (xrt_linear_skinny_accepts(a, w, M, K) && xrt_linear_skinny_takes_norm(M)) {
         return 1;
     }
-    return xrt_linear_split_takes_norm(a, w, M, N, K, mode) ? 1 : 0;
+    if (xrt_linear_split_takes_norm(a, w, M, N, K, mode)) return 1;
+    long unused = 0;
+    return xrt_linear_split_takes_whole_norm(a, w, M, N, K, mode, &unused) ? 2 : 0;
+}
+
+// Floats of workspace for xrt_linear_normed where xrt_linear_takes_norm says 2 (the product's second kernel does the whole norm).
+extern "C" long xrt_linear_whole_norm_workspace(const void* a, const void* w, int dtype, int M, int N, int K, int mode) {
+    long need = 0;
+    if (dtype == XRT_BF16) xrt_linear_split_takes_whole_norm(a, w, M, N, K, mode, &need);
+    return need;
 }
 
 // Tiles of columns for which an accumulating product that xrt_linear_takes_norm accepts writes sums of
@@ -134,6 +144,16 @@ extern "C" int xrt_linear_normed(const void* a, const void* w, const xrt_packing
         XRT_REQUIRE(norm->width_in == K && norm->tiles_in >= (K + 15) / 16 && norm->tiles_in <= (K + 7) / 8,     // tiles of 8 to 16 columns
                     "linear with norm: sums of squares of %d tiles over %d columns for a of %d columns",
                     norm->tiles_in, norm->width_in, K);
+    const bool whole_norm = norm->scaled_out && norm->gain && !norm->squares_out && !norm->squares_in;
+    if (whole_norm) {
+        // many rows: the product's second kernel adds the parts, and writes the rows' RMSNorm (gain, eps) to scaled_out
+        long need = 0;
+        XRT_REQUIRE(norm->gain_dtype == XRT_F32 || norm->gain_dtype == XRT_BF16, "linear with norm: unknown gain dtype %d", norm->gain_dtype);
+        XRT_REQUIRE(xrt_linear_split_takes_whole_norm(a, w, M, N, K, mode, &need) && out_dtype == XRT_F32,
+                    "linear with norm: M=%d N=%d K=%d mode %d is not a product that does the whole norm after it", M, N, K, mode);
+        XRT_REQUIRE(workspace != nullptr && workspace_floats >= need, "linear with norm: the workspace needs %ld floats", need);
+        return xrt_linear_split(a, w, out, out_dtype, M, N, K, mode, activation, layout, workspace, norm, (hipStream_t)stream);
+    }
     const bool emits = norm->squares_out || norm->scaled_out || norm->gain;
     if (emits) {
         XRT_REQUIRE(mode == 1, "linear with norm: only an accumulating product writes what the norm after it needs");

@@ -90,6 +90,10 @@ int xrt_linear_static(const void* a, const void* w, int dtype, void* out, int ou
 // xrt_linear_takes_norm says whether an accumulating product can write these (bfloat16 operands, up to 64 rows,
 // and with more than 16 rows: split along k, N a multiple of 64); then the product after it (same rows) can
 // take them, and xrt_linear_normed refuses what cannot. workspace: as for xrt_linear.
+// xrt_linear_takes_norm returns 2 for an accumulating product of many rows that runs as large tiles splitting k: its second
+// kernel then does the whole norm. For that, scaled_out, gain, gain_dtype and eps are set and the other fields left zero:
+// scaled_out[m, n] = bfloat16((x[m, n] / rms(x[m, :])) * gain[n]), the norm kernel's result to the bit, which the product after
+// it takes like any rows. Its workspace has xrt_linear_whole_norm_workspace(...) floats.
 #define XRT_SQUARES_STRIDE 64
 typedef struct xrt_linear_norm {
     const float* squares_in; int tiles_in; int width_in; float eps;
@@ -97,6 +101,7 @@ typedef struct xrt_linear_norm {
 } xrt_linear_norm;
 int xrt_linear_takes_norm(const void* a, const void* w, const xrt_packing* packing, int dtype, int M, int N, int K, int mode);
 int xrt_linear_norm_tiles(const void* a, const void* w, const xrt_packing* packing, int dtype, int M, int N, int K);   // rows of the table at squares_out
+long xrt_linear_whole_norm_workspace(const void* a, const void* w, int dtype, int M, int N, int K, int mode);
 int xrt_linear_normed(const void* a, const void* w, const xrt_packing* packing, int dtype, void* out, int out_dtype, int M, int N,
                       int K, int mode, const xrt_linear_norm* norm, float* workspace, long workspace_floats, void* stream);
 

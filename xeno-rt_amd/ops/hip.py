@@ -140,6 +140,7 @@ class HipOps:
             raise KernelError(f"{path} keeps {int(self.lib.xrt_block_tokens())} tokens in a cache block, "
                               f"the cache's bookkeeping {BLOCK_TOKENS}: library and package do not belong together")
         self.lib.xrt_linear_workspace.restype = ctypes.c_long
+        self.lib.xrt_linear_whole_norm_workspace.restype = ctypes.c_long
         self.lib.xrt_attention_workspace.restype = ctypes.c_long
         self.lib.xrt_probe_read_bytes.restype = ctypes.c_long
         self.lib.xrt_sample_workspace.restype = ctypes.c_long
@@ -259,7 +260,21 @@ class HipOps:
         # the norm after an accumulating product: only if that product, and one of the same rows
         # over the n columns it writes, can take it
         emit = None
-        if then_norm is not None and mode == 1 and n % 8 == 0 and self.lib.xrt_linear_takes_norm(*packed, m, n, k, mode):
+        takes = int(self.lib.xrt_linear_takes_norm(*packed, m, n, k, mode)) if then_norm is not None and mode == 1 and n % 8 == 0 else 0
+        if takes == 2 and scaled is None and out.dtype == torch.float32:
+            # many rows: the product's second kernel adds its parts and writes the rows' norm outright
+            gain, eps = then_norm
+            self._require(gain, "norm gain", None, (n,), a)
+            normed = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+            norm = _LinearNorm()
+            norm.eps = float(eps)
+            norm.scaled_out, norm.gain, norm.gain_dtype = normed.data_ptr(), gain.data_ptr(), _code(gain)
+            need = int(self.lib.xrt_linear_whole_norm_workspace(*sizes, m, n, k, mode))
+            workspace = torch.empty(need, dtype=torch.float32, device=a.device)
+            self._check(self.lib.xrt_linear_normed(*packed, _ptr(out), _code(out), m, n, k, coded_mode, ctypes.byref(norm),
+                                                   _ptr(workspace), ctypes.c_long(need), self._stream(a)))
+            return normed
+        if takes == 1:
             gain, eps = then_norm
             self._require(gain, "norm gain", None, (n,), a)
             emit = Prescaled(torch.empty((m, n), dtype=torch.bfloat16, device=a.device),
@@ -288,8 +303,9 @@ class HipOps:
 
     def linear(self, a, w, out, accumulate=False, then_norm: Optional[Tuple[torch.Tensor, float]] = None):
         """out (+)= a w^T. `a` may be a Prescaled. then_norm = (gain, eps) of an RMSNorm that follows an
-        accumulating product: if this product can, it returns a Prescaled of the updated `out` for the
-        product after the norm; None means that the caller runs the norm."""
+        accumulating product: if this product can, it returns the normed rows of the updated `out` for the
+        product after the norm (a Prescaled, whose division that product does; with many rows the normed
+        rows themselves); None means that the caller runs the norm."""
         return self._linear(a, w, out, 1 if accumulate else 0, w.shape[0], then_norm)
 
     def linear_glu(self, a, w_gate_up, out, activation: str = "silu"):
