@@ -19,10 +19,10 @@ def pytest_configure(config):
 def pytest_terminal_summary(terminalreporter):
     """The largest errors against the plain model that the run has seen, next to their limits."""
     import helpers
-    for dtype, (worst, rms) in sorted(helpers.SEEN.items()):
+    for dtype, (worst, rms, what) in sorted(helpers.SEEN.items()):
         limit = helpers.TOLERANCE[dtype]
         terminalreporter.write_line(f"logit errors seen [{dtype}]: max {worst:.2e} (limit {limit['max']:.1e}), "
-                                    f"rms {rms:.2e} (limit {limit['rms']:.1e})")
+                                    f"rms {rms:.2e} (limit {limit['rms']:.1e}); the largest in: {what or 'unnamed'}")
 
 
 def pytest_collection_modifyitems(config, items):

@@ -9,9 +9,9 @@ import torch
 #            with the tests' weights (std 0.2: sharp attention, gains above one) that comes
 #            to one or two percent of the largest logit. The root-mean-square bound is
 #            tighter because it does not ride on the single worst element. Largest errors seen over all
-#            tests (printed at the end of every run): max 3.4e-2, rms 7.0e-3 with the tiny models' weights
-#            of std 0.2; max 1.5e-2, rms 2.9e-3 at real layer sizes with std 0.02. The limits are
-#            1.5 and 2 times the former.
+#            tests (printed at the end of every run, with the test that had them): max 4.0e-2, rms 7.0e-3 with
+#            the tiny models' weights of std 0.2 (the stand-in for the kernels on the CPU, which shares no code
+#            with them, has 3.6e-2 at the same request); max 1.5e-2, rms 2.9e-3 at real layer sizes with std 0.02.
 TOLERANCE = {"float32": dict(max=2e-5, rms=5e-6), "bfloat16": dict(max=5e-2, rms=1.5e-2)}
 
 
@@ -23,14 +23,16 @@ def errors(got: torch.Tensor, want: torch.Tensor):
     return float(diff.abs().max()) / scale, float(diff.pow(2).mean().sqrt()) / scale
 
 
-SEEN = {}       # dtype -> [largest max error, largest rms error] that passed: printed at the end of a run
+SEEN = {}       # dtype -> [largest max error, largest rms error, what had the former] that passed: printed at the end of a run
 
 
 def assert_logits(got, want, dtype, what=""):
     assert torch.isfinite(got).all(), f"{what}: logits are not finite"
     worst, rms = errors(got, want)
-    seen = SEEN.setdefault(dtype, [0.0, 0.0])
-    seen[0], seen[1] = max(seen[0], worst), max(seen[1], rms)
+    seen = SEEN.setdefault(dtype, [0.0, 0.0, ""])
+    if worst > seen[0]:
+        seen[0], seen[2] = worst, what
+    seen[1] = max(seen[1], rms)
     limit = TOLERANCE[dtype]
     assert worst <= limit["max"] and rms <= limit["rms"], \
         f"{what} [{dtype}]: max error {worst:.3e} (limit {limit['max']:.1e}), rms {rms:.3e} (limit {limit['rms']:.1e})"
