@@ -8,8 +8,8 @@ the GPU it is the plain reference that each kernel is compared with, alone and a
 sizes other than the engine's. The engine itself never falls back to it.
 
 Layout facts it shares with the kernels (they are the contract, not code):
-qkv rows are [q heads | k heads | v heads]; a cache block holds BLOCK tokens,
-keys as [kv_head][token][dim], values as [kv_head][dim][token].
+qkv rows are [q heads | k heads | v heads]; a cache block holds BLOCK tokens of
+every key/value head, in the order that cache_order.py spells out.
 """
 from __future__ import annotations
 
@@ -17,6 +17,7 @@ import math
 
 import torch
 
+import cache_order
 from xeno_rt_amd.cache import BLOCK_TOKENS as BLOCK      # the cache's own constant: blocks are its unit
 
 
@@ -111,8 +112,8 @@ class EmulatedOps:
                 pos = int(positions[t])
                 block = int(table[slot, pos // BLOCK])
                 assert block >= 0, "write into a block that the sequence does not hold"
-                kv.k[block, :, pos % BLOCK, :] = qkv[t, qw:qw + kw].reshape(n_kv_heads, head_dim).to(kv.k.dtype)
-                kv.v[block, :, :, pos % BLOCK] = v[t].to(kv.v.dtype)
+                cache_order.write_key(kv.k, block, pos % BLOCK, qkv[t, qw:qw + kw].reshape(n_kv_heads, head_dim))
+                cache_order.write_value(kv.v, block, pos % BLOCK, v[t])
 
     def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None):
         tokens = qkv.shape[0]
@@ -130,8 +131,8 @@ class EmulatedOps:
             blocks = table[slot, (index // BLOCK).to(table.device)].long()
             assert int(blocks.min()) >= 0, "read from a block that the sequence does not hold"
             within = (index % BLOCK).to(blocks.device)
-            keys = kv.k[blocks, :, within, :].to(torch.float32)      # [n, kv_heads, dim]
-            values = kv.v[blocks, :, :, within].to(torch.float32)    # [n, kv_heads, dim]
+            keys = cache_order.read_keys(kv.k, blocks, within).to(torch.float32)        # [n, kv_heads, dim]
+            values = cache_order.read_values(kv.v, blocks, within).to(torch.float32)    # [n, kv_heads, dim]
             for head in range(n_heads):
                 kvh = head // group
                 scores = (keys[:, kvh, :] @ q[t, head]) * scale

@@ -9,6 +9,7 @@ from types import SimpleNamespace
 import pytest
 import torch
 
+import cache_order
 from ops_emulation import EmulatedOps
 import plain_llama as P
 
@@ -344,7 +345,7 @@ def test_qkv_prepare(ops, dtype, nh, nkv, hd, rope_dim):
         assert rel(got.float(), want.float()) < tol
         assert rel(kv_got.k.float(), kv_want.k.float()) < tol
         assert torch.equal(kv_got.v, kv_want.v)
-        assert int((kv_got.k != 0).any(-1).sum()) == 8 * nkv      # eight tokens cached, padding not
+        assert int((cache_order.plain_keys(kv_got.k) != 0).any(-1).sum()) == 8 * nkv      # eight tokens cached, padding not
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -373,7 +374,7 @@ def test_qkv_prepare_of_many_tokens(ops, dtype, nh, nkv, hd, rope_dim):
     assert rel(got.float(), want.float()) < tol
     assert rel(kv_got.k.float(), kv_want.k.float()) < tol
     assert torch.equal(kv_got.v, kv_want.v)
-    assert int((kv_got.k != 0).any(-1).sum()) == (tokens - 1) * nkv
+    assert int((cache_order.plain_keys(kv_got.k) != 0).any(-1).sum()) == (tokens - 1) * nkv
 
 
 @pytest.mark.parametrize("nh,nkv,hd,rope_dim,k,tokens", [(32, 8, 128, 128, 4096, 8), (4, 2, 64, 64, 200, 9), (3, 3, 48, 32, 96, 16),
@@ -420,7 +421,7 @@ def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens, packed)
         assert float((got.float() - want.float()).abs().gt(0).float().mean()) < 0.01
         assert rel(kv_got.k.float(), kv_want.k.float()) < ULP["bfloat16"]
         assert torch.equal(kv_got.v, kv_want.v)
-        assert int((kv_got.k != 0).any(-1).sum()) == int((slots >= 0).sum()) * nkv
+        assert int((cache_order.plain_keys(kv_got.k) != 0).any(-1).sum()) == int((slots >= 0).sum()) * nkv
     # without a cache to write (a layer that reads another layer's), and with head norms (two kernels then)
     got = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
     want = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
@@ -476,6 +477,7 @@ def filled_cache(nkv, hd, dtype, lengths, seed=0):
             block = int(kv.block_table[s, n // 64])
             kv.k[block, :, n % 64:, :] = float("nan")
             kv.v[block, :, :, n % 64:] = float("nan")
+    kv.k, kv.v = cache_order.store_keys(kv.k), cache_order.store_values(kv.v)     # from rows into the order the kernels keep
     return kv, keys, values
 
 

@@ -6,6 +6,7 @@ import subprocess
 import pytest
 import torch
 
+import cache_order
 import plain_llama as P
 from reference_cpp import CppReference
 
@@ -75,8 +76,8 @@ def test_preparation_and_attention_over_the_cache(ref, nh, nkv, hd, rope_dim, no
     close(got[:, nh * hd:(nh + nkv) * hd], kk, 1e-4)
     assert torch.equal(got[:, (nh + nkv) * hd:], vv)
     # the cache: token 70 lies in logical block 1 = physical block 0, place 6
-    close(k[0, :, 6, :].reshape(-1), kk[70], 1e-4)
-    assert torch.equal(v[0, :, :, 6].reshape(-1), vv[70])
+    close(cache_order.plain_keys(k)[0, :, 6, :].reshape(-1), kk[70], 1e-4)
+    assert torch.equal(cache_order.plain_values(v)[0, :, :, 6].reshape(-1), vv[70])
     out = ref.attention(got, nh, nkv, hd, k, v, table, positions, slots, 1.0 / math.sqrt(hd))
     close(out, P.causal_attention(q, kk, vv, nh, nkv, hd), 1e-4)
     # a window of 20: the plain attention over the 20 last keys of every query

@@ -7,16 +7,19 @@
 // by the sum); query head h uses key/value head h / group.
 //
 // One wavefront takes one chunk of keys of one (token, key/value head, tile of 16 query
-// heads). Scores: S[key][head] = K Q^T with v_mfma_f32_16x16x32_bf16, keys as rows (A operand,
-// read straight from the cache block, 16 bytes per lane), the query heads as columns. Values:
-// O[dim][head] += V^T P, with the transposed value block as A operand (again 16 contiguous
-// bytes per lane) and the probabilities, still in the registers the scores came in, as B
+// heads). Scores: S[key][head] = K Q^T with v_mfma_f32_16x16x32_bf16, keys as rows (A operand),
+// the query heads as columns. Values: O[dim][head] += V^T P, with the transposed value block
+// as A operand and the probabilities, still in the registers the scores came in, as B
 // operand: key rows are assigned to accumulator rows such that every lane ends up holding
-// eight consecutive keys, exactly the K slots of the next product. All loads of a cache block,
-// keys and values, are issued before anything is computed. The four wavefronts of a workgroup
+// eight consecutive keys, exactly the K slots of the next product. A cache block lies in
+// memory in the order of these operands (cache_layout.h): every load instruction takes one
+// contiguous kilobyte, which nobody else reads, and passes the caches by (non-temporal; with
+// keys as rows of head_dim elements an instruction took half a line of each of 16 keys and the
+// kernel read 6.1 TB/s where it now reads 6.9). A block's values are asked for before its
+// scores are computed, the next block's keys right after. The four wavefronts of a workgroup
 // merge their results (maximum, sum, O) through LDS into one partial result; a second kernel
 // merges the partial results of a token, in order.
-#include "common.h"
+#include "cache_layout.h"
 #include "xrt_hip.h"
 
 namespace {
@@ -27,9 +30,14 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 constexpr int WAVES = 4;
 constexpr float LOG2E = 1.4426950408889634f;
 
-// key (0..31 within a group of 32) that row r of score tile `tile` (0 or 1) stands for:
-// accumulator register i of lane group c is row c*4 + i, and must be key c*8 + tile*4 + i
-__device__ __forceinline__ int key_of_row(int tile, int r) { return (r / 4) * 8 + tile * 4 + (r % 4); }
+// Row r of score tile t (0 or 1) of a group of 32 keys stands for key 8 (r / 4) + 4 t + r % 4: accumulator
+// register i of lane group c is row 4 c + i, and must be key 8 c + 4 t + i. The cache keeps the keys so:
+// lane (r, c) finds its piece of tile ((g * 2 + t) * KS + s) at place r + 16 c, and of the values' tile
+// (g * DT + u) likewise.
+constexpr int lane_place(int r, int c) { return (r + 16 * c) * 8; }
+static_assert(cache_key_offset(32 + 8 * 2 + 4 * 1 + 3, 32 * 3 + 8 * 1, 128) == ((1 * 2 + 1) * 4 + 3) * 512 + lane_place(2 * 4 + 3, 1), "keys of a block");
+static_assert(cache_key_offset(8 * 3 + 4 * 0 + 1, 32 * 1 + 8 * 3 + 5, 64) == ((0 * 2 + 0) * 2 + 1) * 512 + lane_place(3 * 4 + 1, 3) + 5, "keys of a block");
+static_assert(cache_value_offset(16 * 5 + 9, 32 + 8 * 2 + 6, 128) == (1 * 8 + 5) * 512 + lane_place(9, 2) + 6, "values of a block");
 
 template <int HD>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) attention_decode_kernel(
@@ -93,7 +101,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) attention_decode_kernel(
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
-                        kreg[g][t][ks] = *reinterpret_cast<const bf16x8*>(kb + (long)(g * 32 + key_of_row(t, r)) * HD + c * 8 + ks * 32);
+                        kreg[g][t][ks] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(kb + ((g * 2 + t) * KS + ks) * 512 + lane * 8));
         };
         int block = block_of(first_block), next_block = block_of(first_block + 1);
         ask_keys(block);
@@ -104,7 +112,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) attention_decode_kernel(
             for (int g = 0; g < 2; ++g)
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
-                    vreg[g][dt] = *reinterpret_cast<const bf16x8*>(vb + (long)(dt * 16 + r) * XRT_BLOCK_TOKENS + g * 32 + c * 8);
+                    vreg[g][dt] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(vb + (g * DT + dt) * 512 + lane * 8));
 
             // ---- scores of 64 keys: two groups of 32, two tiles of 16 rows each
             floatx4 s[2][2];

@@ -13,7 +13,7 @@
 // A position encoding that acts on the scores instead of on q and k is served here too: with
 // distance_slopes (one float per query head) a key at position j adds slope * (j - P) to the
 // score of the query at position P, after the scale. Not in the reference's model.
-#include "common.h"
+#include "cache_layout.h"
 #include "xrt_hip.h"
 
 namespace {
@@ -57,9 +57,12 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
         const long head_base = ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * head_dim;
         float s = -INFINITY;
         if (valid) {
-            const T* key = k_cache + head_base + (long)lane * head_dim;
             float dot = 0.f;
-            for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(key[d]), dot);
+            for (int d0 = 0; d0 < head_dim; d0 += 8) {          // the key's dims in order, piece by piece of the cache's order
+                const T* piece = k_cache + head_base + cache_key_offset(lane, d0, head_dim);
+                const int dims = min(8, head_dim - d0);
+                for (int e = 0; e < dims; ++e) dot = fmaf(qs[d0 + e], to_float(piece[e]), dot);
+            }
             s = dot * scale;
             if (distance_slopes) s += slope * (float)(j - pos);
         }
@@ -76,9 +79,11 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
         for (int i = 0; i < MAX_OWNED; ++i) {
             const int d = lane + i * XRT_WAVE;
             if (d < head_dim) {
-                const T* value = v_cache + head_base + (long)d * XRT_BLOCK_TOKENS;
                 float sum = 0.f;
-                for (int jj = j_begin; jj <= j_end; ++jj) sum = fmaf(ps[jj], to_float(value[jj]), sum);
+                for (int j0 = j_begin / 8 * 8; j0 <= j_end; j0 += 8) {   // the dim's values in the order of their tokens
+                    const T* piece = v_cache + head_base + cache_value_offset(d, j0, head_dim);
+                    for (int jj = max(j0, j_begin); jj <= min(j0 + 7, j_end); ++jj) sum = fmaf(ps[jj], to_float(piece[jj - j0]), sum);
+                }
                 acc[i] = acc[i] * correction + sum;
             }
         }

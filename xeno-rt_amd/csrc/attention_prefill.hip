@@ -11,7 +11,7 @@
 // multiplies) has two tiles of 128 query tokens of one sequence and one head, a late and an
 // early one, and 32 queries per wavefront; how the two tiles share the wavefronts is told at
 // the kernel. The workgroup walks the sequence's cache blocks (64 keys) in order; every block
-// travels once from global memory into LDS (keys as they lie, values transposed as they lie),
+// travels once from global memory into LDS (keys in rows, values transposed),
 // the next blocks while the current ones are used, and all wavefronts read their operands
 // from there. Everything is kept transposed so that one lane owns one query:
 // S^T[key][query] = K Q^T and O^T[dim][query] += V^T P^T with v_mfma_f32_32x32x16_bf16.
@@ -20,7 +20,7 @@
 // product wants as its B operand: key rows are assigned to accumulator rows such that a lane
 // holds eight consecutive keys per K step, which are also 16 contiguous bytes of the
 // transposed value block.
-#include "common.h"
+#include "cache_layout.h"
 #include "xrt_hip.h"
 
 namespace {
@@ -147,16 +147,18 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     take(helper && has_early ? early_tile : late_tile);
     bool on_early = helper && has_early;
 
-    // ---- moving a cache block into LDS: both parts are contiguous in global memory, and go
-    // straight there (global_load_lds_dwordx4): lane l of an instruction fills the l-th 16 bytes
-    // of a 1024-byte stretch with the chunk that belongs in that place
-    // A wavefront's further loads of a block lie WAVES * 1024 bytes on, in global memory as in LDS: that many bytes are
-    // a multiple of 16 key rows and of 16 value rows, which the swizzles repeat after.
-    static_assert(WAVES * 1024 % (16 * K_CHUNKS * 16) == 0 && WAVES * 1024 % (16 * V_CHUNKS * 16) == 0, "swizzles do not repeat");
-    const int place = wave * XRT_WAVE + lane;                // 16-byte place within the block's LDS image, of the first load
-    const int k_row = place / K_CHUNKS, v_row = place / V_CHUNKS;
-    const unsigned k_from = (unsigned)((k_row * K_CHUNKS + ((place % K_CHUNKS) ^ k_swizzle(k_row))) * 16);   // byte offsets of this lane's chunks within a block
-    const unsigned v_from = (unsigned)((v_row * V_CHUNKS + ((place % V_CHUNKS) ^ v_swizzle(v_row))) * 16);
+    // ---- moving a cache block into LDS: it goes straight there (global_load_lds_dwordx4): lane l of an
+    // instruction fills the l-th 16 bytes of a 1024-byte stretch with the chunk that belongs in that place,
+    // 8 dims of a key or 8 tokens of a value dim, which lie together in the cache block too (cache_layout.h:
+    // the block itself is in the order of the decode kernel's operands, not in rows)
+    unsigned k_from[LOADS], v_from[LOADS];                   // byte offsets of this lane's chunks within a block
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int place = (i * WAVES + wave) * XRT_WAVE + lane;      // 16-byte place within the block's LDS image
+        const int k_row = place / K_CHUNKS, v_row = place / V_CHUNKS;
+        k_from[i] = (unsigned)cache_key_offset(k_row, ((place % K_CHUNKS) ^ k_swizzle(k_row)) * 8, HD) * 2u;
+        v_from[i] = (unsigned)cache_value_offset(v_row, ((place % V_CHUNKS) ^ v_swizzle(v_row)) * 8, HD) * 2u;
+    }
     const unsigned lds_k0 = lds_address(lds_raw), lds_v0 = lds_k0 + 2 * PER_STAGE * BT * HD * (unsigned)sizeof(bf16);
     // The table's entries are read a stage before they are used: read where they are used, every stage would begin
     // with the wait for a scalar load.
@@ -169,8 +171,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
             const unsigned at = (unsigned)((buffer * BT * HD) * 2 + (i * WAVES + wave_uniform) * 1024);
-            load_to_lds(kb + i * WAVES * 1024, k_from, lds_k0 + at);
-            load_to_lds(vb + i * WAVES * 1024, v_from, lds_v0 + at);
+            load_to_lds(kb, k_from[i], lds_k0 + at);
+            load_to_lds(vb, v_from[i], lds_v0 + at);
         }
     };
 

@@ -825,11 +825,11 @@ __global__ void __launch_bounds__(256) split_reduce_qkv_kernel(const float* __re
     if (base < 0) return;
     const int within = pos % XRT_BLOCK_TOKENS;
     if (is_v) {
-        after.v_cache[base + (long)d * XRT_BLOCK_TOKENS + within] = out_lower;
-        after.v_cache[base + (long)(d + half) * XRT_BLOCK_TOKENS + within] = out_upper;
+        after.v_cache[base + cache_value_offset(d, within, after.head_dim)] = out_lower;
+        after.v_cache[base + cache_value_offset(d + half, within, after.head_dim)] = out_upper;
     } else {
-        after.k_cache[base + (long)within * after.head_dim + d] = out_lower;
-        after.k_cache[base + (long)within * after.head_dim + d + half] = out_upper;
+        after.k_cache[base + cache_key_offset(within, d, after.head_dim)] = out_lower;
+        after.k_cache[base + cache_key_offset(within, d + half, after.head_dim)] = out_upper;
     }
 }
 

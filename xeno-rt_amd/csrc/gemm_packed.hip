@@ -301,11 +301,11 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
                 if (base >= 0) {
                     const int within = early_within[r];
                     if (head < after.n_heads + after.n_kv_heads) {
-                        *reinterpret_cast<Four*>(after.k_cache + base + (long)within * after.head_dim + dim) = packed;
+                        *reinterpret_cast<Four*>(after.k_cache + base + cache_key_offset(within, dim, after.head_dim)) = packed;
                     } else {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            after.v_cache[base + (long)(dim + i) * XRT_BLOCK_TOKENS + within] = packed.e[i];
+                            after.v_cache[base + cache_value_offset(dim + i, within, after.head_dim)] = packed.e[i];
                     }
                 }
             }

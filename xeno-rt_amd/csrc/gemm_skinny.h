@@ -1,6 +1,6 @@
 // The product for few rows (gemm_skinny.hip), as the entry points of the products see it.
 #pragma once
-#include "common.h"
+#include "cache_layout.h"
 #include "xrt_hip.h"
 
 // What follows the q/k/v projection of a decode step, done by the product's own epilogue: rotation

@@ -13,11 +13,12 @@
 // head is read and written in 16-byte pieces and the norm's sum is a few lane exchanges. When a
 // step brings many tokens, the values go to their transposed cache blocks through a kernel of
 // their own, which turns tiles of 64 tokens in LDS so that writes to the cache are whole lines.
+// Where a key or a value lies inside its block: cache_layout.h.
 // The general kernel (one wavefront per (token, head), any even head size and rotation width)
 // takes the rest. A token with a negative slot is padding and is not cached. Per head, all
 // kernels use the same formulas in the same order; only the order of the norm's sum differs,
 // and which kernel a model takes depends on its sizes alone, never on the step.
-#include "common.h"
+#include "cache_layout.h"
 #include "xrt_hip.h"
 
 namespace {
@@ -60,7 +61,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) qkv_prepare_kernel(
     if (is_v) {
         if (cache_base >= 0)
             for (int e = lane; e < head_dim; e += XRT_WAVE)
-                v_cache[cache_base + (long)e * XRT_BLOCK_TOKENS + within] = row[e];
+                v_cache[cache_base + cache_value_offset(e, within, head_dim)] = row[e];
         return;
     }
 
@@ -92,7 +93,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) qkv_prepare_kernel(
     for (int e = lane; e < head_dim; e += XRT_WAVE) {
         const T value = from_float<T>(x[e]);
         row[e] = value;
-        if (is_k && cache_base >= 0) k_cache[cache_base + (long)within * head_dim + e] = value;
+        if (is_k && cache_base >= 0) k_cache[cache_base + cache_key_offset(within, e, head_dim)] = value;
     }
 }
 
@@ -143,8 +144,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) qkv_prepare_vector_kernel(
             if (cache_base >= 0) {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    v_cache[cache_base + (long)(at + e) * XRT_BLOCK_TOKENS + within] = lower.e[e];
-                    v_cache[cache_base + (long)(HALF + at + e) * XRT_BLOCK_TOKENS + within] = upper.e[e];
+                    v_cache[cache_base + cache_value_offset(at + e, within, HEAD)] = lower.e[e];
+                    v_cache[cache_base + cache_value_offset(HALF + at + e, within, HEAD)] = upper.e[e];
                 }
             }
             continue;
@@ -181,17 +182,18 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) qkv_prepare_vector_kernel(
         *reinterpret_cast<Pack<T, VEC>*>(row + at) = out_lower;
         *reinterpret_cast<Pack<T, VEC>*>(row + HALF + at) = out_upper;
         if (is_k && cache_base >= 0) {
-            T* dst = k_cache + cache_base + (long)within * HEAD;
-            *reinterpret_cast<Pack<T, VEC>*>(dst + at) = out_lower;
-            *reinterpret_cast<Pack<T, VEC>*>(dst + HALF + at) = out_upper;
+            T* dst = k_cache + cache_base;                  // (16 bytes from a multiple of 16 bytes stay together in the cache's order)
+            *reinterpret_cast<Pack<T, VEC>*>(dst + cache_key_offset(within, at, HEAD)) = out_lower;
+            *reinterpret_cast<Pack<T, VEC>*>(dst + cache_key_offset(within, HALF + at, HEAD)) = out_upper;
         }
     }
 }
 
 // Values of 64 consecutive tokens of a step and one key/value head: read row by row, turned in
-// LDS, and written with one lane per token, so that tokens that follow each other in a sequence
-// fill a line of the transposed cache block together. Tokens of different sequences or blocks
-// may share a tile: every lane finds its own block.
+// LDS, and written so that a store instruction of a wavefront takes 8 tokens of 8 dims: where the
+// tokens follow each other in a sequence these are the eight pieces of one line of the cache block
+// (cache_layout.h). Tokens of different sequences or blocks may share a tile: every token has its
+// own block.
 constexpr int TILE_DIMS = 128;
 template <typename T>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE) value_cache_write_kernel(
@@ -199,16 +201,22 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) value_cache_write_kernel(
     const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ v_cache,
     const int* __restrict__ block_table, int table_stride, int n_blocks) {
     __shared__ T tile[XRT_WAVE][TILE_DIMS + 4 / (int)sizeof(T)];      // rows end one bank further each
+    __shared__ long bases[XRT_WAVE];                                  // of the tile's tokens: their block (-1: none) ...
+    __shared__ int withins[XRT_WAVE];                                 // ... and their place in it
     const int wave = threadIdx.x / XRT_WAVE, lane = threadIdx.x % XRT_WAVE;
     const int first = blockIdx.x * XRT_WAVE, kv_head = blockIdx.y;
     const int heads_total = n_heads + 2 * n_kv_heads;
-    const int token = first + lane;
-    long cache_base = -1;
-    int within = 0;
-    if (token < tokens) {
-        const int pos = positions[token];
-        cache_base = cache_block_base(block_table, table_stride, n_blocks, slots[token], pos, n_kv_heads, kv_head, head_dim);
-        within = pos % XRT_BLOCK_TOKENS;
+    if (wave == 0) {
+        const int token = first + lane;
+        long cache_base = -1;
+        int within = 0;
+        if (token < tokens) {
+            const int pos = positions[token];
+            cache_base = cache_block_base(block_table, table_stride, n_blocks, slots[token], pos, n_kv_heads, kv_head, head_dim);
+            within = pos % XRT_BLOCK_TOKENS;
+        }
+        bases[lane] = cache_base;
+        withins[lane] = within;
     }
     const T* source = qkv + (long)(n_heads + n_kv_heads + kv_head) * head_dim;
     constexpr int VEC = 16 / (int)sizeof(T);                  // the launcher sends only head sizes that are multiples of this
@@ -223,9 +231,14 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) value_cache_write_kernel(
             for (int e = 0; e < VEC; ++e) tile[r][d + e] = piece.e[e];
         }
         __syncthreads();
-        if (cache_base >= 0)
-            for (int d = wave; d < dims; d += WAVES)
-                v_cache[cache_base + (long)(d0 + d) * XRT_BLOCK_TOKENS + within] = tile[lane][d];
+        // a step of a wavefront: tokens 8 g .. 8 g + 7 of the tile (lane % 8), dims 8 h .. 8 h + 7 (lane / 8)
+        const int steps = (dims + 7) / 8 * 8;
+        for (int step = wave; step < steps; step += WAVES) {
+            const int token = step % 8 * 8 + lane % 8, d = step / 8 * 8 + lane / 8;
+            const long cache_base = bases[token];
+            if (cache_base >= 0 && d < dims)
+                v_cache[cache_base + cache_value_offset(d0 + d, withins[token], head_dim)] = tile[token][d];
+        }
         __syncthreads();
     }
 }

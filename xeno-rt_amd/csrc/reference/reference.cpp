@@ -22,7 +22,39 @@
 
 namespace {
 
-constexpr int BLOCK = 64;           // tokens of a cache block: keys [kv_head][token][dim], values [kv_head][dim][token]
+constexpr int BLOCK = 64;           // tokens of a cache block
+
+// Where the elements of a cache block lie. Head sizes that are no multiple of 32: keys [token][dim], values
+// [dim][token]. Multiples of 32: in the order in which a wavefront of the decode kernel holds the block, found here by
+// walking that order: tiles of 64 lanes' pieces of 8 elements, lane (r, c) at place r + 16 c.
+//   keys:   for each half g of the block, each score tile t of it, each 32 dims s: lane (r, c) has dims
+//           32 s + 8 c .. + 7 of key 32 g + 8 (r / 4) + 4 t + r % 4;
+//   values: for each half g, each 16 dims u: lane (r, c) has tokens 32 g + 8 c .. + 7 of dim 16 u + r.
+struct BlockOrder {
+    std::vector<int> key, value;     // [token * head_dim + dim], [dim * BLOCK + token] -> element offset in the block
+    explicit BlockOrder(int head_dim) : key((size_t)BLOCK * head_dim), value((size_t)BLOCK * head_dim) {
+        if (head_dim % 32 != 0) {
+            std::iota(key.begin(), key.end(), 0);
+            std::iota(value.begin(), value.end(), 0);
+            return;
+        }
+        int at = 0;
+        for (int g = 0; g < 2; ++g)
+            for (int t = 0; t < 2; ++t)
+                for (int s = 0; s < head_dim / 32; ++s)
+                    for (int c = 0; c < 4; ++c)
+                        for (int r = 0; r < 16; ++r)
+                            for (int e = 0; e < 8; ++e)
+                                key[(size_t)(32 * g + 8 * (r / 4) + 4 * t + r % 4) * head_dim + 32 * s + 8 * c + e] = at++;
+        at = 0;
+        for (int g = 0; g < 2; ++g)
+            for (int u = 0; u < head_dim / 16; ++u)
+                for (int c = 0; c < 4; ++c)
+                    for (int r = 0; r < 16; ++r)
+                        for (int e = 0; e < 8; ++e)
+                            value[(size_t)(16 * u + r) * BLOCK + 32 * g + 8 * c + e] = at++;
+    }
+};
 
 float activation(float z, int code) {
     (void)code;                      // XRT_ACT_SILU is the only one
@@ -34,6 +66,9 @@ float activation(float z, int code) {
 extern "C" {
 
 int xrt_ref_block_tokens(void) { return BLOCK; }
+
+int xrt_ref_cache_key_offset(int token, int dim, int head_dim) { return BlockOrder(head_dim).key[(size_t)token * head_dim + dim]; }
+int xrt_ref_cache_value_offset(int dim, int token, int head_dim) { return BlockOrder(head_dim).value[(size_t)dim * BLOCK + token]; }
 
 void xrt_ref_embed(const float* table, const int* ids, float* out, int tokens, int hidden) {
     for (int t = 0; t < tokens; ++t)
@@ -98,14 +133,15 @@ void xrt_ref_qkv_prepare(float* qkv, int tokens, int n_heads, int n_kv_heads, in
             }
         }
         if (!k_cache || slots[t] < 0) continue;
+        const BlockOrder order(head_dim);
         const int block = block_table[(long)slots[t] * table_stride + positions[t] / BLOCK];
         if (block < 0 || block >= n_blocks) continue;
         const int within = positions[t] % BLOCK;
         for (int kv = 0; kv < n_kv_heads; ++kv)
             for (int d = 0; d < head_dim; ++d) {
                 const long base = ((long)block * n_kv_heads + kv) * BLOCK * head_dim;
-                k_cache[base + (long)within * head_dim + d] = row[(long)(n_heads + kv) * head_dim + d];
-                v_cache[base + (long)d * BLOCK + within] = row[(long)(n_heads + n_kv_heads + kv) * head_dim + d];
+                k_cache[base + order.key[(size_t)within * head_dim + d]] = row[(long)(n_heads + kv) * head_dim + d];
+                v_cache[base + order.value[(size_t)d * BLOCK + within]] = row[(long)(n_heads + n_kv_heads + kv) * head_dim + d];
             }
     }
 }
@@ -114,6 +150,7 @@ void xrt_ref_attention(const float* qkv, int tokens, int n_heads, int n_kv_heads
                        const float* v_cache, const int* block_table, int table_stride, const int* positions,
                        const int* slots, float* out, float scale, int window, const float* distance_slopes) {
     const int width = (n_heads + 2 * n_kv_heads) * head_dim, group = n_heads / n_kv_heads;
+    const BlockOrder order(head_dim);
     for (int t = 0; t < tokens; ++t)
         for (int head = 0; head < n_heads; ++head) {
             float* dst = out + ((long)t * n_heads + head) * head_dim;
@@ -125,9 +162,10 @@ void xrt_ref_attention(const float* qkv, int tokens, int n_heads, int n_kv_heads
             std::vector<float> scores(pos + 1 - first);
             for (int key = first; key <= pos; ++key) {
                 const int block = block_table[(long)slots[t] * table_stride + key / BLOCK];
-                const float* k = k_cache + (((long)block * n_kv_heads + kv) * BLOCK + key % BLOCK) * head_dim;
+                const float* k = k_cache + ((long)block * n_kv_heads + kv) * BLOCK * head_dim;
+                const int* place = &order.key[(size_t)(key % BLOCK) * head_dim];
                 float dot = 0.f;
-                for (int d = 0; d < head_dim; ++d) dot += q[d] * k[d];
+                for (int d = 0; d < head_dim; ++d) dot += q[d] * k[place[d]];
                 scores[key - first] = dot * scale + (distance_slopes ? distance_slopes[head] * (float)(key - pos) : 0.f);
             }
             const float largest = *std::max_element(scores.begin(), scores.end());
@@ -135,9 +173,9 @@ void xrt_ref_attention(const float* qkv, int tokens, int n_heads, int n_kv_heads
             for (float& s : scores) { s = std::exp(s - largest); total += s; }
             for (int key = first; key <= pos; ++key) {
                 const int block = block_table[(long)slots[t] * table_stride + key / BLOCK];
-                const float* v = v_cache + ((long)block * n_kv_heads + kv) * head_dim * BLOCK + key % BLOCK;
+                const float* v = v_cache + ((long)block * n_kv_heads + kv) * head_dim * BLOCK;
                 const float p = scores[key - first] / total;
-                for (int d = 0; d < head_dim; ++d) dst[d] += p * v[(long)d * BLOCK];
+                for (int d = 0; d < head_dim; ++d) dst[d] += p * v[order.value[(size_t)d * BLOCK + key % BLOCK]];
             }
         }
 }

@@ -7,6 +7,9 @@ extern "C" {
 #endif
 
 int xrt_ref_block_tokens(void);
+// element offset of (token, dim) of a key, and of (dim, token) of a value, within the cache block of one key/value head
+int xrt_ref_cache_key_offset(int token, int dim, int head_dim);
+int xrt_ref_cache_value_offset(int dim, int token, int head_dim);
 void xrt_ref_embed(const float* table, const int* ids, float* out, int tokens, int hidden);
 void xrt_ref_add(float* residual, const float* delta, long count);
 void xrt_ref_rmsnorm(const float* x, const float* weight, float eps, float* out, const int* rows, int n_rows, int hidden);

@@ -61,6 +61,11 @@ int main() {
         const float* q1 = &before[width], *r1 = &qkv[width];    // position 1, first pair of the first head: angle 1
         check(close_to(r1[0], q1[0] * std::cos(1.0f) - q1[2] * std::sin(1.0f)) && close_to(r1[2], q1[0] * std::sin(1.0f) + q1[2] * std::cos(1.0f)), "rotation pairs (i, i + d/2)");
         check(k_cache[1 * hd + 0] == qkv[width + nh * hd] && v_cache[0 * 64 + 1] == before[width + (nh + nkv) * hd], "cache holds rotated keys and raw values");
+        // heads of a multiple of 32: the order of the decode kernel's operands. Worked out by hand: key 13 is row 5 of
+        // score tile 1 of the first half, dims 16 .. 23 are lane group 2 of the first 32: tile (0 * 2 + 1) * 2 + 0,
+        // place 5 + 32; dim 21 of the value of token 45: tile 1 * 4 + 1, row 5, tokens 40 .. 47 are lane group 1
+        check(xrt_ref_cache_key_offset(13, 21, 64) == (2 * 64 + 37) * 8 + 5 && xrt_ref_cache_value_offset(21, 45, 64) == (5 * 64 + 5 + 16) * 8 + 5 &&
+              xrt_ref_cache_key_offset(13, 21, 48) == 13 * 48 + 21 && xrt_ref_cache_value_offset(21, 45, 48) == 21 * 64 + 45, "order of a cache block");
         std::vector<float> out(tokens * nh * hd);
         xrt_ref_attention(qkv.data(), tokens, nh, nkv, hd, k_cache.data(), v_cache.data(), table, 1, positions, slots, out.data(), 0.5f, 0, nullptr);
         bool first_is_value = true;                             // one key: the output is its value

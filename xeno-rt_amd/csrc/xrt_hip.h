@@ -9,9 +9,15 @@ extern "C" {
 
 const char* xrt_last_error(void);
 
-// tokens in one block of the cache: keys [kv_head][token][dim], values [kv_head][dim][token] inside a block.
-// Whoever keeps the block tables must count in the same blocks.
+// tokens in one block of the cache. A cache is [blocks][kv_heads][xrt_block_tokens() * head_dim elements], keys and
+// values apart. Whoever keeps the block tables must count in the same blocks.
 int xrt_block_tokens(void);
+// Where the elements lie inside the part of a block that belongs to one key/value head: the element offset of dim
+// `dim` of the key (of the value) of the block's token `token`. Heads whose size is a multiple of 32 lie in the order
+// in which the matrix cores take them in a decode step (csrc/cache_layout.h); others as keys [token][dim], values
+// [dim][token]. Host functions, for whoever wants to fill or read a cache outside the kernels.
+int xrt_cache_key_offset(int token, int dim, int head_dim);
+int xrt_cache_value_offset(int dim, int token, int head_dim);
 
 // How a bfloat16 weight matrix w[rows][K] is laid out. XRT_PACK_NONE (or a null pointer wherever a packing
 // is passed): rows contiguous along k. Otherwise tiles of 16 rows x 32 columns in the order in which the matrix
