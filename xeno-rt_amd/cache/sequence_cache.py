@@ -6,9 +6,11 @@ value rows have the same shape and window form a group; a group has storage of
 its own (one pool of blocks, one block table) and its own rule for which blocks
 a sequence of a given length holds: all of them, or those a window still sees.
 Storage of one call: keys [blocks, kv_heads, BLOCK_TOKENS, head_dim], values
-[blocks, kv_heads, value_dim, BLOCK_TOKENS] (values transposed inside a block, so
-that the keys of one block are contiguous along head_dim and the values along
-tokens, which is how the attention kernels read them).
+[blocks, kv_heads, value_dim, BLOCK_TOKENS]. The order of the BLOCK_TOKENS * head_dim
+elements behind the last two dimensions belongs to the kernels that write and read
+them (csrc/cache_layout.h: for head sizes that are multiples of 32, the order in
+which the decode attention's wavefronts load them; rows otherwise); nothing in
+the package looks inside a block.
 
 The reference keeps one paged cache per sequence with rows of all KV heads,
 float32 (crates/xrt-runtime/src/kv_cache.rs:4-45); `truncate` follows its
@@ -32,8 +34,8 @@ from .allocator import BLOCK_TOKENS, CacheError, CacheFull, Pool, blocks_for
 class KVView:
     """What an attention kernel needs of one layer call's keys and values."""
     spec: KVSpec
-    k: torch.Tensor             # [blocks, kv_heads, BLOCK_TOKENS, head_dim]
-    v: torch.Tensor             # [blocks, kv_heads, value_dim, BLOCK_TOKENS]
+    k: torch.Tensor             # [blocks, kv_heads, BLOCK_TOKENS, head_dim]: per (block, head) the kernels' own order
+    v: torch.Tensor             # [blocks, kv_heads, value_dim, BLOCK_TOKENS]: likewise
     block_table: torch.Tensor   # int32 [slots, max_blocks]: logical block -> physical block, -1 = none
 
 
