@@ -200,7 +200,9 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) value_cache_write_kernel(
     const T* __restrict__ qkv, int tokens, int n_heads, int n_kv_heads, int head_dim,
     const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ v_cache,
     const int* __restrict__ block_table, int table_stride, int n_blocks) {
-    __shared__ T tile[XRT_WAVE][TILE_DIMS + 4 / (int)sizeof(T)];      // rows end one bank further each
+    // A store step reads 8 tokens (rows) x 8 dims: with rows 8 elements longer than a multiple of 256 bytes the 8 rows
+    // start 4 (bfloat16) or 8 (float32) banks apart, and the step's 32 or 64 words lie in as many banks.
+    __shared__ __attribute__((aligned(16))) T tile[XRT_WAVE][TILE_DIMS + 8];
     __shared__ long bases[XRT_WAVE];                                  // of the tile's tokens: their block (-1: none) ...
     __shared__ int withins[XRT_WAVE];                                 // ... and their place in it
     const int wave = threadIdx.x / XRT_WAVE, lane = threadIdx.x % XRT_WAVE;
@@ -226,18 +228,19 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) value_cache_write_kernel(
         for (int i = threadIdx.x; i < XRT_WAVE * pieces; i += WAVES * XRT_WAVE) {
             const int r = i / pieces, d = (i % pieces) * VEC;
             const long from = min(first + r, tokens - 1);     // rows past the end repeat the last one; nobody writes them
-            const Pack<T, VEC> piece = *reinterpret_cast<const Pack<T, VEC>*>(source + from * heads_total * head_dim + d0 + d);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) tile[r][d + e] = piece.e[e];
+            *reinterpret_cast<Pack<T, VEC>*>(&tile[r][d]) = *reinterpret_cast<const Pack<T, VEC>*>(source + from * heads_total * head_dim + d0 + d);
         }
         __syncthreads();
-        // a step of a wavefront: tokens 8 g .. 8 g + 7 of the tile (lane % 8), dims 8 h .. 8 h + 7 (lane / 8)
-        const int steps = (dims + 7) / 8 * 8;
-        for (int step = wave; step < steps; step += WAVES) {
-            const int token = step % 8 * 8 + lane % 8, d = step / 8 * 8 + lane / 8;
+        // a store of a wavefront: tokens 8 g .. 8 g + 7 of the tile (lane % 8), dims 8 h .. 8 h + 7 (lane / 8);
+        // a wavefront keeps its tokens while it walks the dims
+        for (int g = wave; g < XRT_WAVE / 8; g += WAVES) {
+            const int token = g * 8 + lane % 8;
             const long cache_base = bases[token];
-            if (cache_base >= 0 && d < dims)
-                v_cache[cache_base + cache_value_offset(d0 + d, withins[token], head_dim)] = tile[token][d];
+            const int within = withins[token];
+            if (cache_base < 0) continue;
+#pragma unroll 4
+            for (int d = lane / 8; d < dims; d += 8)
+                v_cache[cache_base + cache_value_offset(d0 + d, within, head_dim)] = tile[token][d];
         }
         __syncthreads();
     }
