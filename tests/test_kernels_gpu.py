@@ -93,7 +93,8 @@ SHAPES = [(1, 64, 64), (3, 200, 96), (8, 1000, 176), (17, 96, 192), (64, 333, 52
           (300, 520, 1032), (1, 3, 5), (5, 7, 13), (33, 4100, 264), (64, 40, 4096), (65, 40, 4096),
           (2048, 6144, 128), (2000, 6200, 136), (70, 300, 64), (300, 520, 1024), (2100, 6100, 320),
           (2100, 8300, 128), (40, 4100, 1024), (64, 333, 640), (33, 130, 128), (17, 700, 192),
-          (600, 520, 8192), (520, 1030, 8320)]         # the last two: many rows, few columns, a very long k (large tiles that split k)
+          (600, 520, 8192), (520, 1030, 8320),         # many rows, few columns, a very long k (large tiles that split k)
+          (12, 8200, 288), (9, 8208, 1056), (16, 16400, 4096), (16, 8192, 4128)]   # 9 to 16 rows, many rows of w, k up to 4096: x stays in registers (the last: k too long for that)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16 packed"])
@@ -122,7 +123,9 @@ def test_linear(ops, dtype, m, n, k):
                                    (2048, 3100, 64), (300, 130, 1032), (2048, 3072, 128), (2000, 3000, 192), (2048, 4224, 64),
                                    (64, 520, 256), (50, 1000, 1024), (200, 1000, 512),
                                    # 17 to 64 rows and tiles enough without a split along k
-                                   (40, 14336, 256), (64, 9002, 128), (33, 20000, 192)])
+                                   (40, 14336, 256), (64, 9002, 128), (33, 20000, 192),
+                                   # 9 to 16 rows and many pairs: x stays in the registers of a workgroup that walks the rows of w
+                                   (13, 4104, 96), (16, 14336, 4096), (9, 8192, 2080)])
 def test_linear_glu(ops, dtype, m, n, k):
     dtype, packed = dtype.split()[0], dtype.endswith("packed")
     if packed and n % 8 != 0:
@@ -176,7 +179,7 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
 
 
 @pytest.mark.parametrize("m,hidden,k,n", [(1, 4096, 512, 1024), (8, 4096, 14336, 6144), (16, 200, 96, 72),
-                                          (5, 1000, 136, 333), (13, 8200, 64, 48),
+                                          (5, 1000, 136, 333), (13, 8200, 64, 48), (13, 4096, 64, 4104), (16, 1056, 96, 8200),
                                           (17, 4096, 512, 1024), (40, 1024, 256, 333), (64, 4096, 14336, 6144), (33, 512, 128, 20000)])
 @pytest.mark.parametrize("packed", [False, True])
 def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n, packed):

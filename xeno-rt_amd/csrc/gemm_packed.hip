@@ -371,6 +371,125 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
     }
 }
 
+
+// The same product where a workgroup has several groups of 16 packed rows to do and k is so short that a wavefront's
+// eighth of x fits its registers (RESIDENT tiles of 32 columns: k up to 4096): the workgroup walks its groups, x is
+// read once, and only w streams, its ring of tiles running on from one group into the next. With 9 to 16 rows of x
+// the kernel above reads as many bytes of x from L2 as of w from memory, for every group again (gate/up of 14336 pairs
+// at 16 rows: 49 us; this way 41 us; a vocabulary of 128256 rows 212 against 168 us); with 8 rows or fewer, half of
+// x's rows are repeats and it gains nothing. Store and gated epilogues, rows of x with or without their RMSNorm's division.
+constexpr int RESIDENT = 16;       // tiles of x that a wavefront keeps
+constexpr int RING = 4;            // tiles of w on their way per wavefront
+static_assert(RESIDENT % RING == 0, "the ring of w tiles runs on from group to group");
+
+template <int MODE, typename TO>
+__global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) gemm_packed_resident_kernel(
+    const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
+    const Packing packing, const LinearNorm norm, int activation) {
+    static_assert(MODE == MODE_STORE || MODE == MODE_GATED, "store or gated");
+    __shared__ floatx4 partial[2][WAVES][XRT_WAVE];
+    __shared__ float square_parts[WAVES * XRT_WAVE / 16][16];
+    __shared__ float inv_rms[16];
+    const int lane = threadIdx.x % XRT_WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / XRT_WAVE);
+    const int r = lane % 16, c = lane / 16;
+    const int k_tiles = K / 32;
+    const int per_wave = (k_tiles + WAVES - 1) / WAVES;
+    const int first_tile = wave * per_wave;
+    const int count = max(0, min(per_wave, k_tiles - first_tile));      // at most RESIDENT: the launcher checks
+    const long rows_w = MODE == MODE_GATED ? 2L * N : N;
+    const long groups = (rows_w + 15) / 16;
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    bf16x8 x_tiles[RESIDENT], ring[RING];
+    const bf16* x_ptr = x + (long)min(r, M - 1) * K + first_tile * 32 + c * 8;      // rows beyond M: the last row again
+    auto w_of = [&](long group) { return w + (group * k_tiles + first_tile) * 512 + lane * 8; };
+    auto ask = [&](const bf16* from, int tile, bool there) {
+        return (there && tile < count) ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(from + (long)tile * 512)) : zero;
+    };
+    {
+        const bf16* first = w_of(blockIdx.x);                  // the grid has no more workgroups than w has groups
+#pragma unroll
+        for (int t = 0; t < RING; ++t) ring[t] = ask(first, t, true);
+    }
+#pragma unroll
+    for (int t = 0; t < RESIDENT; ++t) x_tiles[t] = t < count ? *reinterpret_cast<const bf16x8*>(x_ptr + t * 32) : zero;
+    // 1 / rms of the rows of x, if they come without it: every thread adds up its share of the sums of squares (asked
+    // for now, behind the first tiles of w and x), the shares meet at the first group's barrier, and the wavefront that
+    // writes the first group leaves the result for those that write the others. A fixed order throughout.
+    float my_squares = 0.f;
+    if (norm.squares_in != nullptr) {
+        const int row = threadIdx.x % 16, part = threadIdx.x / 16;
+        for (int t = part; t < norm.tiles_in; t += WAVES * XRT_WAVE / 16)
+            my_squares += norm.squares_in[(long)t * XRT_SQUARES_STRIDE + min(row, M - 1)];
+    }
+
+    int turn = 0;
+    for (long group = blockIdx.x; group < groups; group += gridDim.x, ++turn) {
+        const bf16* here = w_of(group);
+        const long next = group + gridDim.x;
+        const bool more = next < groups;
+        const bf16* there = w_of(more ? next : group);
+        floatx4 chain[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int t = 0; t < RESIDENT; ++t) {
+            const bf16x8 a = ring[t % RING];
+            // the tile RING further on: of this group, or the first ones of the next, before this group's sums meet
+            ring[t % RING] = t + RING < RESIDENT ? ask(here, t + RING, true) : ask(there, t + RING - RESIDENT, more);
+            chain[t % 2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, x_tiles[t], chain[t % 2], 0, 0, 0);
+        }
+        const int slot = turn & 1;                              // a slot is rewritten two groups later, after the next barrier
+        partial[slot][wave][lane] = chain[0] + chain[1];
+        if (turn == 0 && norm.squares_in != nullptr) square_parts[threadIdx.x / 16][threadIdx.x % 16] = my_squares;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // (not __syncthreads: that would wait for the ring's loads too)
+        if (wave != turn % WAVES) continue;                     // the wavefronts take turns at adding up and writing
+        floatx4 total = partial[slot][0][lane];
+#pragma unroll
+        for (int other = 1; other < WAVES; ++other) total += partial[slot][other][lane];
+        float g[4] = {total[0], total[1], total[2], total[3]};  // row r of x against packed rows group * 16 + c * 4 + i of w
+        if (norm.squares_in != nullptr) {
+            float by;
+            if (turn == 0) {
+                float sum = 0.f;
+                for (int other = 0; other < WAVES * XRT_WAVE / 16; ++other) sum += square_parts[other][r];
+                by = 1.0f / sqrtf(sum / (float)norm.width_in + norm.eps);
+                if (c == 0) inv_rms[r] = by;                    // read after later barriers
+            } else {
+                by = inv_rms[r];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) g[i] *= by;
+        }
+        if constexpr (MODE == MODE_GATED) {
+            float u[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) u[i] = __shfl_xor(g[i], 32);
+            const long nn = group * 8 + c * 4;                  // lanes c = 0, 1 hold the gate sums, c = 2, 3 the up sums of the same outputs
+            if (c < 2 && r < M) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (nn + i < N) out[(long)r * N + nn + i] = from_float<TO>(gate_activation(g[i], activation) * u[i]);
+            }
+        } else {
+            const long nn = logical_row(packing, group * 16 + c * 4);
+            if (r < M) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (nn + i < N) out[(long)r * N + nn + i] = from_float<TO>(g[i]);
+            }
+        }
+    }
+}
+
+// Whether the kernel above takes the product, and with how many workgroups. Two fit a compute unit, and a compute
+// unit works its workgroups off at one pace: what counts is the number of groups that the busiest one has.
+int resident_grid(int M, int K, long rows_w, int mode, bool norm_out, bool after) {
+    const long groups = (rows_w + 15) / 16;
+    if (M <= 8 || M > 16 || mode == MODE_ACCUMULATE || norm_out || after) return 0;
+    if ((K / 32 + WAVES - 1) / WAVES > RESIDENT || groups < 512) return 0;
+    const long most_256 = (groups + 255) / 256, most_512 = 2 * ((groups + 511) / 512);
+    return most_512 < most_256 ? 512 : 256;
+}
+
 template <int MT, typename TO>
 int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int mode, int activation, const Packing& packing,
                 const LinearNorm& norm, const QkvAfter* after, hipStream_t s) {
@@ -379,6 +498,14 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
     const dim3 block(WAVES * XRT_WAVE);
     const QkvAfter none = {};
     if constexpr (MT == 1) {
+        if (const int resident = resident_grid(M, K, rows_w, mode, norm.squares_out != nullptr || norm.scaled_out != nullptr, after != nullptr)) {
+            if (mode == MODE_STORE)
+                gemm_packed_resident_kernel<MODE_STORE, TO><<<resident, block, 0, s>>>(x, w, out, M, N, K, packing, norm, activation);
+            else
+                gemm_packed_resident_kernel<MODE_GATED, TO><<<resident, block, 0, s>>>(x, w, out, M, N, K, packing, norm, activation);
+            XRT_LAUNCH_CHECK("linear (packed, x resident)");
+            return 0;
+        }
         if (after) {
             if constexpr (sizeof(TO) == 2) {
                 gemm_packed_kernel<1, MODE_STORE, TO, 2><<<grid, block, 0, s>>>(x, w, out, M, N, K, packing, norm, *after, activation);
