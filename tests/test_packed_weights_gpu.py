@@ -56,8 +56,8 @@ def test_layout_pairs_gate_with_up_rows_and_the_halves_of_rotated_heads(ops):
     packed = ops.pack(w, "rotary", head_dim=hd, rotated_heads=rotated)
     flat = packed.data.cpu()
     for head, d in ((0, 0), (1, 7), (2, 8), (2, 23), (0, 24), (1, 31), (2, 47)):
-        upper, within = d // (hd // 2), d % (hd // 2)            # a group of 16 rows: 4 lower dims, their 4 partners, 4 lower, 4 partners
-        row = head * hd + within // 8 * 16 + within % 8 // 4 * 8 + upper * 4 + within % 4
+        half, within = d // (hd // 2), d % (hd // 2)
+        row = head * hd + within // 8 * 16 + half * 8 + within % 8
         assert flat[place(row, 40, cols)] == w[head * hd + d, 40].cpu(), (head, d)
     for head, d in ((3, 0), (3, 30), (4, 47)):
         assert flat[place(head * hd + d, 40, cols)] == w[head * hd + d, 40].cpu()

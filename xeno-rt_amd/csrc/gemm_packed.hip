@@ -15,8 +15,8 @@
 // Epilogues, as in the product for rows contiguous along k (gemm_skinny.hip): store, accumulate into
 // float32, the gated pair silu(gate) * up (the packing puts the gate and up rows of eight outputs into
 // one tile: a lane finds its partner 32 lanes away), an RMSNorm's halves around the product, and what
-// follows a q/k/v projection (rotation of q and k, cache write; the packing puts four pairs of a rotated
-// head into every eight rows of a tile: lane groups c = 0 and 2 hold lower dims, c = 1 and 3 their partners).
+// follows a q/k/v projection (rotation of q and k, cache write; the packing puts the two halves of a
+// rotated head's pairs into one tile).
 #include "packing.h"
 #include "gemm_skinny.h"
 #include "activation.h"
@@ -60,7 +60,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
     const int r = lane % 16, c = lane / 16;
     const long first = (long)blockIdx.x * 16;                   // the group's first packed row
     // after a q/k/v projection: the tile's head, and the dims of the head that its rows 0..7 and 8..15 make
-    int head = 0, lower_dim = 0, upper_dim = 4, dim_step = 8;     // lane group c holds dims (c % 2 ? upper_dim : lower_dim) + (c / 2) * dim_step ..+ 3
+    int head = 0, lower_dim = 0, upper_dim = 8;
     bool rotates = false;
     if constexpr (QKV) {
         head = (int)(first / after.head_dim);
@@ -68,8 +68,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
         const bool is_value = head >= after.n_heads + after.n_kv_heads;
         rotates = after.rope_theta != nullptr && !is_value;      // (the launcher checks that the packing pairs exactly these heads)
         lower_dim = rotates ? within / 2 : within;
-        upper_dim = rotates ? after.head_dim / 2 + within / 2 : within + 4;
-        dim_step = rotates ? 4 : 8;
+        upper_dim = rotates ? after.head_dim / 2 + within / 2 : within + 8;
     }
 
     const int k_tiles = K / 32;
@@ -137,7 +136,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
             const int token = min(r, M - 1);
             if (rotates && wave < 4) {                          // the lane's four angles, one per wavefront; read by wavefront 0
                 early_pos = after.positions[token];
-                early_theta = after.rope_theta[min(lower_dim + (c / 2) * 4 + wave, after.rope_dim / 2 - 1)];
+                early_theta = after.rope_theta[min(lower_dim + (c % 2) * 4 + wave, after.rope_dim / 2 - 1)];
             }
             if (wave == 4 && c == 0) {
                 early_pos = after.positions[token];
@@ -162,7 +161,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
         if constexpr (QKV) {
             if (rotates && wave < 4) {
                 const float angle = (float)early_pos * after.rope_scale / early_theta;
-                sincosf(angle, &early_sin[lane][wave], &early_cos[lane][wave]);     // lanes c and c ^ 1 hold the two halves of a pair
+                sincosf(angle, &early_sin[lane][wave], &early_cos[lane][wave]);     // lanes c and c ^ 2 hold the two halves of a pair
             }
             if (wave == 4 && c == 0 && early_slot >= 0)
                 early_block = after.block_table[(long)early_slot * after.table_stride + early_pos / XRT_BLOCK_TOKENS];
@@ -283,7 +282,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 mine[i] = to_float(from_float<bf16>(g[i]));
-                other[i] = __shfl_xor(mine[i], 16);
+                other[i] = __shfl_xor(mine[i], 32);
             }
             struct alignas(8) Four { bf16 e[4]; } packed;
 #pragma unroll
@@ -291,12 +290,12 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
                 float value = mine[i];
                 if (rotates) {
                     const float cosine = early_cos[lane][i], sine = early_sin[lane][i];
-                    value = c % 2 == 0 ? mine[i] * cosine - other[i] * sine : other[i] * sine + mine[i] * cosine;
+                    value = c < 2 ? mine[i] * cosine - other[i] * sine : other[i] * sine + mine[i] * cosine;
                 }
                 packed.e[i] = from_float<bf16>(value);
             }
             if (mm < M) {
-                const int dim = (c % 2 == 0 ? lower_dim : upper_dim) + (c / 2) * dim_step;
+                const int dim = (c < 2 ? lower_dim : upper_dim) + (c % 2) * 4;
                 *reinterpret_cast<Four*>((bf16*)out + (long)mm * N + (long)head * after.head_dim + dim) = packed;
                 const long base = early_base[r];
                 if (base >= 0) {

@@ -13,10 +13,8 @@
 //   XRT_PACK_GATED   w is [gate rows 0 .. n-1 | up rows n .. 2n-1] (n a multiple of 8): a group of 16 packed
 //                    rows holds gate rows 8g .. 8g + 7, then the up rows of the same outputs;
 //   XRT_PACK_ROTARY  w is [heads][head_dim] rows; in each of the first `rotated_heads` heads a group of 16
-//                    holds dims 8s .. 8s + 3, then dims head_dim / 2 + 8s .. + 3, then 8s + 4 .. 8s + 7, then
-//                    head_dim / 2 + 8s + 4 .. + 7: the pairs of a rotation over the whole head, four pairs to
-//                    every eight rows, so that either half of a group can be worked on alone. The other
-//                    heads keep their order.
+//                    holds dims 8s .. 8s + 7, then dims head_dim / 2 + 8s .. + 7: the pairs of a rotation
+//                    over the whole head. The other heads keep their order.
 #pragma once
 #include "common.h"
 #include "xrt_hip.h"
@@ -34,8 +32,8 @@ __host__ __device__ inline long logical_row(const Packing& p, long r) {
     if (p.kind == XRT_PACK_ROTARY) {
         const long head = r / p.head_dim, within = r % p.head_dim;
         if (head >= p.rotated_heads) return r;
-        const long s = within / 16, eight = within % 16 / 8, upper = within % 8 / 4, j = within % 4;
-        return head * p.head_dim + upper * (p.head_dim / 2) + s * 8 + eight * 4 + j;
+        const long s = within / 16, half = within % 16 / 8, j = within % 8;
+        return head * p.head_dim + half * (p.head_dim / 2) + s * 8 + j;
     }
     return r;
 }
@@ -50,8 +48,8 @@ __host__ __device__ inline long packed_row(const Packing& p, long l) {
     if (p.kind == XRT_PACK_ROTARY) {
         const long head = l / p.head_dim, d = l % p.head_dim;
         if (head >= p.rotated_heads) return l;
-        const long upper = d / (p.head_dim / 2), within = d % (p.head_dim / 2);
-        return head * p.head_dim + within / 8 * 16 + within % 8 / 4 * 8 + upper * 4 + within % 4;
+        const long half = d / (p.head_dim / 2), within = d % (p.head_dim / 2);
+        return head * p.head_dim + within / 8 * 16 + half * 8 + within % 8;
     }
     return l;
 }

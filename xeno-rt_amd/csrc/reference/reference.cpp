@@ -261,8 +261,7 @@ void xrt_ref_pack_weight(const float* w, float* packed, int rows, int K, int kin
             logical = within < 8 ? group * 8 + within : (long)gated_n + group * 8 + (within - 8);
         } else if (kind == 3 && p / head_dim < rotated_heads) {
             const long head = p / head_dim, within = p % head_dim;
-            // a group of 16: four lower dims, their four partners half a head on, the next four lower dims, their partners
-            logical = head * head_dim + (within % 8 / 4) * (head_dim / 2) + within / 16 * 8 + (within % 16 / 8) * 4 + within % 4;
+            logical = head * head_dim + (within % 16 / 8) * (head_dim / 2) + within / 16 * 8 + within % 8;
         }
         for (int k = 0; k < K; ++k) {
             const long at = ((p / 16) * (K / 32) + k / 32) * 512 + ((k % 32 / 8) * 16 + p % 16) * 8 + k % 8;

@@ -85,8 +85,8 @@ class PackedMatrix:
             packed = j // 8 * 16 + up.long() * 8 + j % 8
         elif p.kind == PACK_ROTARY:
             head, d = logical // p.head_dim, logical % p.head_dim
-            upper, within = d // (p.head_dim // 2), d % (p.head_dim // 2)
-            paired = head * p.head_dim + within // 8 * 16 + within % 8 // 4 * 8 + upper * 4 + within % 4
+            half, within = d // (p.head_dim // 2), d % (p.head_dim // 2)
+            paired = head * p.head_dim + within // 8 * 16 + half * 8 + within % 8
             packed = torch.where(head < p.rotated_heads, paired, logical)
         else:
             packed = logical
