@@ -731,10 +731,12 @@ __global__ void __launch_bounds__(256) split_reduce_rmsnorm_kernel(const float* 
         weight[i] = Four<TW>{};
         if (q < quads) {
             const long index = row + 4L * q;
-            float4 sum = *reinterpret_cast<const float4*>(parts + index);
+            typedef float floatx4 __attribute__((ext_vector_type(4)));
+            const floatx4 first = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(parts + index));     // read once, by nobody else
+            float4 sum = make_float4(first[0], first[1], first[2], first[3]);
             for (int p = 1; p < splits; ++p) {
-                const float4 part = *reinterpret_cast<const float4*>(parts + p * count + index);
-                sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+                const floatx4 part = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(parts + p * count + index));
+                sum.x += part[0]; sum.y += part[1]; sum.z += part[2]; sum.w += part[3];
             }
             const float4 before = *reinterpret_cast<const float4*>(out + index);
             kept[i] = make_float4(before.x + sum.x, before.y + sum.y, before.z + sum.z, before.w + sum.w);
