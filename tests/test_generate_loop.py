@@ -374,7 +374,7 @@ def test_buckets_of_recorded_decode_steps():
     sizes = [batch_bucket(n) for n in range(1, 130)]
     assert all(size >= n for n, size in enumerate(sizes, start=1))            # a bucket holds its batch
     assert sizes == sorted(sizes)
-    assert sorted(set(sizes)) == [1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192]
+    assert sorted(set(sizes)) == [1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192]
     assert [context_bucket(n, 5000) for n in (1, 1024, 1025, 4096, 4097, 5000)] == [1024, 1024, 2048, 4096, 5000, 5000]
 
 

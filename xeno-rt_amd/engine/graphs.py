@@ -26,12 +26,12 @@ MAX_GRAPHS = 32
 
 
 def batch_bucket(count: int) -> int:
-    """Smallest of 1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, ... that holds `count`."""
+    """Smallest of 1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, ... that holds `count`."""
     power = 1
     while power < count:
         power *= 2
     middle = power // 2 + power // 4          # 1.5 x the power of two below
-    return middle if power >= 32 and count <= middle else power
+    return middle if power >= 16 and count <= middle else power
 
 
 def context_bucket(length: int, limit: int) -> int:
