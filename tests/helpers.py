@@ -3,8 +3,10 @@ import torch
 
 # Largest difference allowed between the engine's logits and the plain implementation's,
 # relative to the largest logit of the compared block.
-#   float32: both sides round each operation to 2^-24; sums of a few hundred terms in
-#            different orders differ by about 1e-6 of the largest term.
+#   float32: both sides round each operation to 2^-24; sums of a few hundred to a few thousand terms in
+#            different orders differ by about 1e-6 of the largest term (the kernels add up in two levels,
+#            pieces of 8 or 16 terms and then the pieces' sums, which keeps a long sum's rounding small).
+#            Largest errors seen over all tests: max 4.2e-6, rms 9.5e-7; the limits are 2.4 and 2.6 times that.
 #   bfloat16: activations are rounded to 8 bits (2^-9 relative) about six times per layer;
 #            with the tests' weights (std 0.2: sharp attention, gains above one) that comes
 #            to one or two percent of the largest logit. The root-mean-square bound is
@@ -12,7 +14,7 @@ import torch
 #            tests (printed at the end of every run, with the test that had them): max 4.0e-2, rms 7.0e-3 with
 #            the tiny models' weights of std 0.2 (the stand-in for the kernels on the CPU, which shares no code
 #            with them, has 3.6e-2 at the same request); max 1.5e-2, rms 2.9e-3 at real layer sizes with std 0.02.
-TOLERANCE = {"float32": dict(max=2e-5, rms=5e-6), "bfloat16": dict(max=5e-2, rms=1.5e-2)}
+TOLERANCE = {"float32": dict(max=1e-5, rms=2.5e-6), "bfloat16": dict(max=5e-2, rms=1.5e-2)}
 
 
 def errors(got: torch.Tensor, want: torch.Tensor):

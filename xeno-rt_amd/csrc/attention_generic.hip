@@ -21,6 +21,20 @@ namespace {
 constexpr int MAX_HEAD_DIM = 512;
 constexpr int MAX_OWNED = MAX_HEAD_DIM / XRT_WAVE;
 
+// eight elements from p (aligned to eight elements: a piece of a cache block), as floats, in one or two loads
+template <typename T>
+__device__ __forceinline__ void load_piece(const T* __restrict__ p, float (&v)[8]) {
+    if constexpr (sizeof(T) == 4) {
+        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        struct alignas(16) Eight { T e[8]; };
+        const Eight q = *reinterpret_cast<const Eight*>(p);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = to_float(q.e[e]);
+    }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
     const T* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads, int head_dim,
@@ -41,6 +55,8 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
     const int pos = positions[token];
     const int first = window > 0 ? max(0, pos - window + 1) : 0;
     const float slope = distance_slopes ? distance_slopes[head] : 0.f;
+    // pieces of eight elements can be loaded whole if they are aligned: head sizes that are multiples of 8, caches aligned to 32 bytes
+    const bool whole_pieces = head_dim % 8 == 0 && (uintptr_t)k_cache % 32 == 0 && (uintptr_t)v_cache % 32 == 0;
     const T* q = qkv + (long)token * row_width + (long)head * head_dim;
     for (int e = lane; e < head_dim; e += XRT_WAVE) qs[e] = to_float(q[e]);
     wave_sync();
@@ -57,11 +73,26 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
         const long head_base = ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * head_dim;
         float s = -INFINITY;
         if (valid) {
+            // the key's dims in order, piece by piece of the cache's order: a piece's products are added up, then
+            // the pieces' sums (less rounding than one running sum)
             float dot = 0.f;
-            for (int d0 = 0; d0 < head_dim; d0 += 8) {          // the key's dims in order, piece by piece of the cache's order
-                const T* piece = k_cache + head_base + cache_key_offset(lane, d0, head_dim);
-                const int dims = min(8, head_dim - d0);
-                for (int e = 0; e < dims; ++e) dot = fmaf(qs[d0 + e], to_float(piece[e]), dot);
+            if (whole_pieces) {
+#pragma unroll 4
+                for (int d0 = 0; d0 < head_dim; d0 += 8) {
+                    float key[8], of_piece = 0.f;
+                    load_piece(k_cache + head_base + cache_key_offset(lane, d0, head_dim), key);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) of_piece = fmaf(qs[d0 + e], key[e], of_piece);
+                    dot += of_piece;
+                }
+            } else {
+                for (int d0 = 0; d0 < head_dim; d0 += 8) {
+                    const T* piece = k_cache + head_base + cache_key_offset(lane, d0, head_dim);
+                    const int dims = min(8, head_dim - d0);
+                    float of_piece = 0.f;
+                    for (int e = 0; e < dims; ++e) of_piece = fmaf(qs[d0 + e], to_float(piece[e]), of_piece);
+                    dot += of_piece;
+                }
             }
             s = dot * scale;
             if (distance_slopes) s += slope * (float)(j - pos);
@@ -80,9 +111,18 @@ __global__ void __launch_bounds__(XRT_WAVE) attention_generic_kernel(
             const int d = lane + i * XRT_WAVE;
             if (d < head_dim) {
                 float sum = 0.f;
+#pragma unroll 4
                 for (int j0 = j_begin / 8 * 8; j0 <= j_end; j0 += 8) {   // the dim's values in the order of their tokens
                     const T* piece = v_cache + head_base + cache_value_offset(d, j0, head_dim);
-                    for (int jj = max(j0, j_begin); jj <= min(j0 + 7, j_end); ++jj) sum = fmaf(ps[jj], to_float(piece[jj - j0]), sum);
+                    if (whole_pieces) {
+                        float value[8];                         // (what lies beyond the sequence's end is loaded and not used)
+                        load_piece(piece, value);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (j0 + e >= j_begin && j0 + e <= j_end) sum = fmaf(ps[j0 + e], value[e], sum);
+                    } else {
+                        for (int jj = max(j0, j_begin); jj <= min(j0 + 7, j_end); ++jj) sum = fmaf(ps[jj], to_float(piece[jj - j0]), sum);
+                    }
                 }
                 acc[i] = acc[i] * correction + sum;
             }

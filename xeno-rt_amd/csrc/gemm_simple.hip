@@ -2,9 +2,11 @@
 // on the vector ALUs (no matrix cores, no reduced precision): the product of the 32-bit
 // path, and the fallback of the bfloat16 path for shapes its fast kernels refuse.
 //
-// Every output element is the sum over k = 0, 1, 2, ... in that order, whatever the
-// number of rows, the tile it falls in or the batch around it; so a token's result does
-// not depend on how a request was cut into steps. Semantics of the reference's
+// Every output element is summed in the same order, whatever the number of rows, the tile
+// it falls in or the batch around it, so a token's result does not depend on how a request
+// was cut into steps: the products of 16 consecutive k are added up in order, and these
+// sums are added up in order (a long k then loses less to rounding than one running sum:
+// the error grows with the square root of k / 16 + 16 instead of k). Semantics of the reference's
 // row-major matvec (crates/xrt-kernels/src/cpu/matmul.rs:153-167, 269-288): w is
 // [out][in], no bias.
 #include "common.h"
@@ -72,6 +74,7 @@ __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__
         }
         if (k0 + BK < K) fetch(k0 + BK);
         __syncthreads();
+        float part[RM][4] = {}, part_up[MODE == MODE_GATED ? RM : 1][4] = {};      // this tile's sums
 #pragma unroll
         for (int kk = 0; kk < BK; ++kk) {
             float ar[RM];
@@ -82,16 +85,23 @@ __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__
 #pragma unroll
             for (int i = 0; i < RM; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
+                for (int j = 0; j < 4; ++j) part[i][j] = fmaf(ar[i], wr[j], part[i][j]);
             if constexpr (MODE == MODE_GATED) {
                 const float4 uv = *reinterpret_cast<const float4*>(&Us[kk][tx * 4]);
                 const float ur[4] = {uv.x, uv.y, uv.z, uv.w};
 #pragma unroll
                 for (int i = 0; i < RM; ++i)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) acc_up[i][j] = fmaf(ar[i], ur[j], acc_up[i][j]);
+                    for (int j = 0; j < 4; ++j) part_up[i][j] = fmaf(ar[i], ur[j], part_up[i][j]);
             }
         }
+#pragma unroll
+        for (int i = 0; i < RM; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[i][j] += part[i][j];
+                if constexpr (MODE == MODE_GATED) acc_up[i][j] += part_up[i][j];
+            }
         __syncthreads();
     }
 
