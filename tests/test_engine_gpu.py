@@ -377,3 +377,34 @@ def test_generation_a_step_ahead_equals_generation_through_the_host(dtype, graph
     assert [result.finish_reason for result in got] == ["length" if len(t) == 24 else "stop" for t in want]
     engine.cache.check()
     assert engine.cache.slots.n_held == 0 and engine.cache.held_blocks() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("arch,sizes", [
+    ("llama", dict(hidden_size=400, num_attention_heads=4, num_key_value_heads=2, intermediate_size=232)),     # heads of 100, from hidden / heads
+    ("qwen3", dict(hidden_size=96, num_attention_heads=4, num_key_value_heads=2, head_dim=72)),               # heads of 72, with head norms
+    ("llama", dict(hidden_size=40, num_attention_heads=4, num_key_value_heads=4, intermediate_size=56)),      # heads of 10
+])
+def test_head_sizes_that_are_no_multiple_of_16(dtype, arch, sizes, tmp_path):
+    """The reference takes any head size (llama.rs:125-128; the attention loops of :504-574 know no alignment):
+    heads of 100, 72 and 10 dims, whole, with the tail decoded, and in a batch of unequal lengths."""
+    from xeno_rt_amd.engine import Engine
+    raw = dict(TINY[arch], max_position_embeddings=256, **sizes)
+    folder = make_folder(raw, tmp_path / "heads", seed=19, std=0.08 if raw["hidden_size"] > 200 else 0.2)
+    plain = P.PlainModel(folder)
+    vocab = plain.config.vocab_size
+    engine = Engine.load(folder, dtype=dtype, max_tokens=64 * 12, max_slots=3)
+    requests = [token_ids(vocab, n, seed=500 + n) for n in (150, 70, 9)]
+    wants = [plain.logits(ids) for ids in requests]
+    for ids, want in zip(requests, wants):
+        whole = run_whole(engine, ids)
+        assert_logits(whole, want, dtype, f"{arch} {sizes} whole length {len(ids)}, first bad row {first_bad_position(whole, want, dtype)}")
+        got = run_tail_decoded(engine, ids)
+        assert_logits(got, want, dtype, f"{arch} {sizes} decoded tail length {len(ids)}, first bad row {first_bad_position(got, want, dtype)}")
+        if dtype == "float32":
+            assert torch.equal(got, whole), f"{arch} {sizes}: cutting changed float32 bits"
+    got = run_batched(engine, requests, [100, 66, 1])
+    for ids, logits, want in zip(requests, got, wants):
+        assert_logits(logits, want, dtype, f"{arch} {sizes} batched, request of {len(ids)}")
+    engine.cache.check()
+    assert engine.cache.slots.n_held == 0 and engine.cache.held_blocks() == 0

@@ -189,9 +189,15 @@ def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n, packed):
     w = rand(hidden, k, dtype=torch.bfloat16, seed=2, scale=0.2)
     x = rand(m, hidden, seed=3, scale=2.0)
     x[m // 2] *= 50.0                                            # rows of different size: each needs its own rms
+    eps = 1e-3
+    # a row whose mean square is about eps, and a row of zeros: only an eps that is added once, inside the root,
+    # gives the first its scale (doubled, it would be a fifth off) and the second zeros instead of NaN
+    small, zero = (0, m - 1) if m >= 3 else (None, None)
+    if small is not None:
+        a[small], a[zero] = 0.0, 0.0
+        x[small], x[zero] = rand(hidden, seed=7, scale=0.03), 0.0
     gain = (rand(hidden, seed=4) + 1.0).to(torch.bfloat16)
     v = rand(2 * n, hidden, dtype=torch.bfloat16, seed=5, scale=0.1)
-    eps = 1e-3
     fresh = x.double().cpu() + a.double().cpu() @ w.double().cpu().t()
     normed = P.rmsnorm(fresh, gain.double().cpu(), eps)
     plain_v = v
@@ -222,11 +228,19 @@ def test_rmsnorm_done_by_the_products_around_it(ops, m, hidden, k, n, packed):
         # the rows of y are rounded to bfloat16 before the product, by either way of doing the norm
         unfused = torch.empty(m, hidden, dtype=torch.bfloat16, device=DEV)
         ops.rmsnorm(x, gain, eps, unfused)
-        spread = rel(unfused.double().cpu() @ plain_v.double().cpu().t(), want)
-        assert rel(out.cpu(), want) < 2 * spread + ULP["bfloat16" if out_dtype == torch.bfloat16 else "float32"] * 2
+        by_the_kernel = unfused.double().cpu() @ plain_v.double().cpu().t()
+        spread = rel(by_the_kernel, want)
+        ulps = ULP["bfloat16" if out_dtype == torch.bfloat16 else "float32"] * 2
+        assert rel(out.cpu(), want) < 2 * spread + ulps
+        if small is not None:                                   # compared alone: the error's scale is the row's own
+            assert rel(out[small].cpu(), want[small]) < 2 * rel(by_the_kernel[small], want[small]) + ulps
+            assert float(out[zero].abs().max()) == 0.0
     glu = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
     ops.linear_glu(scaled, v_glu, glu)
     assert rel(glu.cpu(), P.swiglu(want[:, :n], want[:, n:])) < 2e-2
+    if small is not None:
+        assert rel(glu[small].cpu(), P.swiglu(want[small, :n], want[small, n:])) < 2e-2
+        assert float(glu[zero].abs().max()) == 0.0
     # and once more into the residual stream, with the norm after it handed on again
     again = ops.linear(scaled, packed_or_not(ops, plain_v[:hidden % 64 + 64].contiguous(), packed),
                        torch.zeros(m, hidden % 64 + 64, device=DEV), accumulate=True,
@@ -244,8 +258,10 @@ def test_rmsnorm_done_by_the_second_kernel_of_a_product_of_many_rows(ops, m, hid
     w = rand(hidden, k, dtype=torch.bfloat16, seed=2, scale=0.1)
     x = rand(m, hidden, seed=3, scale=2.0)
     x[m // 2] *= 50.0
-    gain = (rand(hidden, seed=4) + 1.0).to(gain_dtype)
     eps = 1e-3
+    a[0], a[m - 1] = 0.0, 0.0                                   # a row whose mean square is about eps, and a row of zeros
+    x[0], x[m - 1] = rand(hidden, seed=7, scale=0.03), 0.0
+    gain = (rand(hidden, seed=4) + 1.0).to(gain_dtype)
     fresh = x.double().cpu() + a.double().cpu() @ w.double().cpu().t()
     alone = x.clone()
     w = packed_or_not(ops, w, packed)
@@ -257,7 +273,10 @@ def test_rmsnorm_done_by_the_second_kernel_of_a_product_of_many_rows(ops, m, hid
     by_the_norm_kernel = torch.empty(m, hidden, dtype=torch.bfloat16, device=DEV)
     ops.rmsnorm(x, gain, eps, by_the_norm_kernel)
     assert torch.equal(normed, by_the_norm_kernel)
-    assert rel(normed.cpu(), P.rmsnorm(fresh, gain.double().cpu(), eps)) < ULP["bfloat16"]
+    want = P.rmsnorm(fresh, gain.double().cpu(), eps)
+    assert rel(normed.cpu(), want) < ULP["bfloat16"]
+    assert rel(normed[0].cpu(), want[0]) < ULP["bfloat16"]      # eps counts here, once and inside the root
+    assert float(normed[m - 1].abs().max()) == 0.0
 
 
 def test_rmsnorm_is_left_to_its_own_kernel_where_the_products_cannot_do_it(ops):
@@ -325,10 +344,13 @@ def i32(values):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nh,nkv,hd,rope_dim", [(4, 2, 16, 16), (6, 3, 32, 32), (8, 1, 128, 128),
-                                                (5, 5, 48, 48), (2, 1, 256, 256), (4, 4, 64, 32)])
+                                                (5, 5, 48, 48), (2, 1, 256, 256), (4, 4, 64, 32),
+                                                (4, 2, 100, 100), (3, 3, 72, 72), (2, 1, 10, 10), (2, 2, 6, 4)])
 def test_qkv_prepare(ops, dtype, nh, nkv, hd, rope_dim):
     tokens = 9
     qkv = rand(tokens, (nh + 2 * nkv) * hd, dtype=DT[dtype], seed=hd)
+    qkv[1] *= 0.01                   # heads whose mean square is about the norm's eps: eps decides their scale
+    qkv[2] = 0.0                     # and heads of zeros, which stay zeros
     positions = i32([0, 1, 63, 64, 65, 127, 128, 500, 1000])
     slots = i32([0, 0, 0, 0, 1, 1, -1, 1, 0])                  # one token is padding
     kv = make_cache(40, nkv, hd, DT[dtype], 2, 16)
@@ -348,7 +370,14 @@ def test_qkv_prepare(ops, dtype, nh, nkv, hd, rope_dim):
         assert rel(got.float(), want.float()) < tol
         assert rel(kv_got.k.float(), kv_want.k.float()) < tol
         assert torch.equal(kv_got.v, kv_want.v)
-        assert int((cache_order.plain_keys(kv_got.k) != 0).any(-1).sum()) == 8 * nkv      # eight tokens cached, padding not
+        assert int((cache_order.plain_keys(kv_got.k) != 0).any(-1).sum()) == 7 * nkv      # seven tokens cached: not the padding, and not the zeros
+        assert float(got[2].abs().max()) == 0.0
+        # the small token alone, against the plain formulas (norm of every head, then the rotation) in 64-bit
+        q = qkv[1:2, :nh * hd].double().cpu()
+        if norms:
+            q = P.head_rmsnorm(q, nh, hd, qn.double().cpu(), 1e-4)
+        q = P.rope(q, nh, hd, torch.tensor([1]), rope_dim, 10000.0)
+        assert rel(got[1, :nh * hd].float().cpu(), q[0]) < (5e-6 if dtype == "float32" else ULP[dtype])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -406,9 +435,13 @@ def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens, packed)
     x = rand(tokens, k, seed=3, scale=2.0)
     gain = (rand(k, seed=4) + 1.0).to(torch.bfloat16)
     inner = 64 if tokens <= 16 else 256
-    scaled = ops.linear(rand(tokens, inner, dtype=torch.bfloat16, seed=5), rand(k, inner, dtype=torch.bfloat16, seed=6), x,
-                        accumulate=True, then_norm=(gain, 1e-4))
+    before = rand(tokens, inner, dtype=torch.bfloat16, seed=5)
+    if tokens >= 3:                  # a row whose mean square is about the norm's eps, and a row of zeros
+        before[1], before[2] = 0.0, 0.0
+        x[1], x[2] = rand(k, seed=8, scale=0.01), 0.0
+    scaled = ops.linear(before, rand(k, inner, dtype=torch.bfloat16, seed=6), x, accumulate=True, then_norm=(gain, 1e-4))
     assert scaled is not None
+    normed_small = P.rmsnorm(x[1:2].double().cpu(), gain.double().cpu(), 1e-4) if tokens >= 3 else None
     # packed as the attention part packs it: the pairs of a rotation over whole heads side by side
     plain_w = w
     w = packed_or_not(ops, w, packed, "rotary", head_dim=hd, rotated_heads=nh + nkv if rope_dim == hd else 0)
@@ -424,7 +457,14 @@ def test_linear_qkv_in_one_kernel(ops, nh, nkv, hd, rope_dim, k, tokens, packed)
         assert float((got.float() - want.float()).abs().gt(0).float().mean()) < 0.01
         assert rel(kv_got.k.float(), kv_want.k.float()) < ULP["bfloat16"]
         assert torch.equal(kv_got.v, kv_want.v)
-        assert int((cache_order.plain_keys(kv_got.k) != 0).any(-1).sum()) == int((slots >= 0).sum()) * nkv
+        zeros = 1 if rows is scaled and tokens >= 3 else 0       # the row of zeros is cached as zeros
+        assert int((cache_order.plain_keys(kv_got.k) != 0).any(-1).sum()) == (int((slots >= 0).sum()) - zeros) * nkv
+        if rows is scaled and tokens >= 3:
+            # the small row alone against the plain formulas: its scale hangs on the eps of the norm before the projection
+            assert float(got[2].abs().max()) == 0.0
+            q = (normed_small @ plain_w[:nh * hd].double().cpu().t())
+            q = P.rope(q, nh, hd, torch.tensor([int(positions[1])]), rope_dim, 10000.0, scale=0.5) if rope_dim else q
+            assert rel(got[1, :nh * hd].float().cpu(), q[0]) < 1e-2
     # without a cache to write (a layer that reads another layer's), and with head norms (two kernels then)
     got = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
     want = torch.empty(tokens, width, dtype=torch.bfloat16, device=DEV)
@@ -485,7 +525,8 @@ def filled_cache(nkv, hd, dtype, lengths, seed=0):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 16), (6, 3, 32), (8, 1, 128), (5, 5, 48), (2, 2, 256), (32, 8, 128)])
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 16), (6, 3, 32), (8, 1, 128), (5, 5, 48), (2, 2, 256), (32, 8, 128),
+                                       (4, 2, 100), (3, 3, 72), (2, 1, 10), (4, 2, 6)])
 def test_attention(ops, dtype, nh, nkv, hd):
     lengths = [200, 65, 1]
     kv, keys, values = filled_cache(nkv, hd, DT[dtype], lengths, seed=hd)

@@ -1,4 +1,4 @@
-"""The engine at the layer sizes of real models (Llama-3-8B and Qwen3-8B shapes, two layers of
+"""The engine at the layer sizes of real models (Llama-3-8B, Qwen3-8B and Qwen3-32B shapes, two layers of
 them) and at a context of 4096, against the plain implementation, in 32-bit and in bfloat16.
 
 Weights come from the random-weights mode in memory (`Engine.random`); the plain model gets the
@@ -26,12 +26,17 @@ SHAPES = {
                      num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
                      rms_norm_eps=1e-6, rope_theta=1000000.0, max_position_embeddings=4096,
                      tie_word_embeddings=False, hidden_act="silu"),
+    # a width that is no power of two, groups of eight query heads, products of k = 25600
+    "qwen3-32b": dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=5120, intermediate_size=25600,
+                      num_hidden_layers=2, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+                      rms_norm_eps=1e-6, rope_theta=1000000.0, max_position_embeddings=4096,
+                      tie_word_embeddings=False, hidden_act="silu"),
 }
-LAYERS_OF_THE_MODELS = {"llama3-8b": 32, "qwen3-8b": 36}       # the tests run two layers of these sizes
+LAYERS_OF_THE_MODELS = {"llama3-8b": 32, "qwen3-8b": 36, "qwen3-32b": 64}       # the tests run two layers of these sizes
 CONTEXT, TAIL = 4096, 40
 PORTIONS = [1024, 2, 2046, 984]             # 4056 tokens: a start on a block's boundary, two tokens, an end at a block's end
 WHOLE = 300
-SEED = {"llama3-8b": 3, "qwen3-8b": 4}
+SEED = {"llama3-8b": 3, "qwen3-8b": 4, "qwen3-32b": 5}
 
 
 def batch_plan(vocab):

@@ -1,7 +1,7 @@
 // Entry point of attention: checks the operands and picks the kernel.
 //   bfloat16, head size 64 or 128, no window: the matrix-core kernels: decode (every sequence
 //   brings one token) or prefill (any token counts);
-//   everything else (float32, other head sizes, windows, scores biased by distance): the general kernel.
+//   everything else (float32, any other head size up to 512, windows, scores biased by distance): the general kernel.
 #include "common.h"
 #include "xrt_hip.h"
 
@@ -40,7 +40,7 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
                              float* workspace, long workspace_floats, void* stream) {
     XRT_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention: head counts %d/%d: the first must be a multiple of the second", n_heads, n_kv_heads);
-    XRT_REQUIRE(head_dim > 0 && head_dim % 16 == 0, "attention: head_dim %d must be a multiple of 16", head_dim);
+    XRT_REQUIRE(head_dim > 0, "attention: head_dim %d must be positive", head_dim);
     XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "attention: unknown dtype %d", dtype);
     XRT_REQUIRE(qkv && k_cache && v_cache && block_table && positions && slots && out, "attention: null operand");
     XRT_REQUIRE(table_stride > 0 && n_blocks > 0, "attention: empty cache");

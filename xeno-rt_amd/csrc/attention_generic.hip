@@ -1,5 +1,5 @@
 // Causal attention of every token of a step over its own sequence's cache, float32 math,
-// for any element type, head size (multiples of 16 up to 512), head grouping and window.
+// for any element type, head size (up to 512), head grouping and window.
 // It is the attention of the 32-bit path and the fallback of the bfloat16 path.
 //
 // Reference: crates/xrt-models/src/llama.rs:504-574 (online softmax: running maximum m and

@@ -121,12 +121,16 @@ class Engine:
                  top_k: int = 0, top_p: float = 1.0, repetition_penalty: float = 1.0, seed: Optional[int] = 0,
                  stop_ids: Optional[Sequence[int]] = None, batch_size: Optional[int] = None) -> List[List[int]]:
         """The generated token ids of every prompt, with one set of sampling options for all
-        (greedy unless told otherwise). `generate()` of this package takes a request per prompt
-        with options of its own and returns finish reasons and timings as well."""
+        (greedy unless told otherwise). Every prompt draws from a stream of its own, made from `seed`
+        and the prompt's index (seed=None: from the system's randomness). `generate()` of this package
+        takes a request per prompt with options of its own and returns finish reasons and timings as well."""
+        from ..sampling import request_seed
         from .generate import GenerateRequest, generate
         requests = [GenerateRequest(list(ids), max_tokens=max_tokens, temperature=temperature, top_k=top_k,
-                                    top_p=top_p, repetition_penalty=repetition_penalty, seed=seed,
-                                    stop_ids=None if stop_ids is None else tuple(stop_ids)) for ids in prompts]
+                                    top_p=top_p, repetition_penalty=repetition_penalty,
+                                    seed=None if seed is None else request_seed(seed, index),
+                                    stop_ids=None if stop_ids is None else tuple(stop_ids))
+                    for index, ids in enumerate(prompts)]
         return [list(result.tokens) for result in generate(self, requests, batch_size=batch_size)]
 
     def get_tensor(self, name: str) -> torch.Tensor:

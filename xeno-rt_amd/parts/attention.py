@@ -36,8 +36,8 @@ class Attention(Mixer):
                  window: Optional[int] = None):
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
             raise ValueError(f"head counts {n_heads}/{n_kv_heads}: the first must be a multiple of the second")
-        if head_dim <= 0 or head_dim % 16 != 0:
-            raise ValueError(f"head_dim {head_dim} must be a positive multiple of 16")
+        if head_dim <= 0 or head_dim % 2 != 0:          # llama.rs:125-128 takes any size; the rotation pairs dims, so an even one
+            raise ValueError(f"head_dim {head_dim} must be positive and even")
         self.prefix = prefix
         self.hidden = hidden
         self.n_heads = n_heads

@@ -12,8 +12,10 @@ sequence, for greedy too (:77-91, :110-125).
 The work is done by one kernel on the device for all rows of a batch. Two things
 differ from the reference by design: tokens whose logit equals the k-th largest
 (or the last of the top_p prefix) are all kept, and the uniform numbers come from
-a counter-based generator keyed by (seed, request, step), so that a request draws
-the same numbers alone and in any batch.
+a counter-based generator keyed by (the request's own seed, step), so that a request
+draws the same numbers alone and in any batch, whatever its place in it. Requests that
+are given one seed therefore draw the same numbers; `request_seed(seed, index)` makes
+a seed of its own for each of several prompts that share one.
 """
 from __future__ import annotations
 
@@ -55,6 +57,11 @@ def uniform(seed: int, request: int, step: int) -> float:
     """A number in [0, 1) that depends only on (seed, request, step)."""
     word = _mix(_mix(_mix(seed & _MASK) ^ (request & _MASK)) ^ (step & _MASK))
     return (word >> 40) / float(1 << 24)
+
+
+def request_seed(seed: int, index: int) -> int:
+    """A seed for the index-th of several requests that were given one seed between them."""
+    return _mix(_mix(seed & _MASK) ^ ((index + 1) & _MASK)) >> 1
 
 
 class TokenLog:
