@@ -170,9 +170,19 @@ def test_far_keys_among_hundreds(dtype, tmp_path):
         assert worst < 0.1 and rms < 0.01, "the stand-in itself is off"
         want = rounded
     engine = Engine.load(folder, dtype=dtype, max_tokens=1024)
-    assert_logits(run_whole(engine, ids), want, dtype, "700 tokens whole")
+    whole = run_whole(engine, ids)
+    assert_logits(whole, want, dtype, "700 tokens whole")
     got = run_tail_decoded(engine, ids)
     assert_logits(got, want, dtype, f"700 tokens, tail decoded, first bad row {first_bad_position(got, want, dtype)}")
+    if dtype == "bfloat16":
+        # and against the plain model itself, so that the engine has a bound that does not hang on the stand-in:
+        # what is asked of the stand-in above, and the plain model's choice of token in nearly every row
+        plain_logits = plain.logits(ids)
+        for what, rows in (("whole", whole), ("tail decoded", got)):
+            worst, rms = errors(rows, plain_logits)
+            assert worst < 0.1 and rms < 0.01, f"700 tokens {what} against the plain model: max {worst:.3e}, rms {rms:.3e}"
+            same = (rows.argmax(-1).cpu() == plain_logits.argmax(-1)).float().mean()
+            assert float(same) > 0.9, f"700 tokens {what}: the plain model's token in only {float(same):.2f} of the rows"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

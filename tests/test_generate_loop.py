@@ -311,6 +311,24 @@ def test_engine_conveniences(pair):
         engine.get_tensor("model.no_such.weight")
 
 
+def test_prompts_that_share_a_seed_draw_from_streams_of_their_own(pair):
+    """Engine.generate gives every prompt a seed made from the one it was given and the prompt's index: equal prompts
+    sampled with a temperature part ways, the same call gives the same tokens again, and a prompt's tokens do not
+    depend on what else is in the call."""
+    from xeno_rt_amd.engine import GenerateRequest, generate
+    from xeno_rt_amd.sampling import request_seed
+    engine, _ = pair
+    prompt = [4, 8, 15, 16]
+    options = dict(max_tokens=12, temperature=1.5, stop_ids=[])
+    first = engine.generate([prompt, prompt, prompt], seed=7, **options)
+    assert first[0] != first[1] and first[1] != first[2] and first[0] != first[2]
+    assert engine.generate([prompt, prompt, prompt], seed=7, **options) == first
+    assert engine.generate([prompt, prompt], seed=8, **options)[0] != first[0]
+    alone = generate(engine, [GenerateRequest(prompt, seed=request_seed(7, 1), repetition_penalty=1.0, top_k=0, top_p=1.0, **options)])
+    assert alone[0].tokens == first[1]
+    assert len({request_seed(7, i) for i in range(1000)} | {request_seed(8, i) for i in range(1000)}) == 2000
+
+
 def test_norms_are_handed_to_the_products_only_where_every_part_agrees(pair, tmp_path):
     """A norm between two products may be done by them (parts with `passes_norms`); the result is the same
     with and without, and a part that does not say so is never given anything but tensors."""

@@ -132,6 +132,66 @@ def test_attention_part_prompt_then_decode(dtype, nh, nkv, hd, qk_norm):
     assert part.scale == 1.0 / math.sqrt(hd)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden,nh,nkv,hd,rope_dim", [(4096, 32, 8, 128, 128), (96, 4, 2, 32, 16)])
+def test_a_rotation_defined_here_takes_the_fused_path_without_being_the_library_s_rotary(dtype, hidden, nh, nkv, hd, rope_dim):
+    """An encoding of this file that rotates half-split pairs by angles from a table of its own (no power law) says so
+    with `rotation()`; the attention part then packs the projection for it and lets the projection's kernel rotate,
+    knowing nothing of the class. A prompt of 20 tokens, then 8 single tokens (at the first sizes: the packed product
+    with the rotation and the cache write in its epilogue), against plain arithmetic."""
+    from xeno_rt_amd.cache import SequenceCache
+    from xeno_rt_amd.parts import Attention
+    from xeno_rt_amd.parts.base import HalfSplitRotation, PositionEncoding
+
+    class TableRotation(PositionEncoding):
+        capturable = True
+
+        def __init__(self, rope_dim, scale):
+            self.rope_dim, self.scale = rope_dim, scale
+            self.table = 1.0 + 3.0 * torch.arange(rope_dim // 2, dtype=torch.float32) ** 1.5
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.theta = self.table.to(runtime.device)
+
+        def rotation(self):
+            return HalfSplitRotation(self.rope_dim, self.scale, self.theta)
+
+        def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch):
+            raise AssertionError("a rotation that describes itself is done by the projection's kernel")
+
+    position = TableRotation(rope_dim, 0.5)
+    part = Attention("a.", hidden, nh, nkv, hd, position=position)
+    w = weights_for(part, 3, std=1.5 / math.sqrt(hidden))
+    rt = runtime(dtype)
+    part.bind(w, rt)
+    if dtype == "bfloat16" and hidden == 4096:
+        assert hasattr(part.w_qkv, "unpacked") and part.w_qkv.packing.rotated_heads == nh + nkv      # the pairs side by side
+    length, prompt = 28, 20
+    h = torch.randn(length, hidden, generator=torch.Generator().manual_seed(8)).to(DT[dtype])
+
+    def rotate(x, heads):
+        x = x.reshape(length, heads, hd).clone()
+        angle = (torch.arange(length, dtype=torch.float32)[:, None] * 0.5 / position.table[None, :]).double()
+        a, b = x[:, :, :rope_dim // 2].clone(), x[:, :, rope_dim // 2:rope_dim].clone()
+        x[:, :, :rope_dim // 2] = a * angle.cos()[:, None] - b * angle.sin()[:, None]
+        x[:, :, rope_dim // 2:rope_dim] = a * angle.sin()[:, None] + b * angle.cos()[:, None]
+        return x.reshape(length, heads * hd)
+
+    q, k, v = (P.linear(h.double(), w[f"a.{n}_proj.weight"].double()) for n in "qkv")
+    want = P.linear(P.causal_attention(rotate(q, nh), rotate(k, nkv), v, nh, nkv, hd), w["a.o_proj.weight"].double())
+    cache = SequenceCache([part.cache_needs()], [0], 128, 1, 128, DT[dtype], DEV)
+    slot = cache.alloc_slot()
+    got = []
+    for first, count in [(0, prompt)] + [(t, 1) for t in range(prompt, length)]:
+        batch, _ = batch_for(cache, [slot], [count])
+        residual = torch.zeros(count, hidden, device=DEV)
+        part.forward(h[first:first + count].to(DEV), batch, cache.layer_cache(0), residual)
+        got.append(residual)
+        cache.commit(slot, first + count)
+    assert rel(torch.cat(got), want) < TOL[dtype]
+
+
 def attention_with_scores_biased_by_distance(rt, dtype, device):
     """A position encoding defined here, which leaves q and k alone and lowers the scores of far keys instead
     (one slope per head): the attention part hands its slopes to the kernel. A prompt, then single tokens.
@@ -204,8 +264,9 @@ def test_parts_are_found_by_kind_and_name():
     assert isinstance(create_part("position", "rotary", rope_dim=8, base=10.0), Rotary)
     with pytest.raises(KeyError, match="no mixer named"):
         create_part("mixer", "nonesuch")
-    with pytest.raises(ValueError, match="multiple of 16"):
-        create_part("mixer", "attention", prefix="a.", hidden=8, n_heads=2, n_kv_heads=1, head_dim=20)
+    assert create_part("mixer", "attention", prefix="a.", hidden=8, n_heads=2, n_kv_heads=1, head_dim=20).head_dim == 20
+    with pytest.raises(ValueError, match="even"):
+        create_part("mixer", "attention", prefix="a.", hidden=8, n_heads=2, n_kv_heads=1, head_dim=21)
     with pytest.raises(ValueError, match="multiple"):
         create_part("mixer", "attention", prefix="a.", hidden=8, n_heads=3, n_kv_heads=2, head_dim=16)
 

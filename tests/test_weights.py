@@ -104,7 +104,8 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
 
 def test_tied_head_in_the_file_is_ignored_untied_head_is_required(tmp_path):
     folder, spec = folder_with(tmp_path, "qwen3", lambda t: t.update({"lm_head.weight": torch.zeros(384, 96)}))
-    assert "lm_head.weight" not in load_tensors(folder, spec.weight_specs(), spec.ignored_names())
+    with pytest.warns(UserWarning, match="lm_head.weight ignored"):        # left alone, and said so
+        assert "lm_head.weight" not in load_tensors(folder, spec.weight_specs(), spec.ignored_names())
     folder, spec = folder_with(tmp_path, "llama", lambda t: t.pop("lm_head.weight"))
     with pytest.raises(WeightError, match="lm_head.weight"):
         load_tensors(folder, spec.weight_specs(), spec.ignored_names())
@@ -230,3 +231,33 @@ def test_sharded_checkpoints_are_read_through_the_index(tmp_path):
         json.dump({"weight_map": weight_map}, handle)
     loaded = load_tensors(folder, spec.weight_specs())
     assert all(torch.equal(loaded[n], tensors[n]) for n in names)
+
+
+def test_an_engine_closes_the_files_of_its_checkpoint_once_the_weights_are_bound(tmp_path):
+    """A tied model whose file also carries the head's matrix: a warning, the same logits; the shards are closed when
+    the parts have bound their tensors, and get_tensor opens them again for its one read."""
+    import warnings
+    from ops_emulation import EmulatedOps
+    from xeno_rt_amd.engine import Engine
+    from xeno_rt_amd.weights import CheckpointSource
+    folder, spec = folder_with(tmp_path, "qwen3", lambda t: None)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")                                      # nothing to warn of here
+        plain = Engine.load(folder, dtype="float32", max_tokens=128, device="cpu", ops=EmulatedOps())
+    assert isinstance(plain.tensors, CheckpointSource) and not plain.tensors.is_open
+    again = plain.get_tensor("model.norm.weight")
+    assert not plain.tensors.is_open and again.shape == (96,)
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as file:
+        tensors = {name: file.read(name) for name in file.names()}
+    assert torch.equal(again, tensors["model.norm.weight"])
+    tensors["lm_head.weight"] = torch.full((384, 96), 3.0)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    with pytest.warns(UserWarning, match="lm_head.weight ignored"):
+        carrying = Engine.load(folder, dtype="float32", max_tokens=128, device="cpu", ops=EmulatedOps())
+    ids = [5, 9, 200, 31]
+    rows = []
+    for engine in (plain, carrying):
+        slot = engine.alloc_slot()
+        rows.append(engine.step([(slot, ids, [3])]))
+        engine.free_slot(slot)
+    assert torch.equal(*rows)

@@ -12,9 +12,6 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
-STATIC_FLOATS = 4 << 20         # XRT_LINEAR_STATIC_FLOATS of the library's header
-
-
 def library():
     from xeno_rt_amd.ops import build
     path = build.find_library() or build.build()
@@ -23,6 +20,7 @@ def library():
     lib.xrt_linear_workspace.restype = ctypes.c_long
     lib.xrt_linear.restype = ctypes.c_int
     lib.xrt_linear_static.restype = ctypes.c_int
+    lib.xrt_linear_static_floats.restype = ctypes.c_long
     return lib
 
 
@@ -72,7 +70,7 @@ def test_two_calls_in_a_row_share_the_fixed_array():
     for m, n, k, mode, seed in ((64, 4096, 4096, 1, 1), (24, 1024, 2048, 0, 2), (40, 1536, 1024, 2, 3),
                                 (8, 512, 256, 0, 4)):
         want, got, need = both_ways(lib, m, n, k, mode, seed)
-        assert need <= STATIC_FLOATS
+        assert need <= int(lib.xrt_linear_static_floats())
         if m > 16 and mode != 2:
             assert need > 0, "this product was meant to be split along k"
         assert torch.equal(want, got), (m, n, k, mode)
@@ -83,7 +81,7 @@ def test_a_product_beyond_the_fixed_array_is_refused_and_nothing_is_written():
     m, n, k = 256, 2048, 8192
     a, w, _ = operands(m, n, k, 0, 5)
     need = int(lib.xrt_linear_workspace(pointer(a), pointer(w), 1, m, n, k, 0))
-    assert need > STATIC_FLOATS
+    assert need > int(lib.xrt_linear_static_floats())
     out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     status = lib.xrt_linear_static(pointer(a), pointer(w), 1, pointer(out), 1, m, n, k, 0, stream)
@@ -92,3 +90,28 @@ def test_a_product_beyond_the_fixed_array_is_refused_and_nothing_is_written():
     assert "fixed buffer" in message and str(need) in message
     torch.cuda.synchronize()
     assert bool((out == 7.0).all())
+
+
+def test_the_calls_allocate_no_device_memory():
+    """What the entry point is for: after a first call (which may load the code object and asks for the array's
+    address), calls of every kind, split along k or not, leave the device's free memory as it was."""
+    lib = library()
+    cases = [(operands(m, n, k, mode, seed), (m, n, k, mode))
+             for m, n, k, mode, seed in ((64, 4096, 4096, 1, 1), (24, 1024, 2048, 0, 2), (40, 1536, 1024, 2, 3), (8, 512, 256, 0, 4))]
+    outs = [start.clone() if mode == 1 else torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+            for (_, _, start), (m, n, k, mode) in cases]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def call_all():
+        for ((a, w, _), (m, n, k, mode)), out in zip(cases, outs):
+            status = lib.xrt_linear_static(pointer(a), pointer(w), 1, pointer(out), 0 if mode == 1 else 1, m, n, k, mode, stream)
+            assert status == 0, lib.xrt_last_error().decode()
+
+    call_all()
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        call_all()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, f"free device memory went from {free_before} to {free_after} bytes"

@@ -62,7 +62,8 @@ def run_generate(args) -> int:
     stops = None if args.stop_ids is None else [int(t) for t in args.stop_ids.replace(",", " ").split()]
     cache_tokens = args.cache_tokens
     if cache_tokens is None:
-        cache_tokens = sum(-(-(len(p) + max(1, args.max_tokens)) // 64) * 64 for p in prompts) + 64
+        from .cache import BLOCK_TOKENS          # requests hold the cache in whole blocks
+        cache_tokens = sum(-(-(len(p) + max(1, args.max_tokens)) // BLOCK_TOKENS) * BLOCK_TOKENS for p in prompts) + BLOCK_TOKENS
     if args.model:
         runtime = Runtime.load(args.model, dtype=args.dtype, max_tokens=cache_tokens)
     else:

@@ -314,7 +314,7 @@ Cut cut_for(int tokens, int n_kv_heads, int q_tiles, int max_context, int head_d
         const int n_chunks = (max_blocks + chunk_blocks - 1) / chunk_blocks;
         const int n_parts = (n_chunks + WAVES - 1) / WAVES;
         if ((long)(n_parts - 1) * WAVES * chunk_blocks >= max_blocks) continue;         // a part without keys: a shorter chunk does the same
-        const long per_unit = (pairs * n_parts + 255) / 256;
+        const long per_unit = (pairs * n_parts + XRT_COMPUTE_UNITS - 1) / XRT_COMPUTE_UNITS;
         const long ns = per_unit * (chunk_blocks * block_ns + group_ns) + (n_parts > 1 ? merge_ns : 0);
         if (best_ns < 0 || ns < best_ns) { best_ns = ns; best = Cut{chunk_blocks, n_parts}; }
     }

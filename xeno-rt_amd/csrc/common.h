@@ -14,6 +14,8 @@ enum { XRT_F32 = 0, XRT_BF16 = 1 };
 // tokens per cache block; keys are [kv_head][token][dim], values [kv_head][dim][token] inside a block
 #define XRT_BLOCK_TOKENS 64
 #define XRT_WAVE 64
+// compute units of the chip: what the launchers count in when they deal work out in rounds
+#define XRT_COMPUTE_UNITS 256
 
 // ---- error reporting -------------------------------------------------------
 void xrt_set_error(const char* format, ...);

@@ -522,7 +522,7 @@ int launch(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int n_fir
 // share its matrix cores), and a partly filled last round costs a whole one. `penalty` is what a
 // tile shape loses against the largest, in percent, from reading its operands more often.
 long rounds_cost(long tiles, int tile_elements, int share, int penalty) {
-    const long rounds = (tiles + 256L * share - 1) / (256L * share);
+    const long rounds = (tiles + (long)XRT_COMPUTE_UNITS * share - 1) / ((long)XRT_COMPUTE_UNITS * share);
     return rounds * share * tile_elements * (100 + penalty) / 100;
 }
 
@@ -539,10 +539,10 @@ int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, cons
     // rest, if those then fit one round: the last round is full of half-sized work instead of
     // half empty.
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 256 / DIV - 1) / (256 / DIV);
-    const int whole_columns = (int)((long)tiles_m * tiles_n / 256 * 256 / tiles_m);     // n-tiles that run in full rounds
+    const int whole_columns = (int)((long)tiles_m * tiles_n / XRT_COMPUTE_UNITS * XRT_COMPUTE_UNITS / tiles_m);     // n-tiles that run in full rounds
     const long rest_tiles = (long)((M + 127) / 128) * (tiles_n - whole_columns);
     long mixed = LONG_MAX;
-    if (whole_k && whole_columns > 0 && whole_columns < tiles_n && rest_tiles <= 256)
+    if (whole_k && whole_columns > 0 && whole_columns < tiles_n && rest_tiles <= XRT_COMPUTE_UNITS)
         mixed = rounds_cost((long)tiles_m * whole_columns, 256 * 256, 1, 0) + rounds_cost(rest_tiles, 128 * 256, 1, 8);
     if (mixed < large && mixed <= medium && mixed <= small) {
         const int split = whole_columns * (256 / DIV);
@@ -597,14 +597,14 @@ SplitPlan split_plan(int M, int N, int K, int mode, bool whole_norm = false) {
     int splits, least, tile = SPLIT_BM;                        // least: pieces of k that a part should have
     const long large_tiles = (long)((M + 255) / 256) * ((rows_w + 255) / 256);
     if (M <= SPLIT_BM) {
-        splits = (int)(256 / tiles_n);                         // one workgroup per compute unit, or fewer
+        splits = (int)(XRT_COMPUTE_UNITS / tiles_n);                         // one workgroup per compute unit, or fewer
         least = 1;
     } else if (large_tiles <= 128 && M >= 512 && mode != MODE_GATED && units >= (whole_norm ? 64 : 128)) {
         // Many rows and a very long k, but so few columns that the largest tiles would leave half of the compute
         // units idle (the projection back from the feed-forward's width): the large tiles split k between them.
         // The tiles of 128 x 128, which fill the chip without a second kernel, read their operands from LDS
         // more often for the same products and take longer here.
-        splits = (int)(256 / large_tiles);
+        splits = (int)(XRT_COMPUTE_UNITS / large_tiles);
         splits = splits > 8 ? 8 : splits;
         least = 24;
         tile = 256;

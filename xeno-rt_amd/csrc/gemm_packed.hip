@@ -486,8 +486,9 @@ int resident_grid(int M, int K, long rows_w, int mode, bool norm_out, bool after
     const long groups = (rows_w + 15) / 16;
     if (M <= 8 || M > 16 || mode == MODE_ACCUMULATE || norm_out || after) return 0;
     if ((K / 32 + WAVES - 1) / WAVES > RESIDENT || groups < 512) return 0;
-    const long most_256 = (groups + 255) / 256, most_512 = 2 * ((groups + 511) / 512);
-    return most_512 < most_256 ? 512 : 256;
+    constexpr int ONCE = XRT_COMPUTE_UNITS, TWICE = 2 * XRT_COMPUTE_UNITS;
+    const long most_once = (groups + ONCE - 1) / ONCE, most_twice = 2 * ((groups + TWICE - 1) / TWICE);
+    return most_twice < most_once ? TWICE : ONCE;
 }
 
 template <int MT, typename TO>

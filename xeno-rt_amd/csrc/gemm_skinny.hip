@@ -450,8 +450,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
 // epilogue moves four values at a time). The tile that the rotation after a q/k/v projection pairs stays at
 // 16 (768 tiles of 8 rows were slower than 384 of 16).
 int balanced_rows(int N, int mode) {
-    const long rounds = ((N + 15) / 16 + 255) / 256;
-    int rows = (int)((N + 256 * rounds - 1) / (256 * rounds));
+    const long rounds = ((N + 15) / 16 + XRT_COMPUTE_UNITS - 1) / XRT_COMPUTE_UNITS;
+    int rows = (int)((N + XRT_COMPUTE_UNITS * rounds - 1) / (XRT_COMPUTE_UNITS * rounds));
     if (mode == MODE_ACCUMULATE) rows = (rows + 3) / 4 * 4;
     return rows < 8 ? 8 : (rows > 16 ? 16 : rows);
 }
@@ -469,7 +469,7 @@ int launch_mode(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int 
         auto most = [&](int kv_rows) {                          // rows of the fullest compute unit (the first)
             const long kv = kv_tiles * (16 / kv_rows);
             long sum = 0;
-            for (long group = 0; group < query_tiles + kv; group += 256) sum += group < query_tiles ? 16 : kv_rows;
+            for (long group = 0; group < query_tiles + kv; group += XRT_COMPUTE_UNITS) sum += group < query_tiles ? 16 : kv_rows;
             return sum;
         };
         then.kv_rows = most(8) < most(16) ? 8 : 16;

@@ -42,6 +42,8 @@ static int scratch_pointer(float** pointer) {
     return 0;
 }
 
+extern "C" long xrt_linear_static_floats(void) { return (long)XRT_LINEAR_STATIC_FLOATS; }
+
 extern "C" int xrt_linear_static(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N,
                                  int K, int mode, void* stream) {
     XRT_REQUIRE(M >= 0 && N > 0 && K > 0, "linear (static): bad sizes M=%d N=%d K=%d", M, N, K);

@@ -54,6 +54,6 @@ extern "C" int xrt_pack_weight(const void* w, void* packed, int rows, int K, con
 extern "C" int xrt_packing_suits(int rows, int K) {
     if (rows <= 0 || K <= 0 || K % 32 != 0) return 0;
     const long groups = ((long)rows + 15) / 16;
-    const long rounds = (groups + 255) / 256;
-    return groups <= 64 || rounds * 256 * 100 <= groups * 135;
+    const long rounds = (groups + XRT_COMPUTE_UNITS - 1) / XRT_COMPUTE_UNITS;
+    return groups <= 64 || rounds * XRT_COMPUTE_UNITS * 100 <= groups * 135;
 }

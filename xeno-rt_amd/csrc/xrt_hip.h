@@ -85,6 +85,7 @@ int xrt_linear_with(const void* a, const void* w, const xrt_packing* packing, in
 // whose partial sums do not fit (xrt_linear_workspace says how many floats a product needs). Calls on one
 // GPU share that array: calls that overlap there (different streams) race.
 #define XRT_LINEAR_STATIC_FLOATS (4L << 20)
+long xrt_linear_static_floats(void);       // XRT_LINEAR_STATIC_FLOATS, for callers that do not read this header
 int xrt_linear_static(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
                       int mode, void* stream);
 

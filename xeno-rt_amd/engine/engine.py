@@ -37,6 +37,9 @@ def compute_dtype(name) -> torch.dtype:
     return _DTYPES[name]
 
 
+MOST_SLOTS_BY_DEFAULT = 1024     # slots of a cache whose maker names no number: a block each, up to this many
+
+
 class StepError(ValueError):
     """A step that cannot run; nothing was computed and the cache is unchanged."""
 
@@ -58,6 +61,8 @@ class Engine:
         # keeps none, so that the device holds every weight once, in the form the parts bound it
         self.tensors = tensors
         self.model = DecoderModel(spec, tensors, self.runtime)
+        if hasattr(tensors, "release"):
+            tensors.release()           # every part has bound what it needs: a checkpoint's files are closed (get_tensor opens them again)
         model_context = getattr(spec.config, "max_position_embeddings", None)
         limit = max_context if max_context is not None else model_context
         if limit is None:
@@ -65,7 +70,7 @@ class Engine:
         if model_context is not None:
             limit = min(limit, model_context)
         if max_slots is None:
-            max_slots = max(1, min((max_tokens + BLOCK_TOKENS - 1) // BLOCK_TOKENS, 1024))
+            max_slots = max(1, min((max_tokens + BLOCK_TOKENS - 1) // BLOCK_TOKENS, MOST_SLOTS_BY_DEFAULT))
         schedule = spec.schedule
         reads_from = [i if call.reads_cache_of is None else call.reads_cache_of
                       for i, call in enumerate(schedule)]

@@ -21,8 +21,8 @@ import torch
 from ..staging import staging_for
 from .batch import StepBatch
 
-CONTEXT_BUCKET = 1024
-MAX_GRAPHS = 32
+CONTEXT_BUCKET = 1024    # a recorded step serves contexts up to the next multiple of this (the decode attention cuts its keys by it)
+MAX_GRAPHS = 32          # recorded steps kept at a time
 
 
 def batch_bucket(count: int) -> int:

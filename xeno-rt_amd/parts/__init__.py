@@ -1,5 +1,5 @@
 """Parts that models are built from."""
-from .base import (Block, CacheNeeds, FeedForward, KVSpec, Mixer, Norm, Part, PositionEncoding,
+from .base import (Block, CacheNeeds, FeedForward, HalfSplitRotation, KVSpec, Mixer, Norm, Part, PositionEncoding,
                    Runtime, StateSpec, WeightSpec, create_part, register_part, registered_parts)
 from .norm import RMSNorm
 from .position import NoPosition, Rotary
@@ -9,7 +9,7 @@ from .block import PreNormBlock
 from .embedding import Embedding, OutputHead
 
 __all__ = [
-    "Block", "CacheNeeds", "FeedForward", "KVSpec", "Mixer", "Norm", "Part", "PositionEncoding",
+    "Block", "CacheNeeds", "FeedForward", "HalfSplitRotation", "KVSpec", "Mixer", "Norm", "Part", "PositionEncoding",
     "Runtime", "StateSpec", "WeightSpec", "create_part", "register_part", "registered_parts",
     "RMSNorm", "NoPosition", "Rotary", "Attention", "GatedMLP", "PreNormBlock", "Embedding", "OutputHead",
 ]

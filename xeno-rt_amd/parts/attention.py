@@ -20,7 +20,6 @@ from typing import Dict, Optional
 import torch
 
 from .base import CacheNeeds, KVSpec, Mixer, PositionEncoding, Runtime, WeightSpec, register_part
-from .position import Rotary
 
 
 class Attention(Mixer):
@@ -74,8 +73,11 @@ class Attention(Mixer):
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         p = self.prefix
+        if self.position is not None:
+            self.position.bind(tensors, runtime)
         # q and k heads that a rotation over the whole head turns: their pairs are kept side by side
-        whole = isinstance(self.position, Rotary) and self.position.rope_dim == self.head_dim
+        rotation = None if self.position is None else self.position.rotation()
+        whole = rotation is not None and rotation.rope_dim == self.head_dim
         self.w_qkv = runtime.weight([tensors[p + name] for name in ("q_proj.weight", "k_proj.weight", "v_proj.weight")],
                                     "rotary", head_dim=self.head_dim,
                                     rotated_heads=self.n_heads + self.n_kv_heads if whole else 0)
@@ -83,8 +85,6 @@ class Attention(Mixer):
         if self.qk_norm:
             self.q_norm = runtime.vector(tensors[p + "q_norm.weight"])
             self.k_norm = runtime.vector(tensors[p + "k_norm.weight"])
-        if self.position is not None:
-            self.position.bind(tensors, runtime)
 
     def forward(self, h, batch, cache, residual: torch.Tensor, then=None):
         rt = self.runtime
@@ -96,14 +96,14 @@ class Attention(Mixer):
         dims = (self.n_heads, self.n_kv_heads, self.head_dim)
         write_to = kv if cache.writable else None
         longest_run = int(getattr(batch, "max_count", 0) or 0)      # picks how the values are written; 0: unknown
-        rotary = self.position if isinstance(self.position, Rotary) else None
-        if rotary is not None or self.position is None:
+        rotation = None if self.position is None else self.position.rotation()
+        if rotation is not None or self.position is None:
             # the projection, then in one pass (in the same kernel, where a step is short): head norms, rotation, cache write
             ops.linear_qkv(h, self.w_qkv, qkv, *dims, batch.positions, batch.slots,
                             q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.qk_norm_eps,
-                            rope_theta=None if rotary is None else rotary.theta,
-                            rope_dim=0 if rotary is None else rotary.rope_dim,
-                            rope_scale=1.0 if rotary is None else rotary.scale,
+                            rope_theta=None if rotation is None else rotation.theta,
+                            rope_dim=0 if rotation is None else rotation.rope_dim,
+                            rope_scale=1.0 if rotation is None else rotation.scale,
                             kv=write_to, longest_run=longest_run)
         else:
             # any other position encoding: norms, then the encoding, then the cache write

@@ -167,7 +167,22 @@ class Norm(Part):
         return None
 
 
+@dataclass(frozen=True)
+class HalfSplitRotation:
+    """What a position encoding says of itself when it rotates the pairs (i, i + rope_dim / 2) of every head of q and k by
+    the angle position * scale / theta[i]: theta is float32 [rope_dim / 2] on the device (None until the encoding is bound)."""
+    rope_dim: int
+    scale: float
+    theta: Optional[torch.Tensor]
+
+
 class PositionEncoding(Part):
+    def rotation(self) -> Optional[HalfSplitRotation]:
+        """An encoding that is such a rotation returns it; the mixer then lets the kernel that follows its q/k/v projection
+        rotate (fused into the projection where a step is short) and, when the rotation spans the whole head, keeps the two
+        rows of a pair side by side in the projection's packed weight. None: the mixer calls `apply`."""
+        return None
+
     def apply(self, qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, batch) -> None:
         """Encode the positions of the step's tokens into q and k, in place.
 

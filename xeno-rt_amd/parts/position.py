@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import PositionEncoding, Runtime, register_part
+from .base import HalfSplitRotation, PositionEncoding, Runtime, register_part
 
 
 class Rotary(PositionEncoding):
@@ -29,6 +29,9 @@ class Rotary(PositionEncoding):
         # float32 power, like the reference's powf (rope.rs:13)
         theta = torch.tensor(self.base, dtype=torch.float32) ** ((2.0 * pair) / float(self.rope_dim))
         self.theta = theta.to(runtime.device)
+
+    def rotation(self) -> HalfSplitRotation:
+        return HalfSplitRotation(self.rope_dim, self.scale, self.theta)
 
     def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch) -> None:
         self.runtime.ops.qkv_prepare(

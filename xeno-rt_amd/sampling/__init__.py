@@ -1,4 +1,4 @@
 """Sampling: greedy, temperature, top-k, top-p, repetition penalty."""
-from .sampler import GREEDY_BELOW, Sampler, SamplerConfig, TokenLog, uniform
+from .sampler import GREEDY_BELOW, Sampler, SamplerConfig, TokenLog, request_seed, uniform
 
-__all__ = ["GREEDY_BELOW", "Sampler", "SamplerConfig", "TokenLog", "uniform"]
+__all__ = ["GREEDY_BELOW", "Sampler", "SamplerConfig", "TokenLog", "request_seed", "uniform"]

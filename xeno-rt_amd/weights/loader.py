@@ -19,7 +19,8 @@ from __future__ import annotations
 
 import json
 import os
-from typing import Dict, Iterable, List
+import warnings
+from typing import Dict, Iterable, List, Optional
 
 import torch
 
@@ -117,19 +118,31 @@ def check_names(where: str, expected: Dict[str, WeightSpec], found: Dict[str, tu
         raise WeightError(where, missing, unexpected, wrong_shape, wrong_dtype)
 
 
+def warn_of_ignored(where: str, found: Iterable[str], ignored: Iterable[str]) -> None:
+    """A checkpoint may carry tensors that the model says it does not read (the head's matrix of a model
+    that ties it to the embedding, llama.rs:301-305): they are left alone, and said so once."""
+    present = sorted(set(ignored) & set(found))
+    if present:
+        warnings.warn(f"{where}: {', '.join(present)} ignored: the model does not read "
+                      f"{'it' if len(present) == 1 else 'them'} (a tied head uses the embedding's table)", stacklevel=3)
+
+
 class CheckpointSource:
     """The tensors of a model folder by name, each read when it is asked for (on the host, as stored).
 
-    The whole set of names, shapes and dtypes is checked against `expected` when the source is made."""
+    The whole set of names, shapes and dtypes is checked against `expected` when the source is made.
+    The files stay open (mapped) until `release()`: whoever has bound what it needs calls it; a tensor
+    asked for after that opens its file again for the one read."""
 
     def __init__(self, folder: str, expected: Dict[str, WeightSpec], ignored: Iterable[str] = ()):
         self.folder = folder
         self.expected = dict(expected)
-        self.files = CheckpointFiles(folder)
+        self.files: Optional[CheckpointFiles] = CheckpointFiles(folder)
         try:
             found = {name: (file.entries[name].dtype, file.entries[name].shape)
                      for name, file in self.files.where.items()}
             check_names(folder, self.expected, found, ignored)
+            warn_of_ignored(folder, found, ignored)
         except Exception:
             self.files.close()
             raise
@@ -143,13 +156,28 @@ class CheckpointSource:
     def __getitem__(self, name: str) -> torch.Tensor:
         if name not in self.expected:
             raise KeyError(name)
-        return _kept(self.files.where[name].read(name))
+        if self.files is not None:
+            return _kept(self.files.where[name].read(name))
+        files = CheckpointFiles(self.folder)            # released: open, read the one tensor, close
+        try:
+            return _kept(files.where[name].read(name))
+        finally:
+            files.close()
 
     def host(self, name: str) -> torch.Tensor:
         return self[name]
 
-    def close(self) -> None:
-        self.files.close()
+    @property
+    def is_open(self) -> bool:
+        return self.files is not None
+
+    def release(self) -> None:
+        """Close the files; tensors can still be asked for, one file opening each."""
+        if self.files is not None:
+            self.files.close()
+            self.files = None
+
+    close = release
 
 
 def load_tensors(folder: str, expected: Dict[str, WeightSpec], ignored: Iterable[str] = (),
@@ -160,6 +188,7 @@ def load_tensors(folder: str, expected: Dict[str, WeightSpec], ignored: Iterable
         found = {name: (file.entries[name].dtype, file.entries[name].shape)
                  for name, file in files.where.items()}
         check_names(folder, expected, found, ignored)
+        warn_of_ignored(folder, found, ignored)
         tensors = {}
         for name in expected:
             tensors[name] = _kept(files.where[name].read(name)).to(device)
