@@ -130,6 +130,173 @@ __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__
     }
 }
 
+// ---- few rows of a (a decode step), float32: the product is bound by reading w once, and the tile kernel above, which
+// multiplies a 16 x 64 tile through LDS in steps of 16 along k, reads it at a tenth of what the memory gives. Here a
+// workgroup of four wavefronts takes ROWS rows of w (gated: ROWS / 2 gate rows and the up rows of the same outputs) and
+// walks k in segments of 64 tiles of 16. In a segment lane t of every wavefront owns tile t: it loads 64 contiguous
+// bytes of each of its wavefront's rows (a wavefront's load is four contiguous kilobytes of a row, non-temporal), takes
+// the rows of a from LDS, where the segment was put once for all, and works out the tile's sum for every row of a:
+// the products of 16 consecutive k, added up in order. The tiles' sums then go through LDS to one thread per output,
+// which adds them to its running sum in the order of k. That is the order of the kernel above, term for term, so an
+// output has the same bits whichever kernel made it, and a token's result does not depend on the step it came in.
+constexpr int STREAM_ROWS = 16, STREAM_WAVES = 4, STREAM_TILES = 64, STREAM_HALF = 8;
+constexpr int STREAM_PITCH = STREAM_TILES + 1;        // of the tiles' sums of one output: the threads that add them up read down a column
+
+template <int MODE>
+__global__ void __launch_bounds__(STREAM_WAVES * XRT_WAVE) gemm_stream_kernel(
+    const float* __restrict__ a, const float* __restrict__ w, float* __restrict__ out, int M, int N, int K, int activation) {
+    constexpr int PER_WAVE = STREAM_ROWS / STREAM_WAVES;
+    constexpr int SEGMENT = STREAM_TILES * BK;                               // columns of k per segment
+    extern __shared__ __attribute__((aligned(16))) float stream_lds[];
+    float* a_segment = stream_lds;                                           // [rows of a][SEGMENT]
+    float* sums = stream_lds + (long)((M + 3) / 4 * 4) * SEGMENT;            // [STREAM_ROWS][STREAM_HALF][STREAM_PITCH]
+    const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
+    constexpr int OUTPUTS = MODE == MODE_GATED ? STREAM_ROWS / 2 : STREAM_ROWS;   // outputs per workgroup
+    const long n0 = (long)blockIdx.x * OUTPUTS;
+    // row of w behind row r of the workgroup's rows (gated: the gate rows of the outputs, then their up rows); clamped
+    // into the matrix, and what a clamped row makes is not written
+    auto w_row = [&](int r) -> long {
+        if constexpr (MODE == MODE_GATED) return min(n0 + r % OUTPUTS, (long)N - 1) + (long)(r / OUTPUTS) * N;
+        return min(n0 + r, (long)N - 1);
+    };
+    const float* rows[PER_WAVE];
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) rows[i] = w + w_row(wave * PER_WAVE + i) * K;
+    // the thread that adds up the sums of output row `mine_r`, row `mine_m` of a half of a's rows
+    const int mine_r = tid / STREAM_HALF, mine_m = tid % STREAM_HALF;
+    const bool adds = mine_r < STREAM_ROWS;
+    float running[2] = {0.f, 0.f};                                           // one per half of a's rows
+    typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+    // this lane's tile of each of its wavefront's rows of w in a segment: zeros beyond K, as the kernel above pads its
+    // last tile. The next segment's tiles are asked for before this segment's sums are worked out.
+    floatx4 ahead[PER_WAVE][BK / 4];
+    auto ask = [&](int k0) {
+        const int columns = min(SEGMENT, K - k0);
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i)
+#pragma unroll
+            for (int q = 0; q < BK / 4; ++q) {
+                const int k = lane * BK + q * 4;
+                ahead[i][q] = floatx4{0.f, 0.f, 0.f, 0.f};
+                if (k < columns) ahead[i][q] = *reinterpret_cast<const floatx4*>(rows[i] + k0 + k);
+            }
+    };
+    ask(0);
+    for (int k0 = 0; k0 < K; k0 += SEGMENT) {
+        const int columns = min(SEGMENT, K - k0);                            // a multiple of 4: the launcher checks
+        const int tiles = (columns + BK - 1) / BK;
+        float wv[PER_WAVE][BK];
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i)
+#pragma unroll
+            for (int q = 0; q < BK / 4; ++q) {
+                const floatx4 v = ahead[i][q];
+                wv[i][q * 4] = v[0]; wv[i][q * 4 + 1] = v[1]; wv[i][q * 4 + 2] = v[2]; wv[i][q * 4 + 3] = v[3];
+            }
+        if (k0 + SEGMENT < K) ask(k0 + SEGMENT);
+        // the segment of a, for all wavefronts: the q-th 16 bytes of tile t of row m lie at [m][q][t], so that the lanes
+        // of a wavefront, which read the same q of neighbouring tiles, read neighbouring places
+        for (int piece = tid; piece < M * (SEGMENT / 4); piece += STREAM_WAVES * XRT_WAVE) {
+            const int m = piece / (SEGMENT / 4), within = piece % (SEGMENT / 4), k = within * 4;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (k < columns) v = *reinterpret_cast<const floatx4*>(a + (long)m * K + k0 + k);
+            *reinterpret_cast<floatx4*>(a_segment + (((long)m * (BK / 4) + within % (BK / 4)) * STREAM_TILES + within / (BK / 4)) * 4) = v;
+        }
+        __syncthreads();
+        for (int half = 0; half * STREAM_HALF < M; ++half) {
+            const int m_count = min(STREAM_HALF, M - half * STREAM_HALF);
+            // the tile's sums: the products of its 16 columns in order, from zero (fmaf as in the kernel above)
+            // (two rows of a at a time, so that eight chains of products run side by side; an odd last row is done twice)
+            for (int m0 = 0; m0 < m_count; m0 += 2) {
+                float av[2][BK];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const float* am = a_segment + (long)(half * STREAM_HALF + min(m0 + u, m_count - 1)) * SEGMENT + lane * 4;
+#pragma unroll
+                    for (int q = 0; q < BK / 4; ++q) {
+                        const floatx4 v = *reinterpret_cast<const floatx4*>(am + q * STREAM_TILES * 4);
+                        av[u][q * 4] = v[0]; av[u][q * 4 + 1] = v[1]; av[u][q * 4 + 2] = v[2]; av[u][q * 4 + 3] = v[3];
+                    }
+                }
+                float part[2][PER_WAVE];
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int i = 0; i < PER_WAVE; ++i) part[u][i] = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < BK; ++kk)
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int i = 0; i < PER_WAVE; ++i) part[u][i] = fmaf(av[u][kk], wv[i][kk], part[u][i]);
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int i = 0; i < PER_WAVE; ++i)
+                        sums[((wave * PER_WAVE + i) * STREAM_HALF + min(m0 + u, m_count - 1)) * STREAM_PITCH + lane] = part[u][i];
+            }
+            __syncthreads();
+            if (adds && mine_m < m_count) {
+                // all tiles' sums are asked for at once, then added in the order of k (those beyond K are not)
+                const float* mine = sums + (mine_r * STREAM_HALF + mine_m) * STREAM_PITCH;
+                float of_tile[STREAM_TILES];
+#pragma unroll
+                for (int t = 0; t < STREAM_TILES; ++t) of_tile[t] = mine[t];
+                float sum = running[half];
+#pragma unroll
+                for (int t = 0; t < STREAM_TILES; ++t) sum = t < tiles ? sum + of_tile[t] : sum;
+                running[half] = sum;
+            }
+            __syncthreads();
+        }
+    }
+    // ---- epilogue: thread (mine_r, mine_m) holds output row mine_r for rows mine_m and mine_m + 8 of a
+    if constexpr (MODE == MODE_GATED) {
+        // the up sums go to the threads that hold the gate sums of the same outputs
+        if (adds && mine_r >= OUTPUTS) { sums[(mine_r * STREAM_HALF + mine_m) * 2] = running[0]; sums[(mine_r * STREAM_HALF + mine_m) * 2 + 1] = running[1]; }
+        __syncthreads();
+    }
+    if (!adds || mine_r >= OUTPUTS || n0 + mine_r >= N) return;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int m = half * STREAM_HALF + mine_m;
+        if (m >= M) continue;
+        float* dst = out + (long)m * N + n0 + mine_r;
+        if constexpr (MODE == MODE_STORE) *dst = running[half];
+        if constexpr (MODE == MODE_ACCUMULATE) *dst = *dst + running[half];
+        if constexpr (MODE == MODE_GATED) *dst = gate_activation(running[half], activation) * sums[((mine_r + OUTPUTS) * STREAM_HALF + mine_m) * 2 + half];
+    }
+}
+
+// Whether the kernel above takes the product: float32, up to 16 rows of a, whole pieces of 16 bytes.
+bool stream_takes(const void* a, const void* w, int M, int K) {
+    return M >= 1 && M <= 2 * STREAM_HALF && K % 4 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
+}
+
+int launch_stream(const float* a, const float* w, float* out, int M, int N, int K, int mode, int activation, hipStream_t s) {
+    const int outputs = mode == MODE_GATED ? STREAM_ROWS / 2 : STREAM_ROWS;
+    const unsigned grid = (unsigned)((N + outputs - 1) / outputs);
+    const size_t lds = ((size_t)((M + 3) / 4 * 4) * STREAM_TILES * BK + (size_t)STREAM_ROWS * STREAM_HALF * STREAM_PITCH) * sizeof(float);
+#define XRT_STREAM(MODE_)                                                                                                    \
+    do {                                                                                                                     \
+        static bool configured = false;                                                                                      \
+        if (!configured) {                                                                                                   \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_stream_kernel<MODE_>),                     \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);                      \
+            XRT_REQUIRE(e == hipSuccess, "linear (plain, few rows): cannot reserve LDS: %s", hipGetErrorString(e));          \
+            configured = true;                                                                                               \
+        }                                                                                                                    \
+        gemm_stream_kernel<MODE_><<<grid, STREAM_WAVES * XRT_WAVE, lds, s>>>(a, w, out, M, N, K, activation);                \
+    } while (0)
+    if (mode == MODE_STORE) XRT_STREAM(MODE_STORE);
+    else if (mode == MODE_ACCUMULATE) XRT_STREAM(MODE_ACCUMULATE);
+    else XRT_STREAM(MODE_GATED);
+#undef XRT_STREAM
+    XRT_LAUNCH_CHECK("linear (plain, few rows)");
+    return 0;
+}
+
 template <typename TI, typename TO, int RM>
 void launch_rows(const void* a, const void* w, void* out, int M, int N, int K, int mode, int activation, hipStream_t s) {
     constexpr int BM = 16 * RM;
@@ -155,6 +322,8 @@ int launch(const void* a, const void* w, void* out, int M, int N, int K, int mod
 
 int xrt_linear_plain(const void* a, const void* w, int dtype, void* out, int out_dtype, int M, int N, int K,
                      int mode, int activation, hipStream_t s) {
+    if (dtype == XRT_F32 && out_dtype == XRT_F32 && stream_takes(a, w, M, K))
+        return launch_stream((const float*)a, (const float*)w, (float*)out, M, N, K, mode, activation, s);
     if (dtype == XRT_F32 && out_dtype == XRT_F32) return launch<float, float>(a, w, out, M, N, K, mode, activation, s);
     if (dtype == XRT_BF16 && out_dtype == XRT_F32) return launch<bf16, float>(a, w, out, M, N, K, mode, activation, s);
     if (dtype == XRT_BF16 && out_dtype == XRT_BF16) return launch<bf16, bf16>(a, w, out, M, N, K, mode, activation, s);
