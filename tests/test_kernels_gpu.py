@@ -550,6 +550,38 @@ def test_attention(ops, dtype, nh, nkv, hd):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 48, None), (8, 2, 128, None), (2, 1, 100, None), (4, 4, 32, 700)])
+def test_general_attention_gives_the_same_bits_with_few_tokens_and_with_many(ops, dtype, nh, nkv, hd, window):
+    """The general kernel takes a step of few tokens with a workgroup of wavefronts per (token, head), which work the
+    chunks of keys off side by side, and a step of many tokens with one wavefront each, which takes the chunks one after
+    the other: the same sums in the same order. Sequences of one, two and six chunks of 512 keys, some ending inside a
+    chunk; the same queries alone and among 3000 others."""
+    lengths = [3000, 513, 512, 70, 1025]
+    kv, keys, values = filled_cache(nkv, hd, DT[dtype], lengths, seed=hd)
+    slots = [0, 1, 2, 3, 4, 0, 0, 4]
+    positions = [2999, 512, 511, 69, 1024, 1536, 600, 1023]
+    few = rand(len(slots), (nh + 2 * nkv) * hd, dtype=DT[dtype], seed=7)
+    out_few = torch.empty(len(slots), nh * hd, dtype=DT[dtype], device=DEV)
+    ops.attention(few, nh, nkv, hd, kv, SimpleNamespace(slots=i32(slots), positions=i32(positions)), out_few,
+                  scale=1.0 / math.sqrt(hd), window=window)
+    crowd = 3000                                               # other tokens of the step: early positions of sequence 0
+    many = torch.cat([rand(crowd, (nh + 2 * nkv) * hd, dtype=DT[dtype], seed=8), few])
+    out_many = torch.empty(crowd + len(slots), nh * hd, dtype=DT[dtype], device=DEV)
+    batch = SimpleNamespace(slots=i32([0] * crowd + slots), positions=i32([t % 64 for t in range(crowd)] + positions))
+    ops.attention(many, nh, nkv, hd, kv, batch, out_many, scale=1.0 / math.sqrt(hd), window=window)
+    assert torch.isfinite(out_few).all()
+    assert torch.equal(out_many[crowd:], out_few)
+    for t, (slot, pos) in enumerate(zip(slots, positions)):    # and both are the plain attention's
+        if window is not None:
+            continue
+        q = few[t:t + 1, :nh * hd].double().cpu()
+        k = keys[slot][:pos + 1].reshape(pos + 1, nkv * hd).double().cpu()
+        v = values[slot][:pos + 1].reshape(pos + 1, nkv * hd).double().cpu()
+        want = P.causal_attention(q, k, v, nh, nkv, hd, start_position=pos)
+        assert rel(out_few[t:t + 1].cpu(), want) < (2e-5 if dtype == "float32" else 1e-2), (t, slot, pos)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_attention_finds_a_far_key(ops, dtype):
     """One key among 900 matches the query: the output must be that key's value, wherever it lies."""
     nh, nkv, hd = 4, 2, 64
