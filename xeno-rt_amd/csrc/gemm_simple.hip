@@ -134,8 +134,8 @@ __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__
 // multiplies a 16 x 64 tile through LDS in steps of 16 along k, reads it at a tenth of what the memory gives. Here a
 // workgroup of four wavefronts takes ROWS rows of w (gated: ROWS / 2 gate rows and the up rows of the same outputs) and
 // walks k in segments of 64 tiles of 16. In a segment lane t of every wavefront owns tile t: it loads 64 contiguous
-// bytes of each of its wavefront's rows (a wavefront's load is four contiguous kilobytes of a row, non-temporal), takes
-// the rows of a from LDS, where the segment was put once for all, and works out the tile's sum for every row of a:
+// bytes of each of its wavefront's rows (a wavefront's load is four contiguous kilobytes of a row), takes the rows of a,
+// eight at a time, from LDS, where their segment was put once for all, and works out the tile's sum for every row of a:
 // the products of 16 consecutive k, added up in order. The tiles' sums then go through LDS to one thread per output,
 // which adds them to its running sum in the order of k. That is the order of the kernel above, term for term, so an
 // output has the same bits whichever kernel made it, and a token's result does not depend on the step it came in.
@@ -148,8 +148,8 @@ __global__ void __launch_bounds__(STREAM_WAVES * XRT_WAVE) gemm_stream_kernel(
     constexpr int PER_WAVE = STREAM_ROWS / STREAM_WAVES;
     constexpr int SEGMENT = STREAM_TILES * BK;                               // columns of k per segment
     extern __shared__ __attribute__((aligned(16))) float stream_lds[];
-    float* a_segment = stream_lds;                                           // [rows of a][SEGMENT]
-    float* sums = stream_lds + (long)((M + 3) / 4 * 4) * SEGMENT;            // [STREAM_ROWS][STREAM_HALF][STREAM_PITCH]
+    float* a_segment = stream_lds;                                           // [STREAM_HALF rows of a][SEGMENT]
+    float* sums = stream_lds + (long)STREAM_HALF * SEGMENT;                  // [STREAM_ROWS][STREAM_HALF][STREAM_PITCH]
     const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
     constexpr int OUTPUTS = MODE == MODE_GATED ? STREAM_ROWS / 2 : STREAM_ROWS;   // outputs per workgroup
     const long n0 = (long)blockIdx.x * OUTPUTS;
@@ -195,24 +195,24 @@ __global__ void __launch_bounds__(STREAM_WAVES * XRT_WAVE) gemm_stream_kernel(
                 wv[i][q * 4] = v[0]; wv[i][q * 4 + 1] = v[1]; wv[i][q * 4 + 2] = v[2]; wv[i][q * 4 + 3] = v[3];
             }
         if (k0 + SEGMENT < K) ask(k0 + SEGMENT);
-        // the segment of a, for all wavefronts: the q-th 16 bytes of tile t of row m lie at [m][q][t], so that the lanes
-        // of a wavefront, which read the same q of neighbouring tiles, read neighbouring places
-        for (int piece = tid; piece < M * (SEGMENT / 4); piece += STREAM_WAVES * XRT_WAVE) {
-            const int m = piece / (SEGMENT / 4), within = piece % (SEGMENT / 4), k = within * 4;
-            floatx4 v = {0.f, 0.f, 0.f, 0.f};
-            if (k < columns) v = *reinterpret_cast<const floatx4*>(a + (long)m * K + k0 + k);
-            *reinterpret_cast<floatx4*>(a_segment + (((long)m * (BK / 4) + within % (BK / 4)) * STREAM_TILES + within / (BK / 4)) * 4) = v;
-        }
-        __syncthreads();
         for (int half = 0; half * STREAM_HALF < M; ++half) {
             const int m_count = min(STREAM_HALF, M - half * STREAM_HALF);
+            // the segment of this half of a's rows, for all wavefronts: the q-th 16 bytes of tile t of row m lie at [m][q][t],
+            // so that the lanes of a wavefront, which read the same q of neighbouring tiles, read neighbouring places
+            for (int piece = tid; piece < m_count * (SEGMENT / 4); piece += STREAM_WAVES * XRT_WAVE) {
+                const int m = piece / (SEGMENT / 4), within = piece % (SEGMENT / 4), k = within * 4;
+                floatx4 v = {0.f, 0.f, 0.f, 0.f};
+                if (k < columns) v = *reinterpret_cast<const floatx4*>(a + (long)(half * STREAM_HALF + m) * K + k0 + k);
+                *reinterpret_cast<floatx4*>(a_segment + (((long)m * (BK / 4) + within % (BK / 4)) * STREAM_TILES + within / (BK / 4)) * 4) = v;
+            }
+            __syncthreads();
             // the tile's sums: the products of its 16 columns in order, from zero (fmaf as in the kernel above)
             // (two rows of a at a time, so that eight chains of products run side by side; an odd last row is done twice)
             for (int m0 = 0; m0 < m_count; m0 += 2) {
                 float av[2][BK];
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
-                    const float* am = a_segment + (long)(half * STREAM_HALF + min(m0 + u, m_count - 1)) * SEGMENT + lane * 4;
+                    const float* am = a_segment + (long)min(m0 + u, m_count - 1) * SEGMENT + lane * 4;
 #pragma unroll
                     for (int q = 0; q < BK / 4; ++q) {
                         const floatx4 v = *reinterpret_cast<const floatx4*>(am + q * STREAM_TILES * 4);
@@ -277,13 +277,13 @@ bool stream_takes(const void* a, const void* w, int M, int K) {
 int launch_stream(const float* a, const float* w, float* out, int M, int N, int K, int mode, int activation, hipStream_t s) {
     const int outputs = mode == MODE_GATED ? STREAM_ROWS / 2 : STREAM_ROWS;
     const unsigned grid = (unsigned)((N + outputs - 1) / outputs);
-    const size_t lds = ((size_t)((M + 3) / 4 * 4) * STREAM_TILES * BK + (size_t)STREAM_ROWS * STREAM_HALF * STREAM_PITCH) * sizeof(float);
+    const size_t lds = ((size_t)STREAM_HALF * STREAM_TILES * BK + (size_t)STREAM_ROWS * STREAM_HALF * STREAM_PITCH) * sizeof(float);
 #define XRT_STREAM(MODE_)                                                                                                    \
     do {                                                                                                                     \
         static bool configured = false;                                                                                      \
         if (!configured) {                                                                                                   \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_stream_kernel<MODE_>),                     \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);                      \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                      \
             XRT_REQUIRE(e == hipSuccess, "linear (plain, few rows): cannot reserve LDS: %s", hipGetErrorString(e));          \
             configured = true;                                                                                               \
         }                                                                                                                    \
