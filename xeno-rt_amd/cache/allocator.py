@@ -7,8 +7,9 @@ giving something back twice, is an error and never silent.
 """
 from __future__ import annotations
 
-import heapq
-from typing import List
+import ctypes
+
+from ..host import ERROR, FULL, OK, last_error, load_host
 
 BLOCK_TOKENS = 64   # tokens per block: the unit in which live requests hold cache (the kernel library is asked for its own
                     # number when it is loaded, and refused if that differs)
@@ -22,53 +23,57 @@ class CacheError(RuntimeError):
     """A slot or block was used in a way its state does not allow."""
 
 
-class Pool:
-    """`size` numbered items; the lowest free one is handed out, released ones are used again."""
+def raise_for(status: int) -> None:
+    """The host library's verdict as an exception, with its message."""
+    if status == FULL:
+        raise CacheFull(last_error())
+    if status != OK:
+        raise CacheError(last_error())
 
-    def __init__(self, size: int, what: str):
+
+class Pool:
+    """`size` numbered items; the lowest free one is handed out, released ones are used again.
+    The bookkeeping is the host library's (csrc/host/xrt_host.cpp); `handle` may name a pool that
+    someone else owns (the blocks of a group's tables)."""
+
+    def __init__(self, size: int, what: str, handle=None):
         if size < 0:
             raise ValueError(f"pool of {what}s needs a non-negative size")
+        self._lib = load_host()
         self.size = size
         self.what = what
-        self._free: List[int] = list(range(size))               # a heap: the lowest number on top
-        self._held = [False] * size
+        self._owned = handle is None
+        self._handle = self._lib.xrt_pool_new(size, what.encode()) if handle is None else handle
+        if not self._handle:
+            raise CacheError(last_error())
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and getattr(self, "_handle", None):
+            self._lib.xrt_pool_delete(self._handle)
+            self._handle = None
 
     @property
     def n_free(self) -> int:
-        return len(self._free)
+        return int(self._lib.xrt_pool_n_free(self._handle))
 
     @property
     def n_held(self) -> int:
-        return self.size - len(self._free)
+        return self.size - self.n_free
 
     def is_held(self, item: int) -> bool:
-        return 0 <= item < self.size and self._held[item]
+        return bool(self._lib.xrt_pool_is_held(self._handle, int(item)))
 
     def acquire(self) -> int:
-        if not self._free:
-            raise CacheFull(f"no free {self.what} (all {self.size} are in use)")
-        item = heapq.heappop(self._free)
-        if self._held[item]:
-            raise CacheError(f"{self.what} {item} was on the free list while held")
-        self._held[item] = True
-        return item
+        item = ctypes.c_int(-1)
+        raise_for(self._lib.xrt_pool_acquire(self._handle, ctypes.byref(item)))
+        return item.value
 
     def release(self, item: int) -> None:
-        if not 0 <= item < self.size:
-            raise CacheError(f"{self.what} {item} does not exist (pool of {self.size})")
-        if not self._held[item]:
-            raise CacheError(f"{self.what} {item} is released twice or was never acquired")
-        self._held[item] = False
-        heapq.heappush(self._free, item)
+        raise_for(self._lib.xrt_pool_release(self._handle, int(item)))
 
     def check(self) -> None:
         """Every item is either free once or held; raises CacheError otherwise."""
-        free = set(self._free)
-        if len(free) != len(self._free):
-            raise CacheError(f"a {self.what} is on the free list twice")
-        for item in range(self.size):
-            if self._held[item] == (item in free):
-                raise CacheError(f"{self.what} {item} is " + ("both held and free" if self._held[item] else "lost"))
+        raise_for(self._lib.xrt_pool_check(self._handle))
 
 
 def blocks_for(tokens: int) -> int:

@@ -18,6 +18,7 @@ rollback (kv_cache.rs:159-168).
 """
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass
 from typing import Dict, List, Optional
 
@@ -27,7 +28,8 @@ import torch
 from ..staging import staging_for
 
 from ..parts.base import CacheNeeds, KVSpec
-from .allocator import BLOCK_TOKENS, CacheError, CacheFull, Pool, blocks_for
+from ..host import last_error, load_host
+from .allocator import BLOCK_TOKENS, CacheError, CacheFull, Pool, blocks_for, raise_for
 
 
 @dataclass
@@ -47,32 +49,44 @@ class LayerCache:
 
 
 class KVGroup:
-    """Storage and block accounting of the layer calls that share one KVSpec."""
+    """Storage and block accounting of the layer calls that share one KVSpec. Which blocks a sequence holds is kept
+    by the host library (csrc/host/xrt_host.cpp), which writes the table that lies here; the device's copy of
+    the table is refreshed from it before a step."""
 
     def __init__(self, spec: KVSpec, calls: List[int], n_blocks: int, max_slots: int,
                  max_blocks_per_sequence: int, dtype: torch.dtype, device):
         self.spec = spec
         self.calls = calls
-        self.pool = Pool(n_blocks, "block")
         self.max_blocks_per_sequence = max_blocks_per_sequence
-        # host table: the truth (numpy, so that single entries are cheap to touch; the torch view
-        # shares its memory); device table: what kernels read, refreshed before a step
+        self.max_slots = max_slots
+        # host table: the truth (the torch view shares the array's memory); device table: what kernels read
         self._table = np.full((max_slots, max_blocks_per_sequence), -1, dtype=np.int32)
         self.table = torch.from_numpy(self._table)
         self.device_table = self.table.to(device)
-        self._changed = set()              # slots whose row of the table the device has not seen yet
-        self._end: Dict[int, int] = {}     # slot -> logical blocks [floor, end) may be held
-        self._floor: Dict[int, int] = {}   # slot -> lowest logical block it may still hold
+        self._lib = load_host()
+        self._handle = self._lib.xrt_tables_new(n_blocks, max_slots, max_blocks_per_sequence, int(spec.window or 0),
+                                                BLOCK_TOKENS, self._table.ctypes.data)
+        if not self._handle:
+            raise CacheError(last_error())
+        self.pool = Pool(n_blocks, "block", handle=self._lib.xrt_tables_pool(self._handle))
+        self._added = (ctypes.c_int * max(1, max_blocks_per_sequence))()
         shape_k = (len(calls), n_blocks, spec.n_kv_heads, BLOCK_TOKENS, spec.head_dim)
         shape_v = (len(calls), n_blocks, spec.n_kv_heads, spec.value_width, BLOCK_TOKENS)
         self.k = torch.zeros(shape_k, dtype=dtype, device=device)
         self.v = torch.zeros(shape_v, dtype=dtype, device=device)
 
+    def __del__(self):
+        if getattr(self, "_handle", None):
+            self._lib.xrt_tables_delete(self._handle)
+            self._handle = None
+
     def first_needed_block(self, length: int) -> int:
         """Lowest logical block that a query at position >= length can still see."""
-        if self.spec.window is None:
-            return 0
-        return max(0, length + 1 - self.spec.window) // BLOCK_TOKENS
+        return int(self._lib.xrt_tables_first_needed_block(self._handle, int(length)))
+
+    def floor(self, slot: int) -> int:
+        """Lowest logical block that the sequence may still hold (a window lets go of those below)."""
+        return int(self._lib.xrt_tables_floor(self._handle, int(slot)))
 
     def held(self, slot: int) -> List[int]:
         row = self._table[slot]
@@ -80,56 +94,35 @@ class KVGroup:
 
     def grow(self, slot: int, new_length: int) -> List[int]:
         """Acquire the blocks that tokens up to new_length need; returns the logical indices added."""
-        need = blocks_for(new_length)
-        if need > self.max_blocks_per_sequence:
-            raise CacheError(f"sequence of {new_length} tokens exceeds the cache's limit per sequence")
-        start = max(self._end.get(slot, 0), self._floor.get(slot, 0))
-        added = []
-        try:
-            for logical in range(start, need):
-                self._table[slot, logical] = self.pool.acquire()
-                added.append(logical)
-        except CacheFull:
-            self.drop(slot, added)
-            raise
-        if added:
-            self._end[slot] = need
-            self._changed.add(slot)
-        return added
+        count = ctypes.c_int(0)
+        raise_for(self._lib.xrt_tables_grow(self._handle, int(slot), int(new_length), self._added, ctypes.byref(count)))
+        return list(self._added[:count.value])
 
     def drop(self, slot: int, logicals: List[int]) -> None:
-        for logical in logicals:
-            self.pool.release(int(self._table[slot, logical]))
-            self._table[slot, logical] = -1
         if logicals:
-            self._changed.add(slot)
-            end = self._end.get(slot, 0)
-            while end > 0 and self._table[slot, end - 1] < 0:
-                end -= 1
-            self._end[slot] = end
+            array = (ctypes.c_int * len(logicals))(*logicals)
+            raise_for(self._lib.xrt_tables_drop(self._handle, int(slot), array, len(logicals)))
 
     def shrink_to(self, slot: int, length: int) -> None:
         """Release what a sequence of `length` tokens no longer needs: blocks past its end,
         and blocks that have slid out of the window."""
-        end = self._end.get(slot, 0)
-        past_end = [l for l in range(blocks_for(length), end) if self._table[slot, l] >= 0]
-        floor = self.first_needed_block(length)
-        below = [l for l in range(self._floor.get(slot, 0), min(floor, end)) if self._table[slot, l] >= 0]
-        self._floor[slot] = floor
-        self.drop(slot, past_end + below)
+        raise_for(self._lib.xrt_tables_shrink_to(self._handle, int(slot), int(length)))
 
     def release_all(self, slot: int) -> None:
-        self.drop(slot, [l for l in range(self._end.get(slot, 0)) if self._table[slot, l] >= 0])
-        self._floor.pop(slot, None)
-        self._end.pop(slot, None)
+        raise_for(self._lib.xrt_tables_release_all(self._handle, int(slot)))
+
+    def check(self, slot_held) -> None:
+        """No block held by two sequences or by none; free slots hold nothing."""
+        flags = (ctypes.c_ubyte * self.max_slots)(*[1 if held else 0 for held in slot_held])
+        raise_for(self._lib.xrt_tables_check(self._handle, flags))
 
     def sync(self) -> None:
         """The rows that changed go to the device through pinned memory, in the order of the stream and
         without waiting for it: a host that prepares the next step while this one runs is not held up."""
-        if self._changed:
-            low, high = min(self._changed), max(self._changed) + 1
-            staging_for(self.device_table.device).upload(self.table[low:high], out=self.device_table[low:high])
-            self._changed.clear()
+        low, high = ctypes.c_int(0), ctypes.c_int(0)
+        self._lib.xrt_tables_take_changed(self._handle, ctypes.byref(low), ctypes.byref(high))
+        if high.value > low.value:
+            staging_for(self.device_table.device).upload(self.table[low.value:high.value], out=self.device_table[low.value:high.value])
 
 
 class SequenceCache:
@@ -239,9 +232,9 @@ class SequenceCache:
             raise CacheError("a cache with per-sequence state cannot be truncated")
         for group in self.groups:
             # a window has let go of the blocks below its floor: a shorter sequence that would look there again cannot be had
-            if group.spec.window is not None and group.first_needed_block(length) < group._floor.get(slot, 0):
+            if group.spec.window is not None and group.first_needed_block(length) < group.floor(slot):
                 raise CacheError(f"slot {slot}: cannot truncate to {length} tokens: a window of {group.spec.window} has "
-                                 f"released the keys before {group._floor[slot] * BLOCK_TOKENS}, which a query there would see")
+                                 f"released the keys before {group.floor(slot) * BLOCK_TOKENS}, which a query there would see")
         self.lengths[slot] = length
         for group in self.groups:
             group.shrink_to(slot, length)
@@ -268,18 +261,6 @@ class SequenceCache:
     def check(self) -> None:
         """Invariants: no slot or block lost or held twice; free slots hold nothing."""
         self.slots.check()
+        held = [self.slots.is_held(slot) for slot in range(self.max_slots)]
         for group in self.groups:
-            group.pool.check()
-            seen = set()
-            for slot in range(self.max_slots):
-                held = group.held(slot)
-                if not self.slots.is_held(slot) and held:
-                    raise CacheError(f"free slot {slot} still holds blocks {held}")
-                for block in held:
-                    if block in seen:
-                        raise CacheError(f"block {block} is held by two sequences")
-                    if not group.pool.is_held(block):
-                        raise CacheError(f"block {block} is in a table but free in the pool")
-                    seen.add(block)
-            if len(seen) != group.pool.n_held:
-                raise CacheError(f"{group.pool.n_held - len(seen)} blocks are held by no sequence")
+            group.check(held)

@@ -13,15 +13,17 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..cache import BLOCK_TOKENS, CacheError, CacheFull, SequenceCache
 from ..config import architecture, load_config
+from ..host import last_error, load_host
 from ..models import DecoderModel, ModelSpec
 from ..parts.base import Runtime
 from ..weights import CheckpointSource, RandomSource
 from ..staging import staging_for
-from .batch import build_batch
+from .batch import build_batch, flatten
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
            "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32}
@@ -199,31 +201,27 @@ class Engine:
         if len(entries) == 0:
             raise StepError("a step needs at least one sequence")
         slots, tokens, wants, starts = [], [], [], []
-        seen = set()
         for slot, ids, want in entries:
-            ids = list(ids)
-            want = list(want)
-            if slot in seen:
-                raise StepError(f"slot {slot} appears twice in one step")
-            seen.add(slot)
             if not self.cache.slots.is_held(slot):
                 raise StepError(f"slot {slot} is not allocated")
-            if len(ids) == 0:                                   # llama.rs:624-626
-                raise StepError(f"slot {slot}: a step needs at least one token per sequence")
-            for token in ids:                                   # llama.rs:1044-1049
-                if not 0 <= int(token) < self.vocab_size:
-                    raise StepError(f"slot {slot}: token id {token} exceeds embedding rows {self.vocab_size}")
-            for index in want:
-                if not 0 <= int(index) < len(ids):
-                    raise StepError(f"slot {slot}: wanted index {index} is outside the {len(ids)} tokens given")
-            start = self.cache.length(slot)
-            if start + len(ids) > self.cache.max_context:
-                raise StepError(f"slot {slot}: {start} + {len(ids)} tokens exceed the context limit "
-                                f"{self.cache.max_context}")
-            slots.append(slot)
-            tokens.append(ids)
-            wants.append(want)
-            starts.append(start)
+            slots.append(int(slot))
+            tokens.append(list(ids))
+            wants.append(list(want))
+            starts.append(self.cache.length(slot))
+        # the rest of the checks are the host library's (no slot twice, a token at least, ids below the embedding's
+        # rows, wanted places inside the tokens given, the context limit): one call for the whole step
+        try:
+            counts, flat_tokens = flatten(tokens)
+            want_counts, flat_wants = flatten(wants)
+        except (OverflowError, ValueError, TypeError):
+            raise StepError("token ids and wanted places must be integers that fit 32 bits") from None
+        host = load_host()
+        as_array = lambda values: np.ascontiguousarray(values, dtype=np.int32)
+        slot_array, start_array = as_array(slots), as_array(starts)
+        if host.xrt_step_check(len(slots), slot_array.ctypes.data, counts.ctypes.data, start_array.ctypes.data,
+                               flat_tokens.ctypes.data, want_counts.ctypes.data, flat_wants.ctypes.data,
+                               int(self.vocab_size), int(self.cache.max_context)) != 0:
+            raise StepError(last_error())
         reserved = []
         try:
             for slot, ids, start in zip(slots, tokens, starts):

@@ -15,10 +15,12 @@ they can be tested without one.
 """
 from __future__ import annotations
 
+import ctypes
 import random
 from dataclasses import dataclass, field
 from typing import Callable, List, Optional, Sequence
 
+from ..host import FINISH_REASONS, last_error, load_host
 from ..sampling import SamplerConfig, uniform
 
 
@@ -76,20 +78,19 @@ def decide(token: int, stops, history_length: int, context: int, produced: int, 
     Order of the reference's loop body (session.rs:116-124): stop token first, then
     full context, then the token is kept; the loop condition (:115) ends the request
     once max_tokens are kept, which here also spares the forward pass of the last token.
+    The decision is the host library's (csrc/host/xrt_host.cpp: xrt_loop_decide).
     """
-    if token in stops:
-        return False, "stop"
-    if history_length >= context:
-        return False, "context"
-    if produced + 1 >= max_tokens:
-        return True, "length"
-    return True, None
+    stop_array = (ctypes.c_int * max(1, len(stops)))(*sorted(stops))
+    keep = ctypes.c_int(0)
+    reason = load_host().xrt_loop_decide(int(token), stop_array, len(stops), int(history_length), int(context),
+                                         int(produced), int(max_tokens), ctypes.byref(keep))
+    return bool(keep.value), FINISH_REASONS[reason]
 
 
 def goes_on_whatever_it_draws(history_length: int, context: int, produced: int, max_tokens: int) -> bool:
     """Whether only a stop token can end the request at the token being sampled: then its next step may
     start before the token has been looked at. The same conditions as in `decide` and in the loop below."""
-    return history_length + 1 < context and produced + 1 < max_tokens
+    return bool(load_host().xrt_loop_goes_on_whatever_it_draws(int(history_length), int(context), int(produced), int(max_tokens)))
 
 
 def plan_batches(prompt_lengths: Sequence[int], max_tokens: Sequence[int], batch_size: int,
@@ -97,21 +98,17 @@ def plan_batches(prompt_lengths: Sequence[int], max_tokens: Sequence[int], batch
     """Cut the requests, in order, into batches that fit the slots and the cache.
 
     A request may come to hold min(context, prompt + max_tokens) tokens, rounded up to blocks."""
-    batches: List[List[int]] = []
-    current: List[int] = []
-    used = 0
-    for index, (length, limit) in enumerate(zip(prompt_lengths, max_tokens)):
-        final = min(context, length + max(0, limit))
-        need = -(-final // block_tokens) * block_tokens
-        if need > cache_tokens:
-            raise ValueError(f"request {index} may hold {need} tokens; the cache holds {cache_tokens}")
-        if current and (len(current) >= batch_size or used + need > cache_tokens):
-            batches.append(current)
-            current, used = [], 0
-        current.append(index)
-        used += need
-    if current:
-        batches.append(current)
+    n = len(prompt_lengths)
+    lengths = (ctypes.c_int * max(1, n))(*[int(v) for v in prompt_lengths])
+    limits = (ctypes.c_int * max(1, n))(*[int(v) for v in max_tokens])
+    batch_of = (ctypes.c_int * max(1, n))()
+    count = load_host().xrt_loop_plan_batches(n, lengths, limits, int(batch_size), int(block_tokens), int(cache_tokens),
+                                              int(context), batch_of)
+    if count < 0:
+        raise ValueError(last_error())
+    batches: List[List[int]] = [[] for _ in range(count)]
+    for index in range(n):
+        batches[batch_of[index]].append(index)
     return batches
 
 

@@ -19,7 +19,7 @@ from typing import Dict, List, Sequence, Tuple
 import torch
 
 from ..staging import staging_for
-from .batch import StepBatch
+from .batch import StepBatch, pack_step
 
 CONTEXT_BUCKET = 1024    # a recorded step serves contexts up to the next multiple of this (the decode attention cuts its keys by it)
 MAX_GRAPHS = 32          # recorded steps kept at a time
@@ -77,10 +77,11 @@ class DecodeGraph:
         size, count = self.size, len(slots)
         pad = size - count
         rows = list(source[1]) if source is not None else [0] * count
-        values = (list(tokens) + [0] * pad + list(starts) + [0] * pad + list(slots) + [-1] * pad
-                  + list(slots) + [-1] * pad + list(range(size + 1)) + list(starts) + [0] * pad + list(range(size))
-                  + rows + [0] * pad)
-        staging_for(self.device).upload(values, out=self.ints)
+        # what fills the bucket up are sequences without a slot that bring token 0 at position 0: the host library packs
+        # all of them alike, straight into the memory the arrays are uploaded from
+        ones = [1] * size
+        pack_step(list(slots) + [-1] * pad, ones, list(starts) + [0] * pad, list(tokens) + [0] * pad, ones, [0] * size,
+                  self.device, extra=rows + [0] * pad, out=self.ints)
         if source is not None:
             torch.index_select(source[0], 0, self.source_rows[:count], out=self.batch.token_ids[:count])
 

@@ -182,6 +182,64 @@ def build_reference(verbose: bool = True) -> str:
     return library
 
 
+# ---- the host library (csrc/host/): the runtime's bookkeeping on the CPU, built with the host compiler ----------
+
+HOST = os.path.join(CSRC, "host")
+HOST_LIBRARY = "libxrt_host.so"
+
+
+def host_hash() -> str:
+    digest = hashlib.sha256()
+    for name in sorted(os.listdir(HOST)):
+        with open(os.path.join(HOST, name), "rb") as handle:
+            digest.update(name.encode())
+            digest.update(handle.read())
+    return digest.hexdigest()[:16]
+
+
+def find_host_library():
+    wanted = host_hash()
+    for folder in library_folders():
+        path = os.path.join(folder, HOST_LIBRARY)
+        stamp = path + ".hash"
+        if os.path.isfile(path) and os.path.isfile(stamp) and open(stamp).read().strip() == wanted:
+            return path
+    return None
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compile csrc/host/xrt_host.cpp for the CPU into a shared library; returns its path."""
+    folder = next((f for f in library_folders() if _writable(f)), None)
+    if folder is None:
+        raise BuildError("no writable folder for the host library")
+    library = os.path.join(folder, HOST_LIBRARY)
+    partial = library + f".{os.getpid()}.tmp"
+    done = subprocess.run([_host_compiler(), *HOST_FLAGS, "-fPIC", "-shared", "-o", partial,
+                           os.path.join(HOST, "xrt_host.cpp")], capture_output=True, text=True)
+    if done.returncode != 0:
+        raise BuildError(f"compiling the host library failed:\n{done.stderr}")
+    os.replace(partial, library)
+    with open(library + ".hash", "w") as handle:
+        handle.write(host_hash() + "\n")
+    if verbose:
+        print(f"[xrt build] built {library}", file=sys.stderr, flush=True)
+    return library
+
+
+def build_host_selftest(sanitize: bool = True) -> str:
+    """Compile the host library with its self-test (csrc/host/selftest.cpp) into a program, under the host's address
+    and undefined-behaviour sanitizers unless told otherwise; returns its path."""
+    folder = os.path.join(next((f for f in library_folders() if _writable(f)), tempfile.gettempdir()), "_build")
+    os.makedirs(folder, exist_ok=True)
+    program = os.path.join(folder, "host_selftest" + ("_sanitized" if sanitize else ""))
+    flags = SANITIZE_FLAGS if sanitize else HOST_FLAGS
+    done = subprocess.run([_host_compiler(), *flags, "-o", program, os.path.join(HOST, "selftest.cpp"),
+                           os.path.join(HOST, "xrt_host.cpp")], capture_output=True, text=True)
+    if done.returncode != 0:
+        raise BuildError(f"compiling the host library's self-test failed:\n{done.stderr}")
+    return program
+
+
 def build_reference_selftest(sanitize: bool = True) -> str:
     """Compile the references with their self-test (csrc/reference/selftest.cpp) into a program, under the host's
     address and undefined-behaviour sanitizers unless told otherwise; returns its path."""
@@ -199,3 +257,4 @@ def build_reference_selftest(sanitize: bool = True) -> str:
 if __name__ == "__main__":
     print(build())
     print(build_reference())
+    print(build_host())

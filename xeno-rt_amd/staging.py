@@ -49,6 +49,32 @@ class Staging:
         return out
 
 
+    def upload_filled(self, count: int, fill, out: torch.Tensor = None) -> torch.Tensor:
+        """`count` int32 values that `fill(array)` writes into host memory (a numpy array of that length: pinned
+        memory where the device is a GPU, so nothing is copied twice), as a tensor on the device (into `out`, if given)."""
+        if self.device.type != "cuda":
+            data = torch.empty(count, dtype=torch.int32)
+            fill(data.numpy())
+            if out is None:
+                return data
+            out.view(-1).copy_(data)
+            return out
+        index = self.turn
+        self.turn = (index + 1) % len(self.buffers)
+        if self.events[index] is not None:
+            self.events[index].synchronize()
+        if self.buffers[index] is None or self.buffers[index].numel() < count:
+            self.buffers[index] = torch.empty(max(count, 4096), dtype=torch.int32).pin_memory()
+        host = self.buffers[index][:count]
+        fill(host.numpy())
+        if out is None:
+            out = torch.empty(count, dtype=torch.int32, device=self.device)
+        out.view(-1).copy_(host, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record(torch.cuda.current_stream(self.device))
+        self.events[index] = event
+        return out
+
     def fetch(self, tensor: torch.Tensor) -> "Fetched":
         """Start copying a small int32 tensor to the host. Work queued on the device after this call does
         not delay the copy; at most as many fetches as there are buffers may be under way."""
