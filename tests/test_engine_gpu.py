@@ -418,3 +418,34 @@ def test_head_sizes_that_are_no_multiple_of_16(dtype, arch, sizes, tmp_path):
         assert_logits(logits, want, dtype, f"{arch} {sizes} batched, request of {len(ids)}")
     engine.cache.check()
     assert engine.cache.slots.n_held == 0 and engine.cache.held_blocks() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_step_of_a_size_seen_before_allocates_nothing_but_its_logits(dtype, models):
+    """Steps that are launched kernel by kernel (prompts, and every step of a model whose steps cannot be recorded) cut
+    their tensors, and the kernels' workspaces, from one stretch of memory that is as long as the largest step so far
+    needed (the reference grows its scratch on demand and keeps it, llama.rs:240-268). What the caller gets (the
+    logits) is memory of its own, and stays valid while later steps run."""
+    from xeno_rt_amd.engine import Engine
+    folder, plain, cases = models["qwen3"]
+    engine = Engine.load(folder, dtype=dtype, max_tokens=64 * 8, max_slots=3, graphs=False)
+    ids, want = cases[129]
+    allocations = lambda: torch.cuda.memory_stats()["allocation.all.allocated"]
+    kept = []
+    for round_ in range(4):
+        slot, other = engine.alloc_slot(), engine.alloc_slot()
+        before = allocations()
+        rows = [engine.step([(slot, ids[:100], list(range(100))), (other, ids[:7], [6])])]
+        after_prompt = allocations()
+        for t in range(100, 129):
+            rows.append(engine.step([(slot, [ids[t]], [0]), (other, [ids[t - 93]], [])]))
+        after_decoding = allocations()
+        engine.free_slot(slot); engine.free_slot(other)
+        if round_ >= 2:         # the first round finds out what a step needs, the second takes it once
+            assert after_prompt - before == 1 and after_decoding - after_prompt == 29, \
+                (after_prompt - before, after_decoding - after_prompt)
+        kept.append(rows)
+    for rows in kept:           # logits of earlier steps are still what they were
+        got = torch.cat([rows[0][:100]] + rows[1:])
+        assert_logits(got, want, dtype, "steps from the arena")
+    assert torch.equal(torch.cat(kept[0]), torch.cat(kept[3]))

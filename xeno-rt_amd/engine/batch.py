@@ -50,7 +50,7 @@ def flatten(lists: Sequence[Sequence[int]]):
 
 
 def pack_step(slots, counts, starts, tokens, want_counts, wants, device, pad_tokens_to: int = 0, extra: Sequence[int] = (),
-              out: torch.Tensor = None):
+              out: torch.Tensor = None, allocate=None):
     """The step's arrays, packed by the host library (csrc/host/xrt_host.cpp: xrt_step_pack) straight into the memory
     they are uploaded from: returns (int32 tensor on the device: [token ids | positions | slots | sequence slots |
     offsets | starts | logit rows | extra], the step's facts). All arguments are int32 arrays; tokens and wants are flat."""
@@ -68,6 +68,8 @@ def pack_step(slots, counts, starts, tokens, want_counts, wants, device, pad_tok
                                         room, ctypes.byref(facts)))
         host[room:] = extra
 
+    if out is None and allocate is not None:
+        out = allocate(room + len(extra))
     packed = staging_for(device).upload_filled(room + len(extra), fill, out=out)
     if status[0] != 0:
         raise ValueError(last_error())
@@ -75,11 +77,12 @@ def pack_step(slots, counts, starts, tokens, want_counts, wants, device, pad_tok
 
 
 def build_batch(slots: Sequence[int], tokens: Sequence[Sequence[int]], starts: Sequence[int],
-                wants: Sequence[Sequence[int]], device, pad_tokens_to: int = 0) -> StepBatch:
-    """Pack the step's sequences. `wants[i]` are indices into `tokens[i]`."""
+                wants: Sequence[Sequence[int]], device, pad_tokens_to: int = 0, allocate=None) -> StepBatch:
+    """Pack the step's sequences. `wants[i]` are indices into `tokens[i]`. allocate(count): where the int32 arrays
+    lie on the device (None: a tensor of their own)."""
     counts, flat_tokens = flatten(tokens)
     want_counts, flat_wants = flatten(wants)
-    dev, facts = pack_step(slots, counts, starts, flat_tokens, want_counts, flat_wants, device, pad_tokens_to)
+    dev, facts = pack_step(slots, counts, starts, flat_tokens, want_counts, flat_wants, device, pad_tokens_to, allocate=allocate)
     n_tokens, n_sequences, n_rows = facts.n_tokens, len(slots), facts.n_rows
     cuts, at = [], 0
     for size in (n_tokens, n_tokens, n_tokens, n_sequences, n_sequences + 1, n_sequences, n_rows):

@@ -162,7 +162,9 @@ class Engine:
             if self.graphs is not None and all(len(ids) == 1 for ids in tokens) and all(w == [0] for w in wants):
                 logits = self.graphs.step(slots, [ids[0] for ids in tokens], starts)
             else:
-                logits = self.model.forward(build_batch(slots, tokens, starts, wants, self.device), self.cache)
+                with self.runtime.step_memory():                # the step's tensors come from memory kept for steps
+                    batch = build_batch(slots, tokens, starts, wants, self.device, allocate=self._step_integers)
+                    logits = self.model.forward(batch, self.cache)
         except Exception:
             for slot in slots:
                 self.cache.cancel(slot)
@@ -184,9 +186,10 @@ class Engine:
             if self.graphs is not None:
                 logits = self.graphs.step(slots, [0] * len(slots), starts, source=(tokens, rows))
             else:
-                batch = build_batch(slots, [[0]] * len(slots), starts, [[0]] * len(slots), self.device)
-                batch.token_ids.copy_(tokens.index_select(0, staging_for(self.device).upload(rows)))
-                logits = self.model.forward(batch, self.cache)
+                with self.runtime.step_memory():
+                    batch = build_batch(slots, [[0]] * len(slots), starts, [[0]] * len(slots), self.device, allocate=self._step_integers)
+                    batch.token_ids.copy_(tokens.index_select(0, staging_for(self.device).upload(rows)))
+                    logits = self.model.forward(batch, self.cache)
         except Exception:
             for slot in slots:
                 self.cache.cancel(slot)
@@ -194,6 +197,9 @@ class Engine:
         for slot, start in zip(slots, starts):
             self.cache.commit(slot, start + 1)
         return logits
+
+    def _step_integers(self, count: int) -> torch.Tensor:
+        return self.runtime.empty((count,), torch.int32)
 
     def prepare(self, entries):
         """Check a step and reserve its cache blocks; returns (slots, tokens, wants, starts) per sequence.

@@ -102,6 +102,6 @@ class DecoderModel:
             then = after.first_norm() if after is not None and getattr(after, "passes_norms", False) else None
             h = block.forward(x, batch, cache.layer_cache(index), h=h, then=then)
         if batch.n_logit_rows == 0:
-            return self.runtime.empty((0, spec.head.vocab), torch.float32)
+            return self.runtime.empty((0, spec.head.vocab), torch.float32, outlives_the_step=True)
         y = spec.final_norm.forward(x, rows=batch.logit_rows)
         return spec.head.forward(y)

@@ -116,6 +116,15 @@ class HipOps:
             cls._instance = cls()
         return cls._instance
 
+    # Where the workspaces of kernels and the rows that one product hands to the next come from: None is torch; a
+    # runtime that keeps a stretch of memory for the tensors of a step puts its own function here while a step runs.
+    allocate = None
+
+    def _empty(self, shape, dtype, device) -> torch.Tensor:
+        if self.allocate is not None:
+            return self.allocate(shape, dtype, device)
+        return torch.empty(shape, dtype=dtype, device=device)
+
     def __init__(self):
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the kernels of this library run on an MI355X only")
@@ -265,21 +274,20 @@ class HipOps:
             # many rows: the product's second kernel adds its parts and writes the rows' norm outright
             gain, eps = then_norm
             self._require(gain, "norm gain", None, (n,), a)
-            normed = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+            normed = self._empty((m, n), torch.bfloat16, a.device)
             norm = _LinearNorm()
             norm.eps = float(eps)
             norm.scaled_out, norm.gain, norm.gain_dtype = normed.data_ptr(), gain.data_ptr(), _code(gain)
             need = int(self.lib.xrt_linear_whole_norm_workspace(*sizes, m, n, k, mode))
-            workspace = torch.empty(need, dtype=torch.float32, device=a.device)
+            workspace = self._empty(need, torch.float32, a.device)
             self._check(self.lib.xrt_linear_normed(*packed, _ptr(out), _code(out), m, n, k, coded_mode, ctypes.byref(norm),
                                                    _ptr(workspace), ctypes.c_long(need), self._stream(a)))
             return normed
         if takes == 1:
             gain, eps = then_norm
             self._require(gain, "norm gain", None, (n,), a)
-            emit = Prescaled(torch.empty((m, n), dtype=torch.bfloat16, device=a.device),
-                             torch.empty((int(self.lib.xrt_linear_norm_tiles(*packed, m, n, k)), SQUARES_STRIDE),
-                                         dtype=torch.float32, device=a.device),
+            emit = Prescaled(self._empty((m, n), torch.bfloat16, a.device),
+                             self._empty((int(self.lib.xrt_linear_norm_tiles(*packed, m, n, k)), SQUARES_STRIDE), torch.float32, a.device),
                              float(eps))
         if scaled is not None or emit is not None:
             norm = _LinearNorm()
@@ -291,12 +299,12 @@ class HipOps:
                 norm.scaled_out, norm.squares_out = emit.values.data_ptr(), emit.squares.data_ptr()
                 norm.gain, norm.gain_dtype = then_norm[0].data_ptr(), _code(then_norm[0])
             need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
-            workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
+            workspace = self._empty(need, torch.float32, a.device) if need > 0 else None
             self._check(self.lib.xrt_linear_normed(*packed, _ptr(out), _code(out), m, n, k, coded_mode, ctypes.byref(norm),
                                                    _ptr(workspace), ctypes.c_long(need), self._stream(a)))
             return emit
         need = int(self.lib.xrt_linear_workspace(*sizes, m, n, k, mode))
-        workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
+        workspace = self._empty(need, torch.float32, a.device) if need > 0 else None
         self._check(self.lib.xrt_linear_with(*packed, _ptr(out), _code(out), m, n, k, coded_mode,
                                              _ptr(workspace), ctypes.c_long(need), self._stream(a)))
         return None
@@ -372,7 +380,7 @@ class HipOps:
             norm = _LinearNorm()
             norm.squares_in, norm.tiles_in, norm.width_in, norm.eps = scaled.squares.data_ptr(), tiles, k, scaled.eps
         need = int(self.lib.xrt_linear_workspace(_ptr(a), _ptr(data), _code(a), m, w.shape[0], k, 0))
-        workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need > 0 else None
+        workspace = self._empty(need, torch.float32, a.device) if need > 0 else None
         self._check(self.lib.xrt_linear_qkv(_ptr(a), _ptr(data), packing, _code(a), _ptr(qkv), m, k,
                                             None if norm is None else ctypes.byref(norm), *prepare,
                                             _ptr(workspace), ctypes.c_long(need), self._stream(a)))
@@ -421,7 +429,7 @@ class HipOps:
             workspace_floats = int(self.lib.xrt_attention_workspace(_code(qkv), tokens, n_heads, n_kv_heads, head_dim,
                                                                     int(window or 0), max_count, max_context))
             if workspace_floats > 0:
-                workspace = torch.empty(workspace_floats, dtype=torch.float32, device=qkv.device)
+                workspace = self._empty(workspace_floats, torch.float32, qkv.device)
         self._check(self.lib.xrt_attention(
             _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(k_cache), _ptr(v_cache),
             _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out),

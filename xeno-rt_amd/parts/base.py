@@ -65,6 +65,47 @@ class CacheNeeds:
     state: Optional[StateSpec] = None
 
 
+class StepArena:
+    """One stretch of device memory that the tensors of a step are cut from, one after another; the next step
+    starts at its beginning again. It is as large as the largest step so far needed (the reference grows its
+    scratch on demand and keeps it, crates/xrt-models/src/llama.rs:240-268): a step that needs more than there is
+    takes what does not fit from torch, and the stretch is made longer before the step after it. So a step of a size
+    that has been seen before allocates nothing. What a step hands to its caller (the logits) never lies here."""
+
+    ALIGN = 256
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self.buffer: Optional[torch.Tensor] = None
+        self.at = 0                 # bytes handed out in this step, those that did not fit included
+        self.wanted = 0             # the most a step has needed
+        self.active = False
+
+    def begin(self) -> None:
+        capacity = 0 if self.buffer is None else self.buffer.numel()
+        if self.wanted > capacity:
+            self.buffer = None                                   # (given back before the longer one is taken)
+            self.buffer = torch.empty(self.wanted + self.wanted // 8, dtype=torch.uint8, device=self.device)
+        self.at = 0
+        self.active = True
+
+    def end(self) -> None:
+        self.wanted = max(self.wanted, self.at)
+        self.active = False
+
+    def take(self, shape, dtype: torch.dtype) -> Optional[torch.Tensor]:
+        """A tensor of this shape from the stretch, or None if it does not fit (the caller takes it from torch)."""
+        count = 1
+        for size in (shape if isinstance(shape, (tuple, list, torch.Size)) else (shape,)):
+            count *= int(size)
+        size = count * torch.empty(0, dtype=dtype).element_size()
+        start = (self.at + self.ALIGN - 1) // self.ALIGN * self.ALIGN
+        self.at = start + size
+        if self.buffer is None or self.at > self.buffer.numel():
+            return None
+        return self.buffer[start:start + size].view(dtype).view(shape)
+
+
 class Runtime:
     """What a part needs to run: the kernels, the compute dtype and the device."""
 
@@ -77,6 +118,7 @@ class Runtime:
         self.dtype = dtype
         self.device = torch.device(device)
         self.pack_weights = pack_weights        # "auto": where the kernels say it pays; "always": wherever it can be done
+        self.arena = StepArena(self.device)     # what `empty` cuts a step's tensors from, while a step is under way
 
     def matrix(self, tensor: torch.Tensor) -> torch.Tensor:
         """A weight matrix in the compute dtype, contiguous, on the device. A tensor that comes from the
@@ -127,8 +169,37 @@ class Runtime:
             return tensor.to(device=self.device).contiguous()
         return tensor.to(device=self.device, dtype=torch.float32).contiguous()
 
-    def empty(self, shape, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    def empty(self, shape, dtype: Optional[torch.dtype] = None, outlives_the_step: bool = False) -> torch.Tensor:
+        """An uninitialised tensor on the device for the step under way. It is gone when the next step begins, unless
+        the part says that it outlives the step (what a model returns to its caller)."""
+        if self.arena.active and not outlives_the_step:
+            taken = self.arena.take(shape, dtype or self.dtype)
+            if taken is not None:
+                return taken
         return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)
+
+    def step_memory(self):
+        """A context in which `empty`, and the kernels' workspaces, come from the step arena."""
+        return _StepMemory(self)
+
+
+class _StepMemory:
+    def __init__(self, runtime: Runtime):
+        self.runtime = runtime
+
+    def __enter__(self):
+        runtime = self.runtime
+        runtime.arena.begin()
+        if hasattr(runtime.ops, "allocate"):                   # the kernels' own workspaces and handed-on rows
+            self.before = runtime.ops.allocate
+            runtime.ops.allocate = lambda shape, dtype, device: runtime.empty(shape, dtype)
+        return runtime.arena
+
+    def __exit__(self, *exc):
+        runtime = self.runtime
+        if hasattr(runtime.ops, "allocate"):
+            runtime.ops.allocate = self.before
+        runtime.arena.end()
 
 
 # ----------------------------------------------------------------------------

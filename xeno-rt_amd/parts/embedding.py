@@ -68,6 +68,6 @@ class OutputHead(Part):
             self.weight = runtime.weight(tensors[self.prefix + "weight"])
 
     def forward(self, y: torch.Tensor) -> torch.Tensor:
-        logits = self.runtime.empty((y.shape[0], self.vocab), torch.float32)
+        logits = self.runtime.empty((y.shape[0], self.vocab), torch.float32, outlives_the_step=True)
         self.runtime.ops.linear(y, self.weight, logits)
         return logits
