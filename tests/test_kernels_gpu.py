@@ -703,6 +703,58 @@ def test_attention_decode_on_matrix_cores(ops, nh, nkv, hd):
     assert torch.equal(out2[:-1], out) and float(out2[-1].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("norms", [True, False])
+@pytest.mark.parametrize("rotated", [True, False])
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 4, 64), (8, 2, 128), (32, 8, 128), (64, 8, 128), (40, 2, 128)])
+def test_attention_decode_that_finishes_q_k_and_v_itself(ops, nh, nkv, hd, rotated, norms):
+    """A decode step in which the attention kernel does what qkv_prepare would have done before it (head norms,
+    rotation, cache write of the new key and value), against the two kernels one after the other: the same
+    formulas, so the results agree to the rounding of bfloat16. Sequences whose newest token is the first of all,
+    the first and the last of a block, and far out (several parts of keys); one padding token."""
+    from xeno_rt_amd.ops.hip import QkvFinish
+    lengths = [1, 64, 65, 700, 128, 2, 1500]
+    kv, keys, values = filled_cache(nkv, hd, torch.bfloat16, lengths, seed=hd + nh)
+    # the newest token's place in the cache holds what an earlier sequence left there: both ways must overwrite it
+    slots = list(range(len(lengths)))
+    positions = [n - 1 for n in lengths]
+    batch = described(slots + [-1], [1] * (len(lengths) + 1), positions + [0])
+    batch.slots, batch.positions = i32(slots + [-1]), i32(positions + [0])
+    tokens = len(lengths) + 1
+    raw = rand(tokens, (nh + 2 * nkv) * hd, dtype=torch.bfloat16, seed=3)
+    raw[3] *= 0.02                                          # heads whose mean square is about the norm's eps
+    theta = (torch.tensor(10000.0) ** (torch.arange(hd // 2) * 2.0 / hd)).to(DEV) if rotated else None
+    qn, kn = (rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0) if norms else (None, None)
+    args = dict(q_norm=qn, k_norm=kn, norm_eps=1e-4, rope_theta=theta, rope_dim=hd if rotated else 0, rope_scale=0.5)
+    scale = 1.0 / math.sqrt(hd)
+    table = ops.rope_table(theta, hd, 0.5, 1500) if rotated else None      # cosines and sines of the positions' angles, made once
+    assert ops.attention_finishes_qkv(torch.bfloat16, nh, nkv, hd, batch, None, args["rope_dim"], table)
+    if rotated:
+        assert not ops.attention_finishes_qkv(torch.bfloat16, nh, nkv, hd, batch, None, hd, table[:1499])   # a position beyond the table
+        angles = torch.arange(1500, dtype=torch.float32)[:, None] * 0.5 / theta.cpu()[None, :]
+        assert rel(table[..., 0].cpu(), torch.cos(angles.double())) < 1e-4 and rel(table[..., 1].cpu(), torch.sin(angles.double())) < 1e-4
+    # the two kernels
+    kv_two, qkv_two = clone_cache(kv), raw.clone()
+    ops.qkv_prepare(qkv_two, nh, nkv, hd, batch.positions, batch.slots, kv=kv_two, **args)
+    out_two = torch.full((tokens, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention(qkv_two, nh, nkv, hd, kv_two, batch, out_two, scale=scale)
+    # the one
+    kv_one, qkv_one = clone_cache(kv), raw.clone()
+    out_one = torch.full((tokens, nh * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention(qkv_one, nh, nkv, hd, kv_one, batch, out_one, scale=scale, finish=QkvFinish(qn, kn, 1e-4, table))
+    assert torch.equal(qkv_one, raw)                        # q, k and v stay as the projection left them
+    assert torch.isfinite(out_one).all() and float(out_one[-1].abs().max()) == 0.0
+    assert rel(out_one[:-1].float(), out_two[:-1].float()) < 1e-2
+    for row in range(tokens - 1):                           # every sequence by itself: short ones are not hidden by long ones
+        assert rel(out_one[row].float(), out_two[row].float()) < 2e-2, row
+    # (what lies beyond the sequences' ends is poisoned with NaN in both caches and stays so)
+    assert torch.equal(torch.nan_to_num(kv_one.v.float(), nan=123.0), torch.nan_to_num(kv_two.v.float(), nan=123.0))
+    plain_one, plain_two = cache_order.plain_keys(kv_one.k).float(), cache_order.plain_keys(kv_two.k).float()
+    same = torch.nan_to_num(plain_one, nan=123.0) == torch.nan_to_num(plain_two, nan=123.0)
+    close = (plain_one - plain_two).abs() <= ULP["bfloat16"] * plain_two.abs().clamp(min=1e-3) * 2
+    assert bool((same | close).all())
+    assert float(same.float().mean()) > 0.999               # only the newest keys can differ at all, by a rounding
+
+
 @pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (24, 8, 64)])
 def test_attention_decode_of_many_sequences(ops, nh, nkv, hd):
     """Seventy sequences: with so many (sequence, key/value head) pairs a workgroup takes all keys of its pair

@@ -81,14 +81,17 @@ def test_gated_mlp_part(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("nh,nkv,hd,qk_norm", [(4, 2, 16, False), (6, 3, 32, True), (8, 8, 64, True), (8, 1, 128, False)])
-def test_attention_part_prompt_then_decode(dtype, nh, nkv, hd, qk_norm):
+@pytest.mark.parametrize("nh,nkv,hd,qk_norm,table", [(4, 2, 16, False, 0), (6, 3, 32, True, 0), (8, 8, 64, True, 0), (8, 1, 128, False, 0),
+                                                     (8, 8, 64, True, 140), (6, 2, 128, True, 1000), (6, 3, 32, True, 1000)])
+def test_attention_part_prompt_then_decode(dtype, nh, nkv, hd, qk_norm, table):
     """The mixer with its cache: a prompt in one step, then single tokens, two sequences of
-    unequal lengths; compared with plain attention over the whole sequences."""
+    unequal lengths; compared with plain attention over the whole sequences. table: positions whose cosines and sines
+    the rotation keeps: with them the attention of a bfloat16 decode step with head norms finishes q, k and v itself,
+    as long as the table covers the step (140: the longer sequence's last steps lie beyond it and take the two kernels)."""
     from xeno_rt_amd.cache import SequenceCache
     from xeno_rt_amd.parts import Attention, Rotary
     hidden = 72
-    part = Attention("a.", hidden, nh, nkv, hd, position=Rotary(hd, 7000.0), qk_norm=qk_norm, qk_norm_eps=1e-5)
+    part = Attention("a.", hidden, nh, nkv, hd, position=Rotary(hd, 7000.0, table_positions=table), qk_norm=qk_norm, qk_norm_eps=1e-5)
     # scores come out with a spread of about two: sharp attention, not a saturated one
     w = weights_for(part, 3, std=0.15)
     rt = runtime(dtype)
@@ -118,10 +121,12 @@ def test_attention_part_prompt_then_decode(dtype, nh, nkv, hd, qk_norm):
     for s, c in zip(slots, prompts):
         cache.commit(s, c)
     at = list(prompts)
+    finished_here = []
     while any(a < n for a, n in zip(at, lengths)):
         live = [i for i in range(2) if at[i] < lengths[i]]
         batch, _ = batch_for(cache, [slots[i] for i in live], [1] * len(live))
         residual = torch.zeros(len(live), hidden, device=DEV)
+        finished_here.append((batch.max_context, bool(qk_norm and rt.ops.attention_finishes_qkv(DT[dtype], nh, nkv, hd, batch, None, hd, part.position.table))))
         part.forward(torch.stack([hs[i][at[i]] for i in live]).to(DEV), batch, cache.layer_cache(0), residual)
         for row, i in enumerate(live):
             got[i].append(residual[row:row + 1].clone())
@@ -130,6 +135,10 @@ def test_attention_part_prompt_then_decode(dtype, nh, nkv, hd, qk_norm):
     for i in range(2):
         assert rel(torch.cat(got[i]), want[i]) < TOL[dtype], i
     assert part.scale == 1.0 / math.sqrt(hd)
+    # which steps the one kernel took: those that the table covers
+    takes = dtype == "bfloat16" and qk_norm and table > 0 and hd in (64, 128)
+    assert [took for _, took in finished_here] == [takes and longest <= table for longest, _ in finished_here]
+    assert [longest for longest, _ in finished_here][:20] == list(range(131, 151))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

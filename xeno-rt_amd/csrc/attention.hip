@@ -14,7 +14,7 @@ long xrt_attention_decode_workspace(int tokens, int n_heads, int n_kv_heads, int
 int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
                          const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                          const int* positions, const int* slots, void* out, float scale, int max_context,
-                         float* workspace, long workspace_floats, hipStream_t s);
+                         float* workspace, long workspace_floats, const xrt_qkv_finish* finish, hipStream_t s);
 bool xrt_attention_prefill_accepts(int head_dim);
 int xrt_attention_prefill(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
                           const void* v_cache, const int* block_table, int table_stride, int n_blocks,
@@ -54,7 +54,7 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
             (need == 0 || (workspace != nullptr && workspace_floats >= need)))
             return xrt_attention_decode(qkv, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
                                         table_stride, n_blocks, positions, slots, out, scale, max_context, workspace,
-                                        workspace_floats, s);
+                                        workspace_floats, nullptr, s);
         if (max_count > 1 && xrt_attention_prefill_accepts(head_dim)) {
             // tokens beyond the sequences (padding) get zeros
             // (their rows are read by nothing, but must not hold what a later product could choke on)
@@ -66,4 +66,32 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
     }
     return xrt_attention_generic(qkv, dtype, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
                                  table_stride, n_blocks, positions, slots, out, scale, window, distance_slopes, s);
+}
+
+// ---- a decode step whose attention also finishes q, k and v (xrt_hip.h)
+
+extern "C" int xrt_attention_finishes_qkv(int dtype, int n_heads, int n_kv_heads, int head_dim, int window, int max_count, int rope_dim,
+                                          int table_positions, int max_context) {
+    return max_context > 0 && takes_decode_kernel(dtype, n_heads, n_kv_heads, head_dim, window, max_count, max_context) &&
+           (rope_dim == 0 || (rope_dim == head_dim && table_positions >= max_context));
+}
+
+extern "C" int xrt_attention_finishing(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
+                                       void* k_cache, void* v_cache, const int* block_table, int table_stride,
+                                       int n_blocks, const int* positions, const int* slots, void* out, float scale,
+                                       const xrt_qkv_finish* finish, int max_context, float* workspace, long workspace_floats, void* stream) {
+    XRT_REQUIRE(finish != nullptr, "attention (finishing q/k/v): nothing to finish");
+    XRT_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+                "attention: head counts %d/%d: the first must be a multiple of the second", n_heads, n_kv_heads);
+    XRT_REQUIRE(xrt_attention_finishes_qkv(dtype, n_heads, n_kv_heads, head_dim, 0, 1, finish->rope_table ? finish->rope_dim : 0,
+                                           finish->table_positions, max_context),
+                "attention (finishing q/k/v): only a bfloat16 decode step with heads of 64 or 128 dims, rotated whole (with a table "
+                "of the rotation's turns that covers the step's positions) or not at all");
+    XRT_REQUIRE(qkv && k_cache && v_cache && block_table && positions && slots && out, "attention: null operand");
+    XRT_REQUIRE(table_stride > 0 && n_blocks > 0, "attention: empty cache");
+    if (tokens == 0) return 0;
+    const long need = xrt_attention_decode_workspace(tokens, n_heads, n_kv_heads, head_dim, max_context);
+    XRT_REQUIRE(need == 0 || (workspace != nullptr && workspace_floats >= need), "attention (finishing q/k/v): the workspace needs %ld floats", need);
+    return xrt_attention_decode(qkv, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table, table_stride, n_blocks,
+                                positions, slots, out, scale, max_context, workspace, workspace_floats, finish, (hipStream_t)stream);
 }

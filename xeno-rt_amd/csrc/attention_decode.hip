@@ -19,10 +19,26 @@
 // scores are computed, the next block's keys right after. The four wavefronts of a workgroup
 // merge their results (maximum, sum, O) through LDS into one partial result; a second kernel
 // merges the partial results of a token, in order.
+//
+// The kernel can also finish what follows the q/k/v projection (xrt_qkv_finish: the RMSNorm of every head of q and k,
+// the rotation, the write of the new key and value into the cache), so that a decode step of a model with head
+// norms needs no kernel between the projection and the attention. The formulas and their order are those of
+// qkv_prepare.hip (crates/xrt-models/src/llama.rs:1025-1040, crates/xrt-kernels/src/cpu/rope.rs:59-89). A lane holds
+// the dims 32 s + 8 c .. + 7 (s = 0 .. HD/32 - 1) of its query head, so the two dims of a rotation's pair (d and
+// d + HD/2) lie in one lane, and the norm's sum over a head is an exchange among four lanes. The new key and
+// value are worked out by the wavefront whose keys end with the sequence's newest block: it puts them into the
+// registers in which the block came from the cache (where the place of the newest token still holds what was
+// there before) and writes them to the cache for the steps to come.
 #include "cache_layout.h"
 #include "xrt_hip.h"
 
 namespace {
+
+struct Finish {                       // xrt_qkv_finish with its pointers typed
+    const void* q_norm; const void* k_norm; int norm_dtype; float norm_eps;
+    const float2* rope_table; int table_positions;     // (cosine, sine) of the positions' angles, [position][pair]; null: no rotation
+    bf16* k_cache; bf16* v_cache;
+};
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -39,13 +55,66 @@ static_assert(cache_key_offset(32 + 8 * 2 + 4 * 1 + 3, 32 * 3 + 8 * 1, 128) == (
 static_assert(cache_key_offset(8 * 3 + 4 * 0 + 1, 32 * 1 + 8 * 3 + 5, 64) == ((0 * 2 + 0) * 2 + 1) * 512 + lane_place(3 * 4 + 1, 3) + 5, "keys of a block");
 static_assert(cache_value_offset(16 * 5 + 9, 32 + 8 * 2 + 6, 128) == (1 * 8 + 5) * 512 + lane_place(9, 2) + 6, "values of a block");
 
-template <int HD>
+// One head (the dims of this lane: 32 s + 8 c .. + 7) through its RMSNorm (weight `gain`, null: none) and the rotation
+// by the token's position (theta null: none), in float32, and back to bfloat16: what qkv_prepare does to a head.
+// turns: the (cosine, sine) of this position's HD / 2 angles, as xrt_rope_table has worked them out (the same sincosf of the
+// same angles as in qkv_prepare.hip: worked out here, for every workgroup again, they would cost more than the kernel saves);
+// null: no rotation.
+template <int HD, typename TW>
+__device__ __forceinline__ void finish_head(bf16x8 (&x)[HD / 32], const TW* __restrict__ gain, float eps,
+                                            const float2* __restrict__ turns, int c) {
+    constexpr int KS = HD / 32;
+    float inv_rms = 1.0f;
+    if (gain != nullptr) {
+        float squares = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) squares = fmaf((float)x[ks][e], (float)x[ks][e], squares);
+        squares += __shfl_xor(squares, 16, XRT_WAVE);          // the four lanes (r, 0 .. 3) hold the head between them
+        squares += __shfl_xor(squares, 32, XRT_WAVE);
+        inv_rms = 1.0f / sqrtf(squares / (float)HD + eps);
+    }
+    // a pair of the rotation at a time (dims d and d + HD / 2 lie in x[ks] and x[ks + KS / 2]): few registers at once
+#pragma unroll
+    for (int ks = 0; ks < KS / 2; ++ks) {
+        float lower[8], upper[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { lower[e] = (float)x[ks][e]; upper[e] = (float)x[ks + KS / 2][e]; }
+        if (gain != nullptr) {
+            struct alignas(sizeof(TW) * 8) Eight { TW e[8]; };
+            const Eight of_lower = *reinterpret_cast<const Eight*>(gain + ks * 32 + c * 8);
+            const Eight of_upper = *reinterpret_cast<const Eight*>(gain + (ks + KS / 2) * 32 + c * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                lower[e] = lower[e] * inv_rms * to_float(of_lower.e[e]);
+                upper[e] = upper[e] * inv_rms * to_float(of_upper.e[e]);
+            }
+        }
+        if (turns != nullptr) {
+            struct alignas(16) Pairs { float2 e[8]; };
+            const Pairs read = *reinterpret_cast<const Pairs*>(turns + ks * 32 + c * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float cosine = read.e[e].x, sine = read.e[e].y;
+                const float a = lower[e], b = upper[e];
+                lower[e] = a * cosine - b * sine;
+                upper[e] = a * sine + b * cosine;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { x[ks][e] = (bf16)lower[e]; x[ks + KS / 2][e] = (bf16)upper[e]; }
+    }
+}
+
+// FINISH: q, k and v come as the projection left them, and `finish` says what is still to do (see the head of this file).
+template <int HD, bool FINISH>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) attention_decode_kernel(
     const bf16* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads,
     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
     float scale, int chunk_blocks, int n_parts, int q_tiles,
-    float* __restrict__ part_o, float* __restrict__ part_ml, bf16* __restrict__ out) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, bf16* __restrict__ out, const Finish finish) {
     constexpr int KS = HD / 32;                    // K steps of the score product
     constexpr int DT = HD / 16;                    // 16-row tiles of the value product
     __shared__ floatx4 merge_o[WAVES][DT][XRT_WAVE];
@@ -87,7 +156,35 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) attention_decode_kernel(
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
             q[ks] = *reinterpret_cast<const bf16x8*>(qkv + (long)token * row_width + (long)head * HD + ks * 32 + c * 8);
-
+        // The sequence's newest token: its block and its place there. What is still to do to q (and, in the wavefront whose
+        // keys end with the newest block, to the new key) is done before the first keys are asked for: behind their loads
+        // it would wait for them, and with a block's keys and values in registers there is no room for it.
+        const int newest_block = (n_keys - 1) / XRT_BLOCK_TOKENS, newest = (n_keys - 1) % XRT_BLOCK_TOKENS;
+        const bool has_newest = FINISH && last_block == newest_block;
+        bf16x8 new_key[KS];
+        bf16 new_value[DT];
+        if constexpr (FINISH) {
+            const int pos = n_keys - 1;
+            const float2* turns = finish.rope_table != nullptr ? finish.rope_table + (long)min(pos, finish.table_positions - 1) * (HD / 2) : nullptr;   // (the host sends only steps that the table covers)
+            if (has_newest) {                          // (the same for all lanes of the wavefront)
+                const bf16* key_row = qkv + (long)token * row_width + (long)(n_heads + kv_head) * HD;
+                const bf16* value_row = key_row + (long)n_kv_heads * HD;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) new_key[ks] = *reinterpret_cast<const bf16x8*>(key_row + ks * 32 + c * 8);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) new_value[dt] = value_row[dt * 16 + r];
+            }
+            if (finish.norm_dtype == XRT_F32)
+                finish_head<HD>(q, (const float*)finish.q_norm, finish.norm_eps, turns, c);
+            else
+                finish_head<HD>(q, (const bf16*)finish.q_norm, finish.norm_eps, turns, c);
+            if (has_newest) {
+                if (finish.norm_dtype == XRT_F32)
+                    finish_head<HD>(new_key, (const float*)finish.k_norm, finish.norm_eps, turns, c);
+                else
+                    finish_head<HD>(new_key, (const bf16*)finish.k_norm, finish.norm_eps, turns, c);
+            }
+        }
         // Loads are always on their way: a block's values are asked for before its scores are computed, and the
         // next block's keys right after, before the softmax and the value product of this one.
         const int* table = block_table + (long)slot * table_stride;
@@ -114,6 +211,43 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) attention_decode_kernel(
                 for (int dt = 0; dt < DT; ++dt)
                     vreg[g][dt] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(vb + (g * DT + dt) * 512 + lane * 8));
 
+            if constexpr (FINISH) {
+                if (has_newest && b == newest_block) {
+                    // The newest key and value take their places in the registers that hold the block (key 32 g + 8 (r / 4) +
+                    // 4 t + r % 4 lies in lane r of kreg[g][t], token 32 g + 8 c + e in element e of vreg[g] of the lanes c),
+                    // and in the cache (one of the workgroups that share the key/value head writes: q_tile 0).
+                    const int g_new = newest / 32, within = newest % 32;
+                    const int t_new = within % 8 / 4, r_new = within / 8 * 4 + within % 4, c_new = within / 8, e_new = newest % 8;
+#pragma unroll
+                    for (int g = 0; g < 2; ++g) {
+                        if (g != g_new) continue;
+#pragma unroll
+                        for (int t = 0; t < 2; ++t)
+                            if (t == t_new && r == r_new) {
+#pragma unroll
+                                for (int ks = 0; ks < KS; ++ks) kreg[g][t][ks] = new_key[ks];
+                            }
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (e == e_new && c == c_new) {
+#pragma unroll
+                                for (int dt = 0; dt < DT; ++dt) vreg[g][dt][e] = new_value[dt];
+                            }
+                    }
+                    if (q_tile == 0) {
+                        const long base = ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * HD;
+                        if (r == 0) {
+#pragma unroll
+                            for (int ks = 0; ks < KS; ++ks)
+                                *reinterpret_cast<bf16x8*>(finish.k_cache + base + cache_key_offset(newest, ks * 32 + c * 8, HD)) = new_key[ks];
+                        }
+                        if (c == 0) {
+#pragma unroll
+                            for (int dt = 0; dt < DT; ++dt) finish.v_cache[base + cache_value_offset(dt * 16 + r, newest, HD)] = new_value[dt];
+                        }
+                    }
+                }
+            }
             // ---- scores of 64 keys: two groups of 32, two tiles of 16 rows each
             floatx4 s[2][2];
 #pragma unroll
@@ -324,7 +458,7 @@ Cut cut_for(int tokens, int n_kv_heads, int q_tiles, int max_context, int head_d
 template <int HD>
 int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
            const int* block_table, int table_stride, int n_blocks, const int* positions, const int* slots, bf16* out,
-           float scale, int max_context, float* workspace, long workspace_floats, hipStream_t s) {
+           float scale, int max_context, float* workspace, long workspace_floats, const Finish* finish, hipStream_t s) {
     const int group = n_heads / n_kv_heads;
     const int q_tiles = (group + 15) / 16;
     const Cut cut = cut_for(tokens, n_kv_heads, q_tiles, max_context, HD);
@@ -336,9 +470,14 @@ int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16*
     const int row_width = (n_heads + 2 * n_kv_heads) * HD;
     XRT_REQUIRE(tokens <= 65535 && n_kv_heads * q_tiles <= 65535, "attention (decode): grid too large");
     const dim3 grid(cut.n_parts, n_kv_heads * q_tiles, tokens);
-    attention_decode_kernel<HD><<<grid, WAVES * XRT_WAVE, 0, s>>>(
-        qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, positions, slots,
-        scale, cut.chunk_blocks, cut.n_parts, q_tiles, part_o, part_ml, out);
+    if (finish != nullptr)
+        attention_decode_kernel<HD, true><<<grid, WAVES * XRT_WAVE, 0, s>>>(
+            qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, positions, slots,
+            scale, cut.chunk_blocks, cut.n_parts, q_tiles, part_o, part_ml, out, *finish);
+    else
+        attention_decode_kernel<HD, false><<<grid, WAVES * XRT_WAVE, 0, s>>>(
+            qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, positions, slots,
+            scale, cut.chunk_blocks, cut.n_parts, q_tiles, part_o, part_ml, out, Finish{});
     XRT_LAUNCH_CHECK("attention (decode)");
     if (cut.n_parts == 1) return 0;
     const int part_keys = cut.chunk_blocks * WAVES * XRT_BLOCK_TOKENS;
@@ -363,12 +502,29 @@ long xrt_attention_decode_workspace(int tokens, int n_heads, int n_kv_heads, int
 int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
                          const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                          const int* positions, const int* slots, void* out, float scale, int max_context,
-                         float* workspace, long workspace_floats, hipStream_t s) {
+                         float* workspace, long workspace_floats, const xrt_qkv_finish* finish, hipStream_t s) {
+    Finish typed{};
+    if (finish != nullptr) {
+        XRT_REQUIRE((finish->q_norm == nullptr) == (finish->k_norm == nullptr), "attention (decode): q_norm and k_norm come together");
+        XRT_REQUIRE(finish->q_norm == nullptr || finish->norm_dtype == XRT_F32 || finish->norm_dtype == XRT_BF16,
+                    "attention (decode): unknown norm dtype %d", finish->norm_dtype);
+        XRT_REQUIRE(finish->rope_table == nullptr || (finish->rope_dim == head_dim && finish->table_positions >= max_context),
+                    "attention (decode): the rotation that is finished here spans the whole head (%d of %d dims) and its table covers the step's positions (%d of %d)",
+                    finish->rope_dim, head_dim, finish->table_positions, max_context);
+        XRT_REQUIRE((uintptr_t)k_cache % 16 == 0 && (uintptr_t)qkv % 16 == 0 && (uintptr_t)finish->q_norm % 32 == 0 &&
+                    (uintptr_t)finish->k_norm % 32 == 0 && (uintptr_t)finish->rope_table % 16 == 0,
+                    "attention (decode): operands must be aligned to 16 bytes (norm weights to 32)");
+        // the new keys and values go where the old ones are read from
+        typed = Finish{finish->q_norm, finish->k_norm, finish->norm_dtype, finish->norm_eps,
+                       (const float2*)finish->rope_table, finish->rope_table ? finish->table_positions : 0,
+                       (bf16*)const_cast<void*>(k_cache), (bf16*)const_cast<void*>(v_cache)};
+    }
+    const Finish* typed_or_none = finish != nullptr ? &typed : nullptr;
     if (head_dim == 64)
         return launch<64>((const bf16*)qkv, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache,
                           block_table, table_stride, n_blocks, positions, slots, (bf16*)out, scale, max_context,
-                          workspace, workspace_floats, s);
+                          workspace, workspace_floats, typed_or_none, s);
     return launch<128>((const bf16*)qkv, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache,
                        block_table, table_stride, n_blocks, positions, slots, (bf16*)out, scale, max_context,
-                       workspace, workspace_floats, s);
+                       workspace, workspace_floats, typed_or_none, s);
 }

@@ -246,7 +246,27 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) value_cache_write_kernel(
     }
 }
 
+__global__ void __launch_bounds__(256) rope_table_kernel(const float* __restrict__ rope_theta, int half, float rope_scale,
+                                                         long entries, float2* __restrict__ table) {
+    const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= entries) return;
+    const int pos = (int)(index / half), i = (int)(index % half);
+    const float angle = (float)pos * rope_scale / rope_theta[i];       // as in the kernels above
+    float sine, cosine;
+    sincosf(angle, &sine, &cosine);
+    table[index] = make_float2(cosine, sine);
+}
+
 }  // namespace
+
+extern "C" int xrt_rope_table(const float* rope_theta, int rope_dim, float rope_scale, int positions, float* table, void* stream) {
+    XRT_REQUIRE(rope_theta && table && rope_dim > 0 && rope_dim % 2 == 0 && positions > 0 && (uintptr_t)table % 8 == 0,
+                "rope_table: a rotation over an even number of dims, at least one position, a table aligned to 8 bytes");
+    const long entries = (long)positions * (rope_dim / 2);
+    rope_table_kernel<<<(unsigned)((entries + 255) / 256), 256, 0, (hipStream_t)stream>>>(rope_theta, rope_dim / 2, rope_scale, entries, (float2*)table);
+    XRT_LAUNCH_CHECK("rope_table");
+    return 0;
+}
 
 extern "C" int xrt_qkv_prepare(void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                                const int* positions, const int* slots, const void* q_norm, const void* k_norm,

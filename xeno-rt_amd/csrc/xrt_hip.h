@@ -143,6 +143,26 @@ int xrt_linear_qkv(const void* a, const void* w, const xrt_packing* packing, int
 // position P, for position encodings that act on the scores (the general kernel serves them).
 long xrt_attention_workspace(int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int window,
                              int max_count, int max_context);
+// A decode step (every sequence brings one token) of bfloat16 heads of 64 or 128 dims can leave to the attention what
+// xrt_qkv_prepare would do between the projection and it: qkv then holds the projection as it came, and the attention
+// kernel norms the heads of q and k (q_norm null: no head norms), rotates them over the whole head (rope_table null: no
+// rotation; rope_dim must be head_dim), uses the new key and value and writes them into the cache, which must be
+// writable. The cosines and sines of the rotation are read from rope_table, which xrt_rope_table has made and which
+// must cover the step's positions (table_positions >= the longest sequence after the step).
+// xrt_attention_finishes_qkv says whether a step is one that xrt_attention_finishing takes.
+typedef struct xrt_qkv_finish {
+    const void* q_norm; const void* k_norm; int norm_dtype; float norm_eps;
+    int rope_dim; const float* rope_table; int table_positions;
+} xrt_qkv_finish;
+// table[p][i] = (cos, sin) of the angle p * rope_scale / rope_theta[i] for p < positions, i < rope_dim / 2, float32:
+// the values that the kernels which rotate work out for themselves
+int xrt_rope_table(const float* rope_theta, int rope_dim, float rope_scale, int positions, float* table, void* stream);
+int xrt_attention_finishes_qkv(int dtype, int n_heads, int n_kv_heads, int head_dim, int window, int max_count, int rope_dim,
+                               int table_positions, int max_context);
+int xrt_attention_finishing(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
+                            void* k_cache, void* v_cache, const int* block_table, int table_stride,
+                            int n_blocks, const int* positions, const int* slots, void* out, float scale,
+                            const xrt_qkv_finish* finish, int max_context, float* workspace, long workspace_floats, void* stream);
 int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                   const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                   int n_blocks, const int* positions, const int* slots, void* out, float scale, int window,

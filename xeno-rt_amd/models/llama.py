@@ -13,15 +13,23 @@ from ..parts import Attention, Embedding, GatedMLP, OutputHead, PreNormBlock, RM
 from .decoder import ModelSpec
 
 
+MOST_TABLE_POSITIONS = 131072          # 64 MB of cosines and sines at a head size of 128
+
+
 def build_llama(config: LlamaConfig) -> ModelSpec:
     c = config
     embedding = Embedding("model.embed_tokens.", c.vocab_size, c.hidden_size)
     layers = []
+    # one rotation for all layers. With head norms a decode step's attention finishes q and k itself and reads the
+    # positions' cosines and sines from a table (positions * head_dim * 4 bytes, made once when the model is bound;
+    # at most MOST_TABLE_POSITIONS: a step with a longer sequence takes the two kernels)
+    rotary = Rotary(c.rope_dim, c.rope_theta,
+                    table_positions=min(c.max_position_embeddings, MOST_TABLE_POSITIONS) if c.qk_norm else 0)
     for index in range(c.num_hidden_layers):
         p = f"model.layers.{index}."
         mixer = Attention(
             p + "self_attn.", c.hidden_size, c.num_attention_heads, c.num_key_value_heads, c.head_dim,
-            position=Rotary(c.rope_dim, c.rope_theta),
+            position=rotary,
             qk_norm=c.qk_norm, qk_norm_eps=c.rms_norm_eps)          # same eps as the block norms (llama.rs:1028)
         layers.append(PreNormBlock(
             RMSNorm(p + "input_layernorm.", c.hidden_size, c.rms_norm_eps),

@@ -100,6 +100,24 @@ def _matrix(w):
     return w, None
 
 
+class _QkvFinish(ctypes.Structure):
+    _fields_ = [("q_norm", ctypes.c_void_p), ("k_norm", ctypes.c_void_p), ("norm_dtype", ctypes.c_int),
+                ("norm_eps", ctypes.c_float), ("rope_dim", ctypes.c_int), ("rope_table", ctypes.c_void_p),
+                ("table_positions", ctypes.c_int)]
+
+
+@dataclass
+class QkvFinish:
+    """What `attention` is to do to q, k and v before it uses them, in place of `qkv_prepare`: the head norms (weights
+    [head_dim] each, or None), the rotation over the whole head (rope_table: what `rope_table` made of the rotation's
+    theta and scale, [positions, head_dim / 2, 2], for at least the step's positions; None: no rotation), and the write
+    of the step's keys and values into the cache."""
+    q_norm: Optional[torch.Tensor] = None
+    k_norm: Optional[torch.Tensor] = None
+    norm_eps: float = 0.0
+    rope_table: Optional[torch.Tensor] = None
+
+
 class _LinearNorm(ctypes.Structure):
     _fields_ = [("squares_in", ctypes.c_void_p), ("tiles_in", ctypes.c_int), ("width_in", ctypes.c_int),
                 ("eps", ctypes.c_float), ("scaled_out", ctypes.c_void_p), ("gain", ctypes.c_void_p),
@@ -109,6 +127,7 @@ class _LinearNorm(ctypes.Structure):
 class HipOps:
     name = "hip"
     _instance = None
+    QkvFinish = QkvFinish                       # (so that a part that holds the operations needs no import of this module)
 
     @classmethod
     def instance(cls) -> "HipOps":
@@ -142,7 +161,8 @@ class HipOps:
         self.lib.xrt_last_error.restype = ctypes.c_char_p
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
                      "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv", "xrt_random_normal",
-                     "xrt_linear_with", "xrt_pack_weight", "xrt_packing_suits", "xrt_block_tokens"):
+                     "xrt_linear_with", "xrt_pack_weight", "xrt_packing_suits", "xrt_block_tokens",
+                     "xrt_attention_finishes_qkv", "xrt_attention_finishing", "xrt_rope_table"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -399,10 +419,32 @@ class HipOps:
             raise KernelError("block table: expected [slots, blocks]")
         return kv.k, kv.v, kv.block_table, kv.block_table.shape[1], n_blocks
 
-    def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None):
+    def rope_table(self, theta: torch.Tensor, rope_dim: int, scale: float, positions: int) -> torch.Tensor:
+        """float32 [positions, rope_dim / 2, 2]: cosine and sine of the angles position * scale / theta[i], as the kernels
+        that rotate work them out; `attention(finish=...)` reads them instead of working them out again."""
+        self._require(theta, "rope_theta", torch.float32, (rope_dim // 2,))
+        table = torch.empty((positions, rope_dim // 2, 2), dtype=torch.float32, device=theta.device)
+        self._check(self.lib.xrt_rope_table(_ptr(theta), int(rope_dim), ctypes.c_float(scale), int(positions), _ptr(table),
+                                            self._stream(theta)))
+        return table
+
+    def attention_finishes_qkv(self, dtype, n_heads, n_kv_heads, head_dim, batch, window=None, rope_dim=0, rope_table=None) -> bool:
+        """Whether `attention` can take this step's q, k and v as the projection left them (finish=...): a bfloat16 decode
+        step with heads of 64 or 128 dims that are not rotated, or rotated whole with a table that covers the step's positions."""
+        if dtype != torch.bfloat16 or getattr(batch, "sequence_offsets", None) is None:
+            return False
+        return bool(self.lib.xrt_attention_finishes_qkv(_CODES[dtype], n_heads, n_kv_heads, head_dim, int(window or 0),
+                                                        int(batch.max_count), int(rope_dim),
+                                                        0 if rope_table is None else int(rope_table.shape[0]), int(batch.max_context)))
+
+    def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None,
+                  finish: Optional[QkvFinish] = None):
         """Causal attention of the step's tokens over the cache. distance_slopes: float32 [n_heads], or None; a key at
-        position j adds slope * (j - P) to the scaled score of the query at position P."""
+        position j adds slope * (j - P) to the scaled score of the query at position P. finish: what is still to do to
+        q, k and v (only where `attention_finishes_qkv` says so); the cache must be writable then."""
         from ..cache import BLOCK_TOKENS
+        if finish is not None:
+            return self._attention_finishing(qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish)
         tokens = qkv.shape[0]
         width = (n_heads + 2 * n_kv_heads) * head_dim
         self._require(qkv, "qkv", None, (tokens, width))
@@ -435,6 +477,36 @@ class HipOps:
             _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out),
             ctypes.c_float(scale), int(window or 0), _ptr(distance_slopes), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
+
+    def _attention_finishing(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish: QkvFinish):
+        from ..cache import BLOCK_TOKENS
+        tokens = qkv.shape[0]
+        width = (n_heads + 2 * n_kv_heads) * head_dim
+        self._require(qkv, "qkv", torch.bfloat16, (tokens, width))
+        self._require(out, "attention out", qkv.dtype, (tokens, n_heads * head_dim), qkv)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), qkv)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), qkv)
+        k_cache, v_cache, table, stride, n_blocks = self._kv(kv, qkv, n_kv_heads, head_dim)
+        if int(batch.max_count) != 1 or int(batch.max_context) > stride * BLOCK_TOKENS:
+            raise KernelError("attention (finishing q/k/v): a decode step whose sequences fit the block table")
+        record = _QkvFinish()
+        if (finish.q_norm is None) != (finish.k_norm is None):
+            raise KernelError("attention (finishing q/k/v): q_norm and k_norm come together")
+        if finish.q_norm is not None:
+            self._require(finish.q_norm, "q_norm", None, (head_dim,), qkv)
+            self._require(finish.k_norm, "k_norm", finish.q_norm.dtype, (head_dim,), qkv)
+            record.q_norm, record.k_norm = finish.q_norm.data_ptr(), finish.k_norm.data_ptr()
+            record.norm_dtype, record.norm_eps = _code(finish.q_norm), float(finish.norm_eps)
+        if finish.rope_table is not None:
+            positions = finish.rope_table.shape[0]
+            self._require(finish.rope_table, "rope_table", torch.float32, (positions, head_dim // 2, 2), qkv)
+            record.rope_dim, record.rope_table, record.table_positions = head_dim, finish.rope_table.data_ptr(), positions
+        need = int(self.lib.xrt_attention_workspace(_code(qkv), tokens, n_heads, n_kv_heads, head_dim, 0, 1, int(batch.max_context)))
+        workspace = self._empty(need, torch.float32, qkv.device) if need > 0 else None
+        self._check(self.lib.xrt_attention_finishing(
+            _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, _ptr(k_cache), _ptr(v_cache), _ptr(table), stride,
+            n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out), ctypes.c_float(scale), ctypes.byref(record),
+            int(batch.max_context), _ptr(workspace), ctypes.c_long(need), self._stream(qkv)))
 
     def sample(self, logits, out, temperature, top_k, top_p, penalty, history, history_spans, uniforms,
                small_top_k=False, append_at=None):

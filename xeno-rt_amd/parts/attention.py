@@ -97,6 +97,19 @@ class Attention(Mixer):
         write_to = kv if cache.writable else None
         longest_run = int(getattr(batch, "max_count", 0) or 0)      # picks how the values are written; 0: unknown
         rotation = None if self.position is None else self.position.rotation()
+        slopes = None if self.position is None else self.position.score_slopes()
+        out = rt.empty((tokens, self.q_width))
+        # A decode step of a model with head norms: the projection only, and the attention kernel finishes q, k and v
+        # itself (norms, rotation, cache write) where it can; without head norms the projection's own kernel does that.
+        finishes = getattr(ops, "attention_finishes_qkv", None)
+        if (self.qk_norm and write_to is not None and slopes is None and (rotation is not None or self.position is None)
+                and finishes is not None and finishes(qkv.dtype, *dims, batch, self.window, 0 if rotation is None else rotation.rope_dim,
+                                                       None if rotation is None else rotation.table)):
+            ops.linear(h, self.w_qkv, qkv)
+            ops.attention(qkv, *dims, kv, batch, out, scale=self.scale,
+                          finish=ops.QkvFinish(self.q_norm, self.k_norm, self.qk_norm_eps, None if rotation is None else rotation.table))
+            return ops.linear(out, self.w_o, residual, accumulate=True,
+                              then_norm=None if then is None else then.row_scale())
         if rotation is not None or self.position is None:
             # the projection, then in one pass (in the same kernel, where a step is short): head norms, rotation, cache write
             ops.linear_qkv(h, self.w_qkv, qkv, *dims, batch.positions, batch.slots,
@@ -115,8 +128,6 @@ class Attention(Mixer):
             if write_to is not None:
                 ops.qkv_prepare(qkv, *dims, batch.positions, batch.slots, kv=write_to, longest_run=longest_run)
 
-        out = rt.empty((tokens, self.q_width))
-        slopes = None if self.position is None else self.position.score_slopes()
         ops.attention(qkv, *dims, kv, batch, out, scale=self.scale, window=self.window,
                       **({} if slopes is None else {"distance_slopes": slopes}))
         return ops.linear(out, self.w_o, residual, accumulate=True,

@@ -245,6 +245,8 @@ class HalfSplitRotation:
     rope_dim: int
     scale: float
     theta: Optional[torch.Tensor]
+    table: Optional[torch.Tensor] = None       # float32 [positions, rope_dim / 2, 2]: cosine and sine of the first positions' angles,
+                                               # made by `ops.rope_table`, for kernels that would rather read than work them out
 
 
 class PositionEncoding(Part):
