@@ -276,15 +276,20 @@ def test_a_step_may_mix_sequences_that_start_with_sequences_that_go_on(name, dty
     engine.cache.check()
 
 
+@pytest.mark.parametrize("arch,sizes", [
+    ("llama", dict(num_attention_heads=4, num_key_value_heads=1, head_dim=64, max_position_embeddings=1200)),
+    # with head norms the attention of a bfloat16 decode step also norms and rotates q and the new key and writes the cache
+    ("qwen3", dict(num_attention_heads=6, num_key_value_heads=2, head_dim=128, max_position_embeddings=1200)),
+    ("qwen3", dict(num_attention_heads=6, num_key_value_heads=3, head_dim=64, max_position_embeddings=1200)),
+])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_decoding_across_a_thousand_tokens(dtype, tmp_path):
+def test_decoding_across_a_thousand_tokens(dtype, arch, sizes, tmp_path):
     """Two sequences decode from just under 1024 tokens to beyond it, one of them from a block edge:
-    the recorded decode steps change their context size on the way (head size 64: in bfloat16 the
+    the recorded decode steps change their context size on the way (head sizes 64 and 128: in bfloat16 the
     matrix-core decode kernel with its split over key chunks and its merge). Every step must equal
     the same step run directly, and the last logits must be the plain model's."""
     from xeno_rt_amd.engine import Engine
-    raw = dict(TINY["llama"], max_position_embeddings=1200, num_hidden_layers=2, num_attention_heads=4,
-               num_key_value_heads=1, head_dim=64, rope_theta=50000.0)
+    raw = dict(TINY[arch], num_hidden_layers=2, rope_theta=50000.0, **sizes)
     folder = make_folder(raw, tmp_path / "long", seed=9, std=0.25)
     plain = P.PlainModel(folder)
     vocab = plain.config.vocab_size
