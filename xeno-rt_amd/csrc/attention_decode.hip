@@ -56,7 +56,7 @@ static_assert(cache_key_offset(8 * 3 + 4 * 0 + 1, 32 * 1 + 8 * 3 + 5, 64) == ((0
 static_assert(cache_value_offset(16 * 5 + 9, 32 + 8 * 2 + 6, 128) == (1 * 8 + 5) * 512 + lane_place(9, 2) + 6, "values of a block");
 
 // One head (the dims of this lane: 32 s + 8 c .. + 7) through its RMSNorm (weight `gain`, null: none) and the rotation
-// by the token's position (theta null: none), in float32, and back to bfloat16: what qkv_prepare does to a head.
+// by the token's position, in float32, and back to bfloat16: what qkv_prepare does to a head.
 // turns: the (cosine, sine) of this position's HD / 2 angles, as xrt_rope_table has worked them out (the same sincosf of the
 // same angles as in qkv_prepare.hip: worked out here, for every workgroup again, they would cost more than the kernel saves);
 // null: no rotation.
