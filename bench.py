@@ -38,10 +38,18 @@ SHAPES = {
     "qwen3-32b": dict(COMMON, architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=5120,
                       intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64, rms_norm_eps=1e-6,
                       rope_theta=1000000.0),
+    # two small shapes: heads of 64, a tied output head, widths at which every kernel's fixed cost weighs most
+    "llama32-1b": dict(COMMON, architectures=["LlamaForCausalLM"], vocab_size=128256, hidden_size=2048, head_dim=64,
+                       intermediate_size=8192, num_hidden_layers=16, rms_norm_eps=1e-5, rope_theta=500000.0,
+                       tie_word_embeddings=True),
+    "qwen3-0.6b": dict(COMMON, architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=1024,
+                       num_attention_heads=16, intermediate_size=3072, num_hidden_layers=28, rms_norm_eps=1e-6,
+                       rope_theta=1000000.0, tie_word_embeddings=True),
 }
-MODEL_NAMES = {"llama3-8b": "Llama-3-8B shape", "qwen3-8b": "Qwen3-8B shape", "qwen3-32b": "Qwen3-32B shape"}
-HEADLINE_BATCH = {"llama3-8b": 8, "qwen3-8b": 8, "qwen3-32b": 32}
-OTHER_BATCHES = {"llama3-8b": (1, 64), "qwen3-8b": (1, 64), "qwen3-32b": (1,)}
+MODEL_NAMES = {"llama3-8b": "Llama-3-8B shape", "qwen3-8b": "Qwen3-8B shape", "qwen3-32b": "Qwen3-32B shape",
+               "llama32-1b": "Llama-3.2-1B shape", "qwen3-0.6b": "Qwen3-0.6B shape"}
+HEADLINE_BATCH = {"llama3-8b": 8, "qwen3-8b": 8, "qwen3-32b": 32, "llama32-1b": 8, "qwen3-0.6b": 8}
+OTHER_BATCHES = {"llama3-8b": (1, 64), "qwen3-8b": (1, 64), "qwen3-32b": (1,), "llama32-1b": (1, 64), "qwen3-0.6b": (1, 64)}
 CONTEXT = 4096
 SHORT_CONTEXT = 128
 PREFILL_TOKENS = 2048
