@@ -1,5 +1,5 @@
-"""The engine at the layer sizes of real models (Llama-3-8B, Qwen3-8B and Qwen3-32B shapes, two layers of
-them) and at a context of 4096, against the plain implementation, in 32-bit and in bfloat16.
+"""The engine at the layer sizes of real models (Llama-3-8B, Qwen3-8B, Qwen3-32B, Llama-3.2-1B and Qwen3-0.6B
+shapes, two layers of them) and at a context of 4096, against the plain implementation, in 32-bit and in bfloat16.
 
 Weights come from the random-weights mode in memory (`Engine.random`); the plain model gets the
 same tensors through `get_tensor`, which makes them again on the host. Schedules: a prompt alone
@@ -31,12 +31,22 @@ SHAPES = {
                       num_hidden_layers=2, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
                       rms_norm_eps=1e-6, rope_theta=1000000.0, max_position_embeddings=4096,
                       tie_word_embeddings=False, hidden_act="silu"),
+    # small shapes: heads of 64 with a width of 2048 (matrices with too few rows to be kept packed), a tied head
+    "llama32-1b": dict(architectures=["LlamaForCausalLM"], vocab_size=128256, hidden_size=2048, intermediate_size=8192,
+                       num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+                       rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=4096,
+                       tie_word_embeddings=True, hidden_act="silu"),
+    # heads that are wider together than the model (16 x 128 against 1024), head norms, a tied head
+    "qwen3-0.6b": dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=1024, intermediate_size=3072,
+                       num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
+                       rms_norm_eps=1e-6, rope_theta=1000000.0, max_position_embeddings=4096,
+                       tie_word_embeddings=True, hidden_act="silu"),
 }
-LAYERS_OF_THE_MODELS = {"llama3-8b": 32, "qwen3-8b": 36, "qwen3-32b": 64}       # the tests run two layers of these sizes
+LAYERS_OF_THE_MODELS = {"llama3-8b": 32, "qwen3-8b": 36, "qwen3-32b": 64, "llama32-1b": 16, "qwen3-0.6b": 28}   # the tests run two layers of these sizes
 CONTEXT, TAIL = 4096, 40
 PORTIONS = [1024, 2, 2046, 984]             # 4056 tokens: a start on a block's boundary, two tokens, an end at a block's end
 WHOLE = 300
-SEED = {"llama3-8b": 3, "qwen3-8b": 4, "qwen3-32b": 5}
+SEED = {"llama3-8b": 3, "qwen3-8b": 4, "qwen3-32b": 5, "llama32-1b": 6, "qwen3-0.6b": 7}
 
 
 def batch_plan(vocab):
@@ -130,8 +140,9 @@ def test_weights_made_on_the_device_are_those_made_on_the_host(case, engines, dt
     p = "model.layers.1.self_attn."
     want = torch.cat([data["wide"][p + f"{n}_proj.weight"] for n in "qkv"]).to(kind)
     assert torch.equal(plain_matrix(mixer.w_qkv).cpu(), want)
-    assert torch.equal(plain_matrix(engine.model.spec.head.weight).cpu(), data["wide"]["lm_head.weight"].to(kind))
-    if dtype == "bfloat16":          # matrices of these sizes are kept in tiles, for the products of few rows
+    head = "model.embed_tokens.weight" if config.tie_word_embeddings else "lm_head.weight"
+    assert torch.equal(plain_matrix(engine.model.spec.head.weight).cpu(), data["wide"][head].to(kind))
+    if dtype == "bfloat16" and config.hidden_size >= 4096:          # matrices of these sizes are kept in tiles, for the products of few rows
         assert hasattr(mixer.w_qkv, "unpacked") and hasattr(engine.model.spec.layers[0].feed_forward.w_gate_up, "unpacked")
     gain = engine.model.spec.layers[0].feed_forward_norm.weight
     assert torch.equal(gain.cpu().float(), data["wide"]["model.layers.0.post_attention_layernorm.weight"].to(gain.dtype).float())
