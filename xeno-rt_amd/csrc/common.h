@@ -45,6 +45,12 @@ template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16 from_float<bf16>(float v) { return (bf16)v; }   // round to nearest even
 
+// The value that the lane 8 places away in this lane's row of 16 lanes holds (lane ^ 8): one instruction of the vector
+// unit (a rotation of the row by half), where a shuffle goes through the LDS hardware.
+__device__ __forceinline__ float from_eight_lanes_away(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+}
+
 // ---- wave reductions (fixed butterfly order: results do not depend on the launch) ----
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -388,19 +388,25 @@ __device__ __forceinline__ void gemm_tile(
     // first_packed + q of w: the outputs are found through the packing.
     const bool packed_columns = DK != 0 && is_packed(packing);
     if (MODE == MODE_GATED && packed_columns) {
-        // a group of 16 packed rows: the gate rows of 8 outputs, then their up rows: a lane's partner is 8 lanes away
+        // A group of 16 packed rows: the gate rows of 8 outputs, then their up rows: a lane's partner is 8 lanes away.
+        // The two share the work: of two neighbouring rows of the tile the lane with the gates finishes the first
+        // (with its partner's up sum), the lane with the ups the second (with its partner's gate sum).
+        const int q = lane % 32;
+        const bool has_gates = q % 16 < 8;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j) {
+                const long n = n0 + (wave_n * WAVE_N + j * 32) / 2 + q / 16 * 8 + q % 8;
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const float mine = acc[i][j][e], other = __shfl_xor(mine, 8, XRT_WAVE);
-                    const int q = lane % 32;
-                    const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
-                    const long n = n0 + (wave_n * WAVE_N + j * 32) / 2 + q / 16 * 8 + q % 8;
-                    if (q % 16 < 8 && m < M && n < N) out[m * (long)N + n] = from_float<TO>(gate_activation(mine, scale.activation) * other);
+                for (int e = 0; e < 16; e += 2) {
+                    const float first = acc[i][j][e], second = acc[i][j][e + 1];
+                    const float partner_first = from_eight_lanes_away(first), partner_second = from_eight_lanes_away(second);
+                    const float gate = has_gates ? first : partner_second, up = has_gates ? partner_first : second;
+                    const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4 + (has_gates ? 0 : 1);
+                    if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(gate_activation<sizeof(TO) == 2>(gate, scale.activation) * up);
                 }
+            }
     } else if constexpr (MODE == MODE_GATED) {
         static_assert(TN % 2 == 0, "a wavefront holds as many gate blocks as up blocks");
 #pragma unroll
@@ -411,7 +417,7 @@ __device__ __forceinline__ void gemm_tile(
                 for (int e = 0; e < 16; ++e) {
                     const long m = m0 + wave_m * WAVE_M + i * 32 + (e / 4) * 8 + (lane / 32) * 4 + e % 4;
                     const long n = n0 + wave_n * (WAVE_N / 2) + j * 32 + lane % 32;
-                    if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(gate_activation(acc[i][j][e], scale.activation) * acc[i][j + TN / 2][e]);
+                    if (m < M && n < N) out[m * (long)N + n] = from_float<TO>(gate_activation<sizeof(TO) == 2>(acc[i][j][e], scale.activation) * acc[i][j + TN / 2][e]);
                 }
     } else {
         long column[TN];                                        // the output column of this lane in each block of 32
@@ -668,7 +674,7 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(const float* __restri
     if (inside) {
         if constexpr (MODE == MODE_STORE) out[index] = from_float<TO>(sum);
         else if constexpr (MODE == MODE_ACCUMULATE) { fresh = to_float(out[index]) + sum; out[index] = from_float<TO>(fresh); }
-        else out[index] = from_float<TO>(gate_activation(sum, activation) * up);
+        else out[index] = from_float<TO>(gate_activation<sizeof(TO) == 2>(sum, activation) * up);
     }
     if constexpr (NORM == 2) {
         float squares = fresh * fresh;

@@ -320,7 +320,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_pack
             if (c < 2 && mm < M) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (nn + i < N) out[(long)mm * N + nn + i] = from_float<TO>(gate_activation(g[i], activation) * u[i]);
+                    if (nn + i < N) out[(long)mm * N + nn + i] = from_float<TO>(gate_activation<sizeof(TO) == 2>(g[i], activation) * u[i]);
             }
             continue;
         }
@@ -467,7 +467,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, 2) gemm_packed_resident_kern
             if (c < 2 && r < M) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (nn + i < N) out[(long)r * N + nn + i] = from_float<TO>(gate_activation(g[i], activation) * u[i]);
+                    if (nn + i < N) out[(long)r * N + nn + i] = from_float<TO>(gate_activation<sizeof(TO) == 2>(g[i], activation) * u[i]);
             }
         } else {
             const long nn = logical_row(packing, group * 16 + c * 4);

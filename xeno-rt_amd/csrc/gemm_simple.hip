@@ -125,7 +125,7 @@ __global__ void __launch_bounds__(256) gemm_simple_kernel(const TI* __restrict__
             TO* dst = out + m * (long)N + n;
             if constexpr (MODE == MODE_STORE) *dst = from_float<TO>(acc[i][j]);
             if constexpr (MODE == MODE_ACCUMULATE) *dst = from_float<TO>(before[i][j] + acc[i][j]);
-            if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(gate_activation(acc[i][j], activation) * acc_up[i][j]);
+            if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(gate_activation<sizeof(TO) == 2>(acc[i][j], activation) * acc_up[i][j]);
         }
     }
 }

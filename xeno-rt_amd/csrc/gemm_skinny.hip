@@ -413,7 +413,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE, (MT == 1 ? 4 : 2)) gemm_skin
                         fresh[i] = to_float(*dst) + g[i];
                         *dst = from_float<TO>(fresh[i]);
                     }
-                    if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(gate_activation(g[i], activation) * u[i]);
+                    if constexpr (MODE == MODE_GATED) *dst = from_float<TO>(gate_activation<sizeof(TO) == 2>(g[i], activation) * u[i]);
                 }
             }
             if constexpr (AROUND && MODE == MODE_ACCUMULATE) {
