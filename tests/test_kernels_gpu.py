@@ -94,7 +94,9 @@ SHAPES = [(1, 64, 64), (3, 200, 96), (8, 1000, 176), (17, 96, 192), (64, 333, 52
           (2048, 6144, 128), (2000, 6200, 136), (70, 300, 64), (300, 520, 1024), (2100, 6100, 320),
           (2100, 8300, 128), (40, 4100, 1024), (64, 333, 640), (33, 130, 128), (17, 700, 192),
           (600, 520, 8192), (520, 1030, 8320),         # many rows, few columns, a very long k (large tiles that split k)
-          (12, 8200, 288), (9, 8208, 1056), (16, 16400, 4096), (16, 8192, 4128)]   # 9 to 16 rows, many rows of w, k up to 4096: x stays in registers (the last: k too long for that)
+          (12, 8200, 288), (9, 8208, 1056), (16, 16400, 4096), (16, 8192, 4128),   # 9 to 16 rows, many rows of w, k up to 4096: x stays in registers (the last: k too long for that)
+          # 65 to 256 rows, too few columns to fill the chip: tiles of 128 x 64 that split k in long parts (the last two: a long k keeps tiles of 128 x 128, in three stages)
+          (72, 4096, 4096), (130, 1000, 2048), (256, 4104, 1024), (200, 700, 4160), (100, 2048, 8192), (250, 1030, 14336)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16 packed"])
@@ -125,7 +127,9 @@ def test_linear(ops, dtype, m, n, k):
                                    # 17 to 64 rows and tiles enough without a split along k
                                    (40, 14336, 256), (64, 9002, 128), (33, 20000, 192),
                                    # 9 to 16 rows and many pairs: x stays in the registers of a workgroup that walks the rows of w
-                                   (13, 4104, 96), (16, 14336, 4096), (9, 8192, 2080)])
+                                   (13, 4104, 96), (16, 14336, 4096), (9, 8192, 2080),
+                                   # 65 to 128 rows and about a round of tiles of 128 x 128: no split, three stages
+                                   (72, 14336, 1024), (128, 13000, 512), (100, 15000, 192)])
 def test_linear_glu(ops, dtype, m, n, k):
     dtype, packed = dtype.split()[0], dtype.endswith("packed")
     if packed and n % 8 != 0:

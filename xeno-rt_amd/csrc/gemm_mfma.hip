@@ -538,6 +538,11 @@ int launch_mode(const bf16* a, const bf16* w, TO* out, int M, int N, int K, cons
     constexpr int DIV = MODE == MODE_GATED ? 2 : 1;
     auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn / DIV - 1) / (bn / DIV)); };
     const bool whole_k = K % 64 == 0;
+    // Up to 128 rows of a, gated: one round of tiles of 128 x 128 (or nearly), bound by reading w: three stages keep more of
+    // it on its way than the two that the tiles below have (gate/up of 14336 pairs and 128 rows: 76 us split in three
+    // with a second kernel, 49 us so).
+    if constexpr (MODE == MODE_GATED)
+        if (whole_k && M <= 128) return launch_kernel<128, 128, 2, 2, MODE, 64, 3, TO>(a, w, out, M, N, K, 0, N, packing, s, 1, 0, RowScale{nullptr, 0, 0, 0.f, activation});
     const long large = rounds_cost(tiles(256, 256), 256 * 256, 1, 0);
     const long medium = whole_k && MODE != MODE_GATED ? rounds_cost(tiles(256, 192), 256 * 192, 1, 5) : LONG_MAX;
     const long small = rounds_cost(tiles(128, 128), 128 * 128, 2, 18);
@@ -592,7 +597,7 @@ int launch_shape(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
 // few to fill the chip: such products are still bound by reading w.
 constexpr int SPLIT_BM = 64, SPLIT_BN = 128;
 
-struct SplitPlan { int splits, k_per_split; long rows_w; int tile; };      // tile: rows of x per tile (64, 128 or 256)
+struct SplitPlan { int splits, k_per_split; long rows_w; int tile, columns; };      // tile: rows of x per tile (64, 128 or 256), columns: rows of w
 
 // whole_norm: an RMSNorm follows that the second kernel can do outright, which is worth a split in two where the product alone
 // would do as well without (k from 4096 on instead of from 8192 on).
@@ -600,7 +605,7 @@ SplitPlan split_plan(int M, int N, int K, int mode, bool whole_norm = false) {
     const long rows_w = mode == MODE_GATED ? 2L * N : N;
     const long tiles_n = (rows_w + SPLIT_BN - 1) / SPLIT_BN;
     const int units = K / 64;                                  // k is dealt out in pieces of 64
-    int splits, least, tile = SPLIT_BM;                        // least: pieces of k that a part should have
+    int splits, least, tile = SPLIT_BM, columns = SPLIT_BN;    // least: pieces of k that a part should have
     const long large_tiles = (long)((M + 255) / 256) * ((rows_w + 255) / 256);
     if (M <= SPLIT_BM) {
         splits = (int)(XRT_COMPUTE_UNITS / tiles_n);                         // one workgroup per compute unit, or fewer
@@ -613,18 +618,37 @@ SplitPlan split_plan(int M, int N, int K, int mode, bool whole_norm = false) {
         splits = (int)(XRT_COMPUTE_UNITS / large_tiles);
         splits = splits > 8 ? 8 : splits;
         least = 24;
-        tile = 256;
+        tile = columns = 256;
     } else {
-        const long tiles = (long)((M + 127) / 128) * tiles_n;  // two of these workgroups share a compute unit
-        splits = tiles >= 384 ? 1 : (int)((512 + tiles - 1) / tiles);
-        least = 4;
-        tile = 128;
+        // Some hundred rows of x: still bound by reading w, and too few tiles to fill the chip without a split.
+        // Every part of k writes its sums and the second kernel reads them again (16 parts of a square w and 128 rows
+        // of x: as many bytes as w has), so the parts are few and long (1024 of k at least), and where tiles of 128 x 128
+        // are fewer than the compute units and k is short, tiles of 128 x 64 make up the number instead of further parts.
+        // With a long k the partial sums are small against w and the wider tile, which reads x half as often, is kept
+        // (at the sizes of the 8B models, 128 rows: q/k/v 31 -> 25 us, o 24 -> 18, down 40 -> 37).
+        // Beyond 256 rows the matrix cores begin to count: tiles of 128 x 128, two to a compute unit, in as many parts as
+        // fill those places.
+        long tiles = (long)((M + 127) / 128) * tiles_n;
+        tile = columns = 128;
+        if (M <= 256) {
+            if (tiles < XRT_COMPUTE_UNITS && mode != MODE_GATED && K < 8192) {
+                columns = 64;
+                tiles = (long)((M + 127) / 128) * ((rows_w + 63) / 64);
+            }
+            // a gated product with a round of tiles or nearly so does without a split: its tiles apply the epilogue themselves
+            const int target = M <= 128 && columns == 64 ? 2 * XRT_COMPUTE_UNITS : XRT_COMPUTE_UNITS;
+            splits = tiles >= 384 || (mode == MODE_GATED && tiles >= 200) ? 1 : (int)((target + tiles - 1) / tiles);
+            least = columns == 64 ? 16 : 8;
+        } else {
+            splits = tiles >= 384 ? 1 : (int)((512 + tiles - 1) / tiles);
+            least = 4;
+        }
     }
     splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
     splits = splits > units / least ? (units / least < 1 ? 1 : units / least) : splits;
     const int per = (units + splits - 1) / splits;
     splits = (units + per - 1) / per;                          // no empty part
-    return SplitPlan{splits, per * 64, rows_w, tile};
+    return SplitPlan{splits, per * 64, rows_w, tile, columns};
 }
 
 // NORM 1: the rows of a came without their RMSNorm's division (norm.squares_in): the sums are multiplied by
@@ -873,6 +897,12 @@ int launch_split(const bf16* a, const bf16* w, TO* out, int M, int N, int K, int
         : plan.tile == 256
         ? launch_kernel<256, 256, 2, 4, MODE_STORE, 64, 2, float>(
               a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split)
+        : plan.columns == 64
+        ? launch_kernel<128, 64, 2, 2, MODE_STORE, 64, 3, float>(
+              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split)
+        : M <= 256          // (one workgroup to a compute unit anyway: a third stage keeps more of w on its way; with more, two share a unit)
+        ? launch_kernel<128, 128, 2, 2, MODE_STORE, 64, 3, float>(
+              a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split)
         : launch_kernel<128, 128, 2, 2, MODE_STORE, 64, 2, float>(
               a, w, workspace, M, (int)plan.rows_w, K, 0, (int)plan.rows_w, packing, s, plan.splits, plan.k_per_split);
     if (status != 0) return status;
@@ -948,7 +978,8 @@ bool xrt_linear_split_takes(const void* a, const void* w, int M, int N, int K, i
 }
 
 // Whether an accumulating product of many rows runs as large tiles that split k, so that its second kernel can do the
-// RMSNorm that follows it outright; and the floats of workspace it then needs.
+// RMSNorm that follows it outright; and the floats of workspace it then needs. (With the smaller tiles' few rows the
+// kernel that takes a row per workgroup has too few workgroups: 5.75 against 5.65 ms a prompt of 128 tokens.)
 bool xrt_linear_split_takes_whole_norm(const void* a, const void* w, int M, int N, int K, int mode, long* workspace_floats) {
     *workspace_floats = 0;
     if (mode != MODE_ACCUMULATE || M <= SPLIT_BM || K % 64 != 0 || N % 4 != 0 || N > NORM_QUADS * 256 * 4 ||
