@@ -78,7 +78,7 @@ def test_two_calls_in_a_row_share_the_fixed_array():
 
 def test_a_product_beyond_the_fixed_array_is_refused_and_nothing_is_written():
     lib = library()
-    m, n, k = 256, 2048, 8192
+    m, n, k = 1024, 2048, 8192              # large tiles that split k in eight: 16 Mi floats of partial sums
     a, w, _ = operands(m, n, k, 0, 5)
     need = int(lib.xrt_linear_workspace(pointer(a), pointer(w), 1, m, n, k, 0))
     assert need > int(lib.xrt_linear_static_floats())
