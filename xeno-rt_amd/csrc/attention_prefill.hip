@@ -178,23 +178,27 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 
     const int row_key = key_of_row(col);                     // the key this lane's A-operand row stands for
 
-    // One tile of 32 keys (half a block) against this wavefront's 32 queries. edge: some key of the tile may lie beyond
-    // some query, or beyond the sequence's end; the other tiles, nearly all, skip the masks (a scalar branch each).
-    auto tile32 = [&](bool edge, int buffer, int k0, int in_block) {
+    // The operand of the score product for a tile of 32 keys (half a block: in_block is 0 or 32): this lane's key row.
+    auto keys_of = [&](bf16x8 (&k)[KS], int buffer, int in_block) {
         const bf16* kb = &lds_k[buffer][(in_block + row_key) * HD];
-        const int k_turn = k_swizzle(in_block + row_key);     // in_block is 0 or 32: the swizzle of this lane's key row
+        const int k_turn = k_swizzle(in_block + row_key);     // the swizzle of this lane's key row
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) k[ks] = *reinterpret_cast<const bf16x8*>(kb + ((ks * 2 + half) ^ k_turn) * 8);
+    };
+    // One tile of 32 keys against this wavefront's 32 queries. edge: some key of the tile may lie beyond
+    // some query, or beyond the sequence's end; the other tiles, nearly all, skip the masks (a scalar branch each).
+    // k: the tile's keys, already asked for; behind_the_scores: what the caller wants issued right behind the score
+    // products (the read of the next tile's keys, which then has the softmax and the value products to arrive in).
+    auto tile32 = [&](bool edge, int buffer, int k0, int in_block, bf16x8 (&k)[KS], auto&& behind_the_scores) {
         const bf16* vb = &lds_v[buffer][0];
         const int v_first = in_block / 8 + half;              // chunk of a value row that step 0 reads
-        auto k_at = [&](int ks) { return *reinterpret_cast<const bf16x8*>(kb + ((ks * 2 + half) ^ k_turn) * 8); };
         auto v_at = [&](int step, int dt) {
             const int v_row = dt * 32 + col;
             return *reinterpret_cast<const bf16x8*>(vb + v_row * BT + ((v_first + step * 2) ^ v_swizzle(v_row)) * 8);
         };
-        // All operands of the score product, and the values of the first 16 keys, are asked for at once and before the
-        // first product: left to itself the compiler reads one operand, waits for it, multiplies, reads the next.
-        bf16x8 k[KS], v[DT];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) k[ks] = k_at(ks);
+        // The values of the first 16 keys are asked for before the first product (the keys came a tile ago, or just now
+        // for the first tile of a block): left to itself the compiler reads one operand, waits for it, multiplies, reads the next.
+        bf16x8 v[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) v[dt] = v_at(0, dt);
         __builtin_amdgcn_sched_barrier(0);
@@ -203,6 +207,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k[ks], q[ks], s, 0, 0, 0);
+        behind_the_scores();
 
         // register i is key k0 + (i/8)*16 + half*8 + i%8, for this lane's query
         if (edge) {
@@ -278,13 +283,19 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         }
         // one body of code for all tiles of the stage: the kernel stays small enough for the instruction cache
 #pragma unroll 1
-        for (int item = 0; item < PER_STAGE * 2; ++item) {
-            const int b = first + item / 2, in_block = item % 2 * 32;
-            const int k0 = b * BT + in_block;
+        for (int i = 0; i < PER_STAGE; ++i) {
+            const int b = first + i, k0 = b * BT;
             if (b > last_block || k0 > last_key) break;      // uniform in the wavefront, like all that follows
             if (b >= turns_from && ((b - turns_from) % 2 == 1) != helper) continue;
-            const int buffer = stage * PER_STAGE + item / 2;
-            tile32(k0 + 31 > first_masked, buffer, k0, in_block);
+            const int buffer = stage * PER_STAGE + i;
+            // The block's two tiles. The second one's keys are read from LDS behind the first one's score products, so
+            // that they have a softmax and the value products to arrive in (a prompt of 2048 tokens: 62 -> 57 us; with every
+            // tile's keys read a tile ahead, across the blocks of a stage too, 59).
+            const bool both = k0 + 32 <= last_key;
+            bf16x8 first_keys[KS], second_keys[KS];
+            keys_of(first_keys, buffer, 0);
+            tile32(k0 + 31 > first_masked, buffer, k0, 0, first_keys, [&] { if (both) keys_of(second_keys, buffer, 32); });
+            if (both) tile32(k0 + 63 > first_masked, buffer, k0 + 32, 32, second_keys, [] {});
         }
         if (on_early && first + PER_STAGE >= early_blocks) {  // the early tile is done: its result goes out, the late tile's queries come in
             l += __shfl_xor(l, 32, XRT_WAVE);
