@@ -558,8 +558,9 @@ def test_attention(ops, dtype, nh, nkv, hd):
 def test_general_attention_gives_the_same_bits_with_few_tokens_and_with_many(ops, dtype, nh, nkv, hd, window):
     """The general kernel takes a step of few tokens with a workgroup of wavefronts per (token, head), which work the
     chunks of keys off side by side, and a step of many tokens with one wavefront each, which takes the chunks one after
-    the other: the same sums in the same order. Sequences of one, two and six chunks of 512 keys, some ending inside a
-    chunk; the same queries alone and among 3000 others."""
+    the other, and there two or four query heads of a key/value head together (groups of 2 and 4 here): the same sums in
+    the same order. Sequences of one, two and six chunks of 512 keys, some ending inside a chunk; the same queries alone
+    and among 3000 others."""
     lengths = [3000, 513, 512, 70, 1025]
     kv, keys, values = filled_cache(nkv, hd, DT[dtype], lengths, seed=hd)
     slots = [0, 1, 2, 3, 4, 0, 0, 4]
