@@ -73,7 +73,9 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 
     const int tid = threadIdx.x, lane = tid % XRT_WAVE, wave = tid / XRT_WAVE;
     const int col = lane % 32, half = lane / 32;
-    const int head = blockIdx.x;
+    // Workgroup ids are dealt to the 8 XCDs round-robin: the heads are renumbered so that the heads of one group of
+    // key/value heads run on one XCD, at the same time, and find each other's cache blocks in its L2.
+    const int head = n_heads % 8 == 0 ? (int)(blockIdx.x % 8) * (n_heads / 8) + (int)blockIdx.x / 8 : (int)blockIdx.x;
     const int wave_uniform = __builtin_amdgcn_readfirstlane(wave);      // in a scalar register: what depends on it alone is decided by scalar branches
     const int group = wave_uniform % GROUPS;                 // the 32 queries of a tile that this wavefront holds
     const bool helper = wave_uniform >= GROUPS;              // early tile first, then half of the late tile's blocks
@@ -176,6 +178,30 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         }
     };
 
+    // The blocks of the next stage are asked for piece by piece (an instruction for a kilobyte of keys and one of values),
+    // one piece at the stage's start and one behind each tile's score products and value products, the rest before the
+    // barrier. Asked for all at once right after the barrier, the 64 instructions of eight wavefronts queue up: a
+    // wavefront then spends 550 to 1550 cycles of a stage of some 3000 getting its eight accepted (counted with the
+    // shader clock), the wavefronts of the early tile, the younger ones, the longest.
+    constexpr int PIECES = PER_STAGE * LOADS;
+    int next_piece = PIECES, piece_blocks[PER_STAGE], piece_buffer = 0, pieces_wanted = 0;
+    auto fetch_piece = [&]() {
+        if (next_piece >= pieces_wanted) return;
+        const int i = next_piece / LOADS, l = next_piece % LOADS;
+        int block = piece_blocks[0];
+        unsigned kf = k_from[0], vf = v_from[0];
+#pragma unroll
+        for (int j = 1; j < PER_STAGE; ++j) if (i == j) block = piece_blocks[j];
+#pragma unroll
+        for (int j = 1; j < LOADS; ++j) if (l == j) { kf = k_from[j]; vf = v_from[j]; }
+        block = min(max(block, 0), n_blocks - 1);            // the host never hands out anything else
+        const char* kb = reinterpret_cast<const char*>(k_cache + ((long)block * n_kv_heads + kv_head) * BT * HD);
+        const char* vb = reinterpret_cast<const char*>(v_cache + ((long)block * n_kv_heads + kv_head) * HD * BT);
+        const unsigned at = (unsigned)(((piece_buffer + i) * BT * HD) * 2 + (l * WAVES + wave_uniform) * 1024);
+        load_to_lds(kb, kf, lds_k0 + at);
+        load_to_lds(vb, vf, lds_v0 + at);
+        ++next_piece;
+    };
     const int row_key = key_of_row(col);                     // the key this lane's A-operand row stands for
 
     // The operand of the score product for a tile of 32 keys (half a block: in_block is 0 or 32): this lane's key row.
@@ -196,18 +222,21 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
             const int v_row = dt * 32 + col;
             return *reinterpret_cast<const bf16x8*>(vb + v_row * BT + ((v_first + step * 2) ^ v_swizzle(v_row)) * 8);
         };
-        // The values of the first 16 keys are asked for before the first product (the keys came a tile ago, or just now
-        // for the first tile of a block): left to itself the compiler reads one operand, waits for it, multiplies, reads the next.
-        bf16x8 v[DT];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) v[dt] = v_at(0, dt);
-        __builtin_amdgcn_sched_barrier(0);
+        // The values of the first 16 keys are asked for right behind the score products (left to itself the compiler reads
+        // one operand, waits for it, multiplies, reads the next): they have the products and half the softmax to arrive in,
+        // and the wait for the keys before the first product of a block does not wait for them too.
         floatx16 s;
 #pragma unroll
         for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k[ks], q[ks], s, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        bf16x8 v[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) v[dt] = v_at(0, dt);
         behind_the_scores();
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_piece();
 
         // register i is key k0 + (i/8)*16 + half*8 + i%8, for this lane's query
         if (edge) {
@@ -259,6 +288,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
                 if (step == 0) v[dt] = v_at(1, dt);    // the values of the other 16 keys, behind the product that used the register
             }
         }
+        fetch_piece();
     };
 
     // ---- the blocks of the sequence, in order: the next stage's blocks travel while this stage's are used
@@ -276,11 +306,15 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     for (int first = 0; first <= last_block; first += PER_STAGE) {
         const int stage = (first / PER_STAGE) & 1;
         // the other stage's buffers were read in the step before, ahead of the last barrier
+        pieces_wanted = max(0, min(PER_STAGE, last_block - first - PER_STAGE + 1)) * LOADS;
+        next_piece = 0;
+        piece_buffer = (stage ^ 1) * PER_STAGE;
 #pragma unroll
         for (int i = 0; i < PER_STAGE; ++i) {
-            if (first + PER_STAGE + i <= last_block) fetch(coming[i], (stage ^ 1) * PER_STAGE + i);
+            piece_blocks[i] = coming[i];
             coming[i] = block_of(first + 2 * PER_STAGE + i);
         }
+        fetch_piece();
         // one body of code for all tiles of the stage: the kernel stays small enough for the instruction cache
 #pragma unroll 1
         for (int i = 0; i < PER_STAGE; ++i) {
@@ -303,6 +337,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
             take(late_tile);
             on_early = false;
         }
+        while (next_piece < pieces_wanted) fetch_piece();     // a wavefront with few tiles in this stage, or none
         wait_loads_and_barrier<0>();                         // the next blocks have arrived from every wavefront, these have been read by all
     }
 
