@@ -54,7 +54,7 @@ TINY = {"llama": TINY_LLAMA, "qwen3": TINY_QWEN3}
 
 def make_folder(raw_config, folder, seed, std=0.02, randomize_norms=True):
     """Write a model folder with the engine's random-weights mode. Norm weights are then
-    replaced by random values around 1, so that a norm in the wrong place, or a weight
+    replaced by random values near 1, so that a norm in the wrong place, or a weight
     that is not applied, changes the logits."""
     from xeno_rt_amd.config import parse_config
     from xeno_rt_amd.weights import SafetensorsFile, write_random_model, write_safetensors
