@@ -640,19 +640,12 @@ SplitPlan split_plan(int M, int N, int K, int mode, bool whole_norm = false) {
             splits = tiles >= 384 || (mode == MODE_GATED && tiles >= 200) ? 1 : (int)((target + tiles - 1) / tiles);
             least = columns == 64 ? 16 : 8;
         } else {
-            // The workgroups run two to a compute unit, in rounds of 512; a round takes as long as its part of k is, and every
-            // further part sends its sums through memory once more. (Filling the places and a little over, 96 tiles in 6 parts,
-            // ran a second round for a few: down at 384 rows 93 -> 66 us; q/k/v at 832 rows was split in two for nothing: 76 -> 66.)
+            // The workgroups run two to a compute unit: as many parts as still fit those 512 places at once, and none where
+            // that is one. A few workgroups over (96 tiles in 6 parts) run a second round for a few; so do parts enough for
+            // two rounds of shorter workgroups, which an estimate by rounds prefers and the clock does not. (The four products
+            // of a layer at 384 rows 295 -> 251 us; q/k/v at 512 rows 54 -> 45 us, at 768 rows 77 -> 65; o at 768 rows 55 -> 47.)
+            splits = (int)(2 * XRT_COMPUTE_UNITS / tiles);
             least = 4;
-            splits = 1;
-            if (tiles < 384) {
-                long best = LONG_MAX;
-                for (int parts = 1; parts <= 16 && parts <= units / least; ++parts) {
-                    const long rounds = (tiles * parts + 2 * XRT_COMPUTE_UNITS - 1) / (2 * XRT_COMPUTE_UNITS);
-                    const long cost = rounds * ((units + parts - 1) / parts) * (100 + 4 * (parts - 1));
-                    if (cost < best) { best = cost; splits = parts; }
-                }
-            }
         }
     }
     splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
