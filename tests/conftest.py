@@ -48,8 +48,13 @@ TINY_QWEN3 = {
     "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 32, "rms_norm_eps": 1e-6,
     "rope_theta": 1000000.0, "max_position_embeddings": 256, "tie_word_embeddings": True,
     "hidden_act": "silu", "eos_token_id": [2, 5], "bos_token_id": 3, "torch_dtype": "bfloat16",
+    # the rotation's two options (llama.rs:92-94, 103-106): half of a head rotated, positions divided by 4
+    "partial_rotary_factor": 0.5, "rope_scaling": {"rope_type": "linear", "factor": 4.0},
 }
 TINY = {"llama": TINY_LLAMA, "qwen3": TINY_QWEN3}
+# On top of a tiny configuration: the whole head is rotated again (the positions' scale stays). For tests that are after
+# what only such a model takes: the rotation in a projection's epilogue, the attention that finishes q, k and v itself.
+WHOLE_ROTATION = {"partial_rotary_factor": 1.0}
 
 
 def make_folder(raw_config, folder, seed, std=0.02, randomize_norms=True):

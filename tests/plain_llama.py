@@ -151,7 +151,11 @@ class PlainConfig:
         self.head_dim = int(raw.get("head_dim") or self.hidden // self.n_heads)  # llama.rs:125-128
         self.eps = float(raw.get("rms_norm_eps", 1e-5))                        # llama.rs:95-98
         self.rope_theta = float(raw.get("rope_theta", 10000.0))                # llama.rs:99-102
-        self.rope_dim = self.head_dim                                          # llama.rs:92-94
+        # llama.rs:92-94 (dims of a head that are rotated) and :103-106 (what multiplies a position, rope.rs:25); in a
+        # config.json a share of the head and a linear rule whose factor divides the positions
+        rule = raw.get("rope_scaling") or {}
+        self.rope_dim = int(self.head_dim * float(raw.get("partial_rotary_factor") or 1.0))
+        self.rope_scale = 1.0 / float(rule["factor"]) if rule.get("rope_type", rule.get("type")) == "linear" else 1.0
         self.tied = bool(raw.get("tie_word_embeddings", False))
         self.qk_norm = self.architecture == "Qwen3ForCausalLM"
         self.max_position = int(raw["max_position_embeddings"])
@@ -203,8 +207,8 @@ class PlainModel:
         if c.qk_norm:                                                              # :489-496
             q = head_rmsnorm(q, c.n_heads, c.head_dim, self.w(p + "self_attn.q_norm.weight"), c.eps)
             k = head_rmsnorm(k, c.n_kv_heads, c.head_dim, self.w(p + "self_attn.k_norm.weight"), c.eps)
-        q = rope(q, c.n_heads, c.head_dim, positions[first:], c.rope_dim, c.rope_theta)    # :498-500
-        k = rope(k, c.n_kv_heads, c.head_dim, positions, c.rope_dim, c.rope_theta)
+        q = rope(q, c.n_heads, c.head_dim, positions[first:], c.rope_dim, c.rope_theta, c.rope_scale)    # :498-500
+        k = rope(k, c.n_kv_heads, c.head_dim, positions, c.rope_dim, c.rope_theta, c.rope_scale)
         attn = causal_attention(q, k, v, c.n_heads, c.n_kv_heads, c.head_dim, start_position=first)   # :504-574
         x = x[first:] + linear(attn, self.w(p + "self_attn.o_proj.weight"))       # :576-577
         normed = rmsnorm(x, self.w(p + "post_attention_layernorm.weight"), c.eps)  # :579-580

@@ -38,10 +38,28 @@ def test_defaults_of_absent_keys_are_the_references():
 
 
 def test_rotary_base_inside_rope_parameters_is_read_not_ignored():
-    raw = {k: v for k, v in TINY["qwen3"].items() if k != "rope_theta"}
-    raw["rope_parameters"] = {"rope_theta": 1000000.0, "rope_type": "default"}
+    raw = {k: v for k, v in TINY["qwen3"].items() if k not in ("rope_theta", "rope_scaling", "partial_rotary_factor")}
+    raw["rope_parameters"] = {"rope_theta": 1000000.0, "rope_type": "linear", "factor": 4.0, "partial_rotary_factor": 0.5}
     assert parse_config(raw).rope_theta == 1000000.0
     assert parse_config(raw) == parse_config(TINY["qwen3"])
+    raw = {k: v for k, v in TINY["llama"].items() if k != "rope_theta"}
+    raw["rope_parameters"] = {"rope_theta": 10000.0, "rope_type": "default"}
+    assert parse_config(raw) == parse_config(TINY["llama"])
+
+
+def test_the_rotation_s_options():
+    """How many dims of a head are rotated and what multiplies a position (llama.rs:92-94, 103-106): a share of the
+    head and a linear rule whose factor divides the positions."""
+    plain = parse_config(TINY["llama"])
+    assert plain.rope_dim == plain.head_dim == 16 and plain.rope_scale == 1.0
+    assert "rope_scaling" not in plain.to_dict() and "partial_rotary_factor" not in plain.to_dict()
+    both = parse_config(TINY["qwen3"])
+    assert both.head_dim == 32 and both.rope_dim == 16 and both.rope_scale == 0.25
+    assert parse_config(both.to_dict()) == both
+    older = parse_config(dict(TINY["llama"], rope_scaling={"type": "linear", "factor": 2}))     # the older spelling of the key
+    assert older.rope_scale == 0.5 and older.rope_dim == 16
+    assert parse_config(dict(TINY["llama"], rope_scaling={"rope_type": "default"})) == plain
+    assert parse_config(dict(TINY["llama"], partial_rotary_factor=1.0, rope_scaling=None)) == plain
 
 
 def test_written_config_names_its_model_type(tmp_path):
@@ -63,7 +81,12 @@ def test_eos_may_be_a_number_or_a_list():
     ({"num_key_value_heads": 3}, "not divisible"),
     ({"num_key_value_heads": 0}, "non-zero"),
     ({"head_dim": 15}, "even"),
-    ({"rope_scaling": {"type": "linear", "factor": 2.0}}, "rope_scaling"),
+    ({"rope_scaling": {"rope_type": "yarn", "factor": 2.0}}, "rope_type"),
+    ({"rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0}}, "not supported"),
+    ({"rope_scaling": {"type": "linear"}}, "factor"),
+    ({"rope_scaling": {"type": "linear", "factor": 0}}, "factor"),
+    ({"rope_scaling": {"factor": 2.0}}, "without a rule"),
+    ({"rope_scaling": {"type": "linear", "factor": 2.0}, "rope_parameters": {"rope_type": "linear", "factor": 4.0}}, "disagree"),
     ({"hidden_act": "gelu"}, "hidden_act"),
     ({"attention_bias": True}, "attention_bias"),
     ({"mlp_bias": True}, "mlp_bias"),
@@ -72,9 +95,13 @@ def test_eos_may_be_a_number_or_a_list():
     ({"vocab_size": "many"}, "vocab_size"),
     ({"model_type": "qwen3"}, "model_type"),
     ({"rope_parameters": {"rope_theta": 10000.0, "rope_type": "yarn"}}, "rope_type"),
-    ({"rope_parameters": {"rope_theta": 10000.0, "factor": 4.0}}, "rope_parameters"),
+    ({"rope_parameters": {"rope_theta": 10000.0, "factor": 4.0}}, "without a rule"),
+    ({"rope_parameters": {"rope_theta": 10000.0, "beta_fast": 32}}, "not supported"),
     ({"rope_parameters": {"rope_theta": 500000.0}}, "disagree"),
-    ({"partial_rotary_factor": 0.5}, "partial_rotary_factor"),
+    ({"partial_rotary_factor": 0.2}, "rotated dims"),          # 3.2 of 16 dims: three
+    ({"partial_rotary_factor": 1.5}, "partial_rotary_factor"),
+    ({"partial_rotary_factor": 0.01}, "rotated dims"),
+    ({"partial_rotary_factor": 0.5, "rope_parameters": {"partial_rotary_factor": 0.25}}, "disagree"),
 ])
 def test_bad_configs_are_refused(change, text):
     with pytest.raises(ConfigError, match=text):

@@ -4,7 +4,7 @@ and in bfloat16, for two tiny configurations that differ in every size and optio
 import pytest
 import torch
 
-from conftest import TINY, make_folder
+from conftest import TINY, WHOLE_ROTATION, make_folder
 from helpers import (TOLERANCE, assert_logits, errors, first_bad_position, run_batched, run_tail_decoded, run_whole,
                      token_ids)
 import plain_llama as P
@@ -278,9 +278,15 @@ def test_a_step_may_mix_sequences_that_start_with_sequences_that_go_on(name, dty
 
 @pytest.mark.parametrize("arch,sizes", [
     ("llama", dict(num_attention_heads=4, num_key_value_heads=1, head_dim=64, max_position_embeddings=1200)),
-    # with head norms the attention of a bfloat16 decode step also norms and rotates q and the new key and writes the cache
+    # half of a head rotated, positions halved: the projection's epilogue does not rotate such heads, a kernel after it does
+    ("llama", dict(num_attention_heads=4, num_key_value_heads=2, head_dim=128, hidden_size=64, max_position_embeddings=1200,
+                   partial_rotary_factor=0.5, rope_scaling={"rope_type": "linear", "factor": 2.0})),
+    # with head norms and heads rotated whole, the attention of a bfloat16 decode step also norms and rotates q and the new key
+    # and writes the cache (angles from a table, here of positions divided by 4, and of plain positions)
+    ("qwen3", dict(num_attention_heads=6, num_key_value_heads=2, head_dim=128, max_position_embeddings=1200, **WHOLE_ROTATION)),
+    ("qwen3", dict(num_attention_heads=6, num_key_value_heads=3, head_dim=64, max_position_embeddings=1200, rope_scaling=None, **WHOLE_ROTATION)),
+    # head norms and half of a head rotated: the preparation kernel stays between projection and attention
     ("qwen3", dict(num_attention_heads=6, num_key_value_heads=2, head_dim=128, max_position_embeddings=1200)),
-    ("qwen3", dict(num_attention_heads=6, num_key_value_heads=3, head_dim=64, max_position_embeddings=1200)),
 ])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_decoding_across_a_thousand_tokens(dtype, arch, sizes, tmp_path):
@@ -322,7 +328,7 @@ def test_a_batch_of_forty_sequences(dtype, arch, head_dim, tmp_path):
     also does the norms' work and, without head norms (llama), the rotation and the cache write)."""
     from xeno_rt_amd.engine import Engine
     raw = dict(TINY[arch], hidden_size=128, intermediate_size=320, num_attention_heads=4, num_key_value_heads=2,
-               head_dim=head_dim, num_hidden_layers=2, max_position_embeddings=128)
+               head_dim=head_dim, num_hidden_layers=2, max_position_embeddings=128, **WHOLE_ROTATION)
     folder = make_folder(raw, tmp_path / "wide", seed=13, std=0.15)
     plain = P.PlainModel(folder)
     vocab = plain.config.vocab_size

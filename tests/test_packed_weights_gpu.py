@@ -4,7 +4,7 @@ what is refused, and whole tiny models whose every matrix is packed against the 
 import pytest
 import torch
 
-from conftest import TINY, make_folder
+from conftest import TINY, WHOLE_ROTATION, make_folder
 from helpers import assert_logits, first_bad_position, run_batched, run_tail_decoded, run_whole, token_ids
 import plain_llama as P
 
@@ -98,7 +98,7 @@ def test_what_does_not_fit_is_refused(ops):
 def models(tmp_path_factory):
     """Tiny models whose widths are multiples of 32, so that every matrix can be packed: name -> (folder, plain model)."""
     out = {}
-    for name, changes in (("llama", dict(intermediate_size=160, head_dim=32)), ("qwen3", {})):
+    for name, changes in (("llama", dict(intermediate_size=160, head_dim=32)), ("qwen3", dict(WHOLE_ROTATION))):
         raw = dict(TINY[name], **changes)
         folder = make_folder(raw, tmp_path_factory.mktemp(f"packed_{name}"), seed=61 if name == "llama" else 67, std=0.2)
         out[name] = (folder, P.PlainModel(folder))

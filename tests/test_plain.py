@@ -98,6 +98,33 @@ def test_rope_leaves_the_tail_beyond_rope_dim():
     assert float((y[:, :8] - x[:, :8]).abs().max()) > 1e-3
 
 
+def test_rope_scale_multiplies_the_position():
+    """rope.rs:25, 63, 109: angle = position * scale / theta. Position 8 at scale 0.25 is position 2 at scale 1; a scale
+    that divided the position, or multiplied theta, would make it position 32."""
+    x = torch.randn(3, 2 * 16)
+    at = lambda p: torch.tensor([p, p, p])
+    close(P.rope(x, 2, 16, at(8), 16, 1e4, 0.25), P.rope(x, 2, 16, at(2), 16, 1e4, 1.0), 1e-6)
+    assert float((P.rope(x, 2, 16, at(8), 16, 1e4, 0.25) - P.rope(x, 2, 16, at(32), 16, 1e4, 1.0)).abs().max()) > 1e-2
+    # with fewer dims rotated the pairs are (i, i + rope_dim / 2) of the first rope_dim dims, and theta's exponent is over rope_dim
+    y = P.rope(x, 2, 16, at(5), 8, 1e4, 0.5)
+    z = (x.view(3, 2, 16)[:, :, :4].double().numpy() + 1j * x.view(3, 2, 16)[:, :, 4:8].double().numpy()) \
+        * np.exp(1j * 5 * 0.5 / (1e4 ** (np.arange(4) * 2.0 / 8)))
+    close(y.view(3, 2, 16)[:, :, :4], z.real, 1e-5)
+    close(y.view(3, 2, 16)[:, :, 4:8], z.imag, 1e-5)
+
+
+def test_the_plain_model_reads_the_rotation_s_options(tmp_path):
+    """The second tiny configuration rotates half of a head and divides positions by 4; the plain model must see both
+    (a model that ignored them would agree with the engine only if the engine ignored them too)."""
+    from conftest import TINY, make_folder
+    model = P.PlainModel(make_folder(TINY["qwen3"], tmp_path / "m", seed=5))
+    assert model.config.rope_dim == 16 and model.config.head_dim == 32 and model.config.rope_scale == 0.25
+    ids = list(range(3, 23))
+    with_options = model.logits(ids)
+    model.config.rope_scale, model.config.rope_dim = 1.0, 32
+    assert float((model.logits(ids) - with_options).abs().max()) > 1e-3 * float(with_options.abs().max())
+
+
 # ---- softmax, silu, linear ---------------------------------------------------------
 
 def test_softmax_reference_vector():

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import ROOT, TINY, make_folder
+from conftest import ROOT, TINY, WHOLE_ROTATION, make_folder
 from helpers import assert_logits, token_ids
 import plain_llama as P
 
@@ -121,7 +121,7 @@ def test_replay_in_portions(head_dim, dtype, tmp_path):
     block's boundary; a portion of two tokens; one that ends at a block's end again; then token by token, while
     a second request of the same steps starts later and runs beside it."""
     raw = dict(TINY["qwen3" if head_dim == 128 else "llama"], hidden_size=128, num_attention_heads=2, num_key_value_heads=1,
-               head_dim=head_dim, max_position_embeddings=512)
+               head_dim=head_dim, max_position_embeddings=512, **WHOLE_ROTATION)
     # (weights of std 0.1: at this width std 0.2 makes scores so large that their rounding to bfloat16 alone moves
     # logits by 5 % of the largest, in the kernels as in the stand-in that only rounds where they round)
     folder = make_folder(raw, tmp_path / "model", seed=head_dim, std=0.1)

@@ -55,6 +55,12 @@ class LlamaConfig:
     eos_token_ids: Tuple[int, ...] = ()
     bos_token_id: Optional[int] = None
     torch_dtype: str = "bfloat16"
+    rope_dim: int = 0            # dims of a head that are rotated, the first ones (llama.rs:92-94); 0: the whole head
+    rope_scale: float = 1.0      # what a position is multiplied by before it becomes an angle (llama.rs:103-106, rope.rs:25)
+
+    def __post_init__(self):
+        if self.rope_dim == 0:
+            object.__setattr__(self, "rope_dim", self.head_dim)
 
     # Architectures that this class parses, and whether each norms q and k per head.
     QK_NORM_BY_ARCHITECTURE = {"LlamaForCausalLM": False, "Qwen3ForCausalLM": True}
@@ -68,10 +74,6 @@ class LlamaConfig:
     @property
     def kv_width(self) -> int:           # llama.rs:134-136
         return self.num_key_value_heads * self.head_dim
-
-    @property
-    def rope_dim(self) -> int:           # llama.rs:92-94: the whole head is rotated
-        return self.head_dim
 
     @classmethod
     def from_dict(cls, raw: dict) -> "LlamaConfig":
@@ -108,27 +110,62 @@ class LlamaConfig:
         model_type = raw.get("model_type")
         if model_type is not None and model_type != cls.MODEL_TYPE_BY_ARCHITECTURE[architecture]:
             raise ConfigError(f"config.json: model_type {model_type!r} does not belong to {architecture}")
-        if raw.get("rope_scaling") not in (None, {}):
-            raise ConfigError("config.json: 'rope_scaling' is not supported (must be null or absent)")
-        # newer checkpoint folders carry the rotary base inside `rope_parameters`; anything there that would
-        # change the angles (a scaling rule, a factor) is refused, never ignored
+        # The rotation's options. The reference has two beside the base: how many dims of a head are rotated
+        # (llama.rs:92-94) and a number that multiplies every position (llama.rs:103-106, rope.rs:25: GGUF's
+        # `rope.scale_linear`). In config.json these are `partial_rotary_factor` (a share of the head) and a linear
+        # `rope_scaling` whose `factor` divides the positions, so the multiplier is 1 / factor. Newer folders carry all
+        # of it, with the base, inside `rope_parameters`. Every other scaling rule is refused, never ignored.
+        rope_scale, rotary_share = 1.0, raw.get("partial_rotary_factor")
+
+        def linear_factor(rule: dict, where: str) -> float:
+            kind = rule.get("rope_type", rule.get("type"))
+            unknown = sorted(set(rule) - {"rope_type", "type", "factor", "rope_theta", "partial_rotary_factor"})
+            if unknown:
+                raise ConfigError(f"config.json: '{where}' has keys that are not supported: {unknown}")
+            if kind in (None, "default"):
+                if rule.get("factor") not in (None, 1, 1.0):
+                    raise ConfigError(f"config.json: '{where}' has a factor without a rule (rope_type 'linear')")
+                return 1.0
+            if kind != "linear":
+                raise ConfigError(f"config.json: rope_type {kind!r} is not supported (only 'default' and 'linear')")
+            factor = rule.get("factor")
+            if isinstance(factor, bool) or not isinstance(factor, (int, float)) or not factor > 0:
+                raise ConfigError(f"config.json: '{where}' of type 'linear' needs a positive 'factor', found {factor!r}")
+            return 1.0 / float(factor)
+
+        rope_scaling = raw.get("rope_scaling")
+        if rope_scaling not in (None, {}):
+            if not isinstance(rope_scaling, dict):
+                raise ConfigError("config.json: 'rope_scaling' must be an object or null")
+            if "rope_theta" in rope_scaling or "partial_rotary_factor" in rope_scaling:
+                raise ConfigError("config.json: 'rope_scaling' holds the rule and its factor only")
+            rope_scale = linear_factor(rope_scaling, "rope_scaling")
         rope_parameters = raw.get("rope_parameters")
         if rope_parameters is not None:
             if not isinstance(rope_parameters, dict):
                 raise ConfigError("config.json: 'rope_parameters' must be an object")
-            unknown = sorted(set(rope_parameters) - {"rope_theta", "rope_type"})
-            if unknown:
-                raise ConfigError(f"config.json: 'rope_parameters' has keys that are not supported: {unknown}")
-            if rope_parameters.get("rope_type") not in (None, "default"):
-                raise ConfigError(f"config.json: rope_type {rope_parameters.get('rope_type')!r} is not supported "
-                                  "(only 'default')")
+            inner_scale = linear_factor(rope_parameters, "rope_parameters")
+            if rope_scaling not in (None, {}) and inner_scale != rope_scale:
+                raise ConfigError("config.json: 'rope_scaling' and 'rope_parameters' disagree")
+            rope_scale = inner_scale
             inner = rope_parameters.get("rope_theta")
             if inner is not None:
                 if raw.get("rope_theta") is not None and float(raw["rope_theta"]) != float(inner):
                     raise ConfigError("config.json: 'rope_theta' and 'rope_parameters.rope_theta' disagree")
                 raw = dict(raw, rope_theta=inner)
-        if raw.get("partial_rotary_factor") not in (None, 1, 1.0):
-            raise ConfigError("config.json: 'partial_rotary_factor' must be 1 or absent (the whole head is rotated)")
+            inner_share = rope_parameters.get("partial_rotary_factor")
+            if inner_share is not None:
+                if rotary_share is not None and float(rotary_share) != float(inner_share):
+                    raise ConfigError("config.json: 'partial_rotary_factor' and 'rope_parameters.partial_rotary_factor' disagree")
+                rotary_share = inner_share
+        rope_dim = head_dim
+        if rotary_share is not None:
+            if isinstance(rotary_share, bool) or not isinstance(rotary_share, (int, float)) or not 0 < rotary_share <= 1:
+                raise ConfigError(f"config.json: 'partial_rotary_factor' must lie in (0, 1], found {rotary_share!r}")
+            rope_dim = int(head_dim * float(rotary_share))
+            if rope_dim < 2 or rope_dim % 2 != 0:
+                raise ConfigError(f"config.json: partial_rotary_factor {rotary_share} of head_dim {head_dim} gives {rope_dim} "
+                                  "rotated dims; an even number, two at least, is needed (rotary pairs)")
         activation = raw.get("hidden_act", "silu")
         if activation != "silu":
             raise ConfigError(f"config.json: hidden_act must be 'silu', found {activation!r}")
@@ -175,6 +212,8 @@ class LlamaConfig:
             eos_token_ids=eos_ids,
             bos_token_id=None if bos is None else int(bos),
             torch_dtype=str(raw.get("torch_dtype", "bfloat16")),
+            rope_dim=rope_dim,
+            rope_scale=rope_scale,
         )
 
     def to_dict(self) -> dict:
@@ -198,6 +237,8 @@ class LlamaConfig:
             "eos_token_id": None if not eos else (eos[0] if len(eos) == 1 else eos),
             "bos_token_id": self.bos_token_id,
             "torch_dtype": self.torch_dtype,
+            **({} if self.rope_dim == self.head_dim else {"partial_rotary_factor": self.rope_dim / self.head_dim}),
+            **({} if self.rope_scale == 1.0 else {"rope_scaling": {"rope_type": "linear", "factor": 1.0 / self.rope_scale}}),
         }
 
 

@@ -23,8 +23,8 @@ def build_llama(config: LlamaConfig) -> ModelSpec:
     # one rotation for all layers. With head norms a decode step's attention finishes q and k itself and reads the
     # positions' cosines and sines from a table (positions * head_dim * 4 bytes, made once when the model is bound;
     # at most MOST_TABLE_POSITIONS: a step with a longer sequence takes the two kernels)
-    rotary = Rotary(c.rope_dim, c.rope_theta,
-                    table_positions=min(c.max_position_embeddings, MOST_TABLE_POSITIONS) if c.qk_norm else 0)
+    rotary = Rotary(c.rope_dim, c.rope_theta, scale=c.rope_scale,
+                    table_positions=min(c.max_position_embeddings, MOST_TABLE_POSITIONS) if c.qk_norm and c.rope_dim == c.head_dim else 0)
     for index in range(c.num_hidden_layers):
         p = f"model.layers.{index}."
         mixer = Attention(
