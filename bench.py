@@ -231,6 +231,8 @@ def main() -> int:
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
     parser.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
                         help="for profiling: run only the decode steps, or only the prefill (prints a partial record)")
+    parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                        help="with --phase prefill: the prompt's length (the record's prefill is always of 2048 tokens)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this library runs on a single MI355X)")
@@ -250,7 +252,7 @@ def main() -> int:
         args.skip_points = True
     others = () if args.skip_points else tuple(b for b in OTHER_BATCHES[args.shape] if b != batch)
     largest_batch = max((batch,) + others)
-    context = args.context
+    context = args.context if args.phase != "prefill" else max(args.context, args.prefill_tokens)
     engine = Engine.random(config, seed=args.seed, dtype=args.dtype, max_tokens=largest_batch * context,
                            max_slots=largest_batch, max_context=context if args.skip_points else max(context, LONG_PREFILL))
     bench = Bench(engine, args.seed)
@@ -260,9 +262,9 @@ def main() -> int:
         return step_bytes / (ms * 1e-3) / 1e9
 
     if args.phase == "prefill":
-        seconds = bench.prefill([PREFILL_TOKENS])
-        print(json.dumps({"phase": "prefill", "tokens": PREFILL_TOKENS, "ms": round(seconds * 1e3, 3),
-                          "frac": round(prefill_flops(config, [PREFILL_TOKENS]) / seconds / PEAK_FLOPS[short], 4)}), flush=True)
+        seconds = bench.prefill([args.prefill_tokens])
+        print(json.dumps({"phase": "prefill", "tokens": args.prefill_tokens, "ms": round(seconds * 1e3, 3),
+                          "frac": round(prefill_flops(config, [args.prefill_tokens]) / seconds / PEAK_FLOPS[short], 4)}), flush=True)
         return 0
     tokens_per_s, ms_per_step, mean_length = bench.decode(batch, args.steps, args.warmup, context, check=args.phase == "all")
     if args.phase == "decode":
