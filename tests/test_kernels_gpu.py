@@ -49,14 +49,15 @@ def rel(got, want):
 
 # ---- embedding, add, rmsnorm -----------------------------------------------------------
 
+@pytest.mark.parametrize("hidden", [200, 201, 4096])          # rows of 16-byte pieces, rows that are not, rows longer than a workgroup's step
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_embed_and_add(ops, dtype):
-    table = rand(777, 200, dtype=DT[dtype])
+def test_embed_and_add(ops, dtype, hidden):
+    table = rand(777, hidden, dtype=DT[dtype])
     ids = torch.tensor([0, 776, 5, 5, 123], dtype=torch.int32, device=DEV)
-    out = torch.empty(5, 200, device=DEV)
+    out = torch.empty(5, hidden, device=DEV)
     ops.embed(table, ids, out)
     assert torch.equal(out, table[ids.long()].float())
-    delta = rand(5, 200, dtype=DT[dtype], seed=2)
+    delta = rand(5, hidden, dtype=DT[dtype], seed=2)
     want = out + delta.float()
     ops.add(out, delta)
     assert torch.equal(out, want)

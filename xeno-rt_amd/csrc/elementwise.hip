@@ -8,12 +8,27 @@
 #include "xrt_hip.h"
 #include "packing.h"
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
                              float* __restrict__ out, int hidden) {
     const long token = blockIdx.x;
     const T* row = table + (long)ids[token] * hidden;
     float* dst = out + token * hidden;
+    if constexpr (sizeof(T) == 2) {
+        if (hidden % 8 == 0) {              // 16 bytes of the row a lane and step (a row then starts at a multiple of 16 bytes)
+            for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
+                const bf16x8 eight = *reinterpret_cast<const bf16x8*>(row + i);
+                float4 low, high;
+                low.x = (float)eight[0]; low.y = (float)eight[1]; low.z = (float)eight[2]; low.w = (float)eight[3];
+                high.x = (float)eight[4]; high.y = (float)eight[5]; high.z = (float)eight[6]; high.w = (float)eight[7];
+                *reinterpret_cast<float4*>(dst + i) = low;
+                *reinterpret_cast<float4*>(dst + i + 4) = high;
+            }
+            return;
+        }
+    }
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]);
 }
 
